@@ -1,0 +1,286 @@
+"""The cache manager: pages of keys and values with a block table per request, and slots of
+fixed-size state per request.
+
+A model names its cache needs as one spec per cache entry (an entry is what one run of a layer
+reads and writes): `KvSpec` for a mixer that keeps keys and values, `StateSpec` for a mixer
+with state of fixed size, None for a layer without memory.  Entries with equal `KvSpec` form
+a group; a group has its own pool of pages (one page id is valid in every entry of the
+group), its own block tables and its own rule for giving pages back (all keys kept, or only a
+window).  The bookkeeping itself (free lists, tables, lengths, invariants) is native code in
+csrc/host/cache_manager.cpp; this module owns the device memory and keeps the device copies
+of the block tables current.
+
+Device layout of a group: k and v slabs [entries, num_pages, kv_heads, page_size, head_dim];
+block table int32 [max_slots, max_blocks], -1 where no page is mapped.  Unused memory is
+filled with NaN so that a read of a never-written key shows (the reference fills its cache
+with 0xFF for the same reason, src/minillm/cuda/storage.cpp:199-200).
+"""
+from __future__ import annotations
+
+import ctypes
+from dataclasses import dataclass
+from typing import Optional, Tuple
+
+import numpy as np
+import torch
+
+from ..kernels import build
+
+
+class CacheError(RuntimeError):
+    pass
+
+
+class CacheFull(CacheError):
+    """Not enough free pages (or slots) for what was asked; nothing was changed."""
+
+
+@dataclass(frozen=True)
+class KvSpec:
+    kv_heads: int
+    head_dim: int
+    window: Optional[int] = None      # None: all keys are kept
+
+
+@dataclass(frozen=True)
+class StateSpec:
+    shape: Tuple[int, ...]
+    dtype: torch.dtype = torch.float32
+
+
+@dataclass
+class KvView:
+    k_pages: torch.Tensor             # [num_pages, kv_heads, page_size, head_dim]
+    v_pages: torch.Tensor
+    block_table: torch.Tensor         # device int32 [max_slots, max_blocks]
+    page_size: int
+    window: Optional[int]
+    group: int
+
+
+def _host_lib():
+    lib = build.load("host")
+    if not getattr(lib, "_mlr_typed", False):
+        lib.mlr_cache_create.restype = ctypes.c_void_p
+        lib.mlr_cache_create.argtypes = [ctypes.c_int, ctypes.c_int]
+        lib.mlr_cache_destroy.argtypes = [ctypes.c_void_p]
+        lib.mlr_cache_destroy.restype = None
+        lib.mlr_cache_add_group.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int]
+        lib.mlr_cache_max_blocks.argtypes = [ctypes.c_void_p, ctypes.c_int]
+        lib.mlr_cache_free_pages.argtypes = [ctypes.c_void_p, ctypes.c_int]
+        lib.mlr_cache_free_slots.argtypes = [ctypes.c_void_p]
+        lib.mlr_cache_table.argtypes = [ctypes.c_void_p, ctypes.c_int]
+        lib.mlr_cache_table.restype = ctypes.POINTER(ctypes.c_int32)
+        lib.mlr_cache_length.argtypes = [ctypes.c_void_p, ctypes.c_int]
+        lib.mlr_cache_acquire_slot.argtypes = [ctypes.c_void_p]
+        lib.mlr_cache_release_slot.argtypes = [ctypes.c_void_p, ctypes.c_int]
+        i32p = ctypes.POINTER(ctypes.c_int32)
+        intp = ctypes.POINTER(ctypes.c_int)
+        lib.mlr_cache_prepare.argtypes = [ctypes.c_void_p, i32p, i32p, ctypes.c_int, intp, intp]
+        lib.mlr_cache_commit.argtypes = [ctypes.c_void_p, i32p, i32p, ctypes.c_int]
+        lib.mlr_cache_retire.argtypes = [ctypes.c_void_p, i32p, ctypes.c_int]
+        lib.mlr_cache_take_dirty.argtypes = [ctypes.c_void_p, ctypes.c_int, i32p]
+        lib.mlr_cache_check.argtypes = [ctypes.c_void_p]
+        lib._mlr_typed = True
+    return lib
+
+
+def _i32(values):
+    arr = np.ascontiguousarray(values, dtype=np.int32)
+    return arr, arr.ctypes.data_as(ctypes.POINTER(ctypes.c_int32))
+
+
+class PageBook:
+    """The native bookkeeping alone (no device memory): usable and testable without a GPU."""
+
+    def __init__(self, max_slots, max_length):
+        self._lib = _host_lib()
+        self._h = self._lib.mlr_cache_create(max_slots, max_length)
+        if not self._h:
+            raise CacheError("max_slots and max_length must be positive")
+        self.max_slots, self.max_length = max_slots, max_length
+        self.groups = []                  # (page_size, num_pages, window)
+
+    def __del__(self):
+        h, self._h = getattr(self, "_h", None), None
+        if h:
+            self._lib.mlr_cache_destroy(h)
+
+    def add_group(self, page_size, num_pages, window=None):
+        g = self._lib.mlr_cache_add_group(self._h, page_size, num_pages, window or 0)
+        if g < 0:
+            raise CacheError("page_size and num_pages must be positive")
+        self.groups.append((page_size, num_pages, window))
+        return g
+
+    def max_blocks(self, group):
+        return self._lib.mlr_cache_max_blocks(self._h, group)
+
+    def free_pages(self, group=0):
+        return self._lib.mlr_cache_free_pages(self._h, group)
+
+    def free_slots(self):
+        return self._lib.mlr_cache_free_slots(self._h)
+
+    def table(self, group=0):
+        """Host view [max_slots, max_blocks] of the group's block table (not a copy)."""
+        ptr = self._lib.mlr_cache_table(self._h, group)
+        return np.ctypeslib.as_array(ptr, shape=(self.max_slots, self.max_blocks(group)))
+
+    def length(self, slot):
+        n = self._lib.mlr_cache_length(self._h, slot)
+        if n < 0:
+            raise CacheError(f"slot {slot} is not live")
+        return n
+
+    def acquire_slot(self):
+        s = self._lib.mlr_cache_acquire_slot(self._h)
+        if s < 0:
+            raise CacheFull("no free request slot")
+        return s
+
+    def release_slot(self, slot):
+        if self._lib.mlr_cache_release_slot(self._h, slot) != 0:
+            raise CacheError(f"slot {slot} is not live (released twice?)")
+
+    def _raise(self, rc, group, need_free):
+        if rc == -1:
+            raise CacheError("batch names a slot that is not live")
+        if rc == -2:
+            raise CacheError(f"a request would grow beyond max_length {self.max_length}")
+        if rc == -3:
+            raise CacheFull(f"cache group {group} needs {need_free[0]} more pages but only "
+                            f"{need_free[1]} are free")
+        if rc == -4:
+            raise CacheError("a batch entry must bring at least one token")
+        if rc == -5:
+            raise CacheError("a slot appears twice in one batch")
+        raise CacheError(f"cache bookkeeping failed ({rc})")
+
+    def prepare(self, slots, counts):
+        """Raises if the batch {slot: number of new tokens} cannot be taken; changes nothing."""
+        s, sp = _i32(slots)
+        c, cp = _i32(counts)
+        group = ctypes.c_int(-1)
+        need_free = (ctypes.c_int * 2)(0, 0)
+        rc = self._lib.mlr_cache_prepare(self._h, sp, cp, len(s), ctypes.byref(group), need_free)
+        if rc != 0:
+            self._raise(rc, group.value, need_free)
+
+    def commit(self, slots, counts):
+        self.prepare(slots, counts)
+        s, sp = _i32(slots)
+        c, cp = _i32(counts)
+        rc = self._lib.mlr_cache_commit(self._h, sp, cp, len(s))
+        if rc != 0:
+            self._raise(rc, -1, (0, 0))
+
+    def retire(self, slots):
+        s, sp = _i32(slots)
+        rc = self._lib.mlr_cache_retire(self._h, sp, len(s))
+        if rc < 0:
+            raise CacheError("retire names a slot that is not live")
+        return rc
+
+    def take_dirty(self, group=0):
+        out = np.empty(self.max_slots, dtype=np.int32)
+        n = self._lib.mlr_cache_take_dirty(self._h, group, out.ctypes.data_as(ctypes.POINTER(ctypes.c_int32)))
+        return out[:n].tolist()
+
+    def check(self):
+        rc = self._lib.mlr_cache_check(self._h)
+        if rc != 0:
+            raise CacheError(f"page bookkeeping invariant {rc} is broken")
+
+
+class CacheManager:
+    """Device memory for every cache entry of a model plus the bookkeeping above."""
+
+    def __init__(self, entry_specs, dtype, device, page_size, max_tokens, max_slots, max_length):
+        if page_size <= 0 or max_tokens <= 0:
+            raise CacheError("page_size and max_tokens must be positive")
+        self.dtype, self.device, self.page_size = dtype, torch.device(device), page_size
+        self.max_slots, self.max_length = max_slots, max_length
+        self.num_pages = (max_tokens + page_size - 1) // page_size
+        self.book = PageBook(max_slots, max_length)
+        self.entry_specs = list(entry_specs)
+        self._group_of_spec = {}
+        self._entry_place = {}            # cache id -> (group, index within the group)
+        members = []
+        for cid, spec in enumerate(self.entry_specs):
+            if isinstance(spec, KvSpec):
+                if spec not in self._group_of_spec:
+                    self._group_of_spec[spec] = self.book.add_group(page_size, self.num_pages, spec.window)
+                    members.append([])
+                g = self._group_of_spec[spec]
+                self._entry_place[cid] = (g, len(members[g]))
+                members[g].append(cid)
+        self.group_specs = [None] * len(members)
+        for spec, g in self._group_of_spec.items():
+            self.group_specs[g] = spec
+        self._k, self._v, self._tables = [], [], []
+        for g, spec in enumerate(self.group_specs):
+            shape = (len(members[g]), self.num_pages, spec.kv_heads, page_size, spec.head_dim)
+            self._k.append(torch.full(shape, float("nan"), dtype=dtype, device=self.device))
+            self._v.append(torch.full(shape, float("nan"), dtype=dtype, device=self.device))
+            self._tables.append(torch.full((max_slots, self.book.max_blocks(g)), -1, dtype=torch.int32,
+                                           device=self.device))
+        self._states = {}
+        for cid, spec in enumerate(self.entry_specs):
+            if isinstance(spec, StateSpec):
+                self._states[cid] = torch.zeros((max_slots, *spec.shape), dtype=spec.dtype, device=self.device)
+
+    # -- views for the parts ---------------------------------------------------------------------
+    def kv_view(self, cache_id):
+        g, i = self._entry_place[cache_id]
+        spec = self.group_specs[g]
+        return KvView(self._k[g][i], self._v[g][i], self._tables[g], self.page_size, spec.window, g)
+
+    def state_view(self, cache_id):
+        return self._states[cache_id]
+
+    def kv_bytes(self):
+        return sum(t.numel() * t.element_size() for t in self._k + self._v)
+
+    # -- requests --------------------------------------------------------------------------------
+    def acquire_slot(self):
+        slot = self.book.acquire_slot()
+        for state in self._states.values():
+            state[slot].zero_()
+        return slot
+
+    def release_slot(self, slot):
+        self.book.release_slot(slot)
+
+    def length(self, slot):
+        return self.book.length(slot)
+
+    def free_pages(self, group=0):
+        return self.book.free_pages(group)
+
+    def prepare(self, slots, counts):
+        self.book.prepare(slots, counts)
+
+    def commit(self, slots, counts):
+        self.book.commit(slots, counts)
+        self.sync_tables()
+
+    def retire(self, slots):
+        """After a step: give back what windows have passed.  The device tables are brought up
+        to date before the next step (commit)."""
+        return self.book.retire(slots)
+
+    def sync_tables(self):
+        for g, dev in enumerate(self._tables):
+            rows = self.book.take_dirty(g)
+            if not rows:
+                continue
+            host = torch.from_numpy(self.book.table(g))
+            if len(rows) * 4 >= self.max_slots:
+                dev.copy_(host)
+            else:
+                for s in rows:
+                    dev[s].copy_(host[s])
+
+    def check(self):
+        self.book.check()

@@ -1,0 +1,192 @@
+// out[M, N] = a[M, K] . w[N, K]^T  (both operands row-major with K contiguous, the layout of
+// an activation and of a projection's weight), accumulated in 32-bit.
+//
+// Float engine: a plain tiled FMA kernel; every output element is one sequential sum over k,
+// so a row's result does not depend on the other rows of the batch.
+// Bfloat16 engine: MFMA (v_mfma_f32_16x16x32_bf16) tiles staged through LDS; the k order of
+// every output element is fixed as well (no split over k).
+#include "common.h"
+
+#if !MLR_BF16
+// ------------------------------------------------------------------------------ float
+#define BM 64
+#define BN 64
+#define BK 16
+
+__global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__ a,
+                                                       const float* __restrict__ w,
+                                                       float* __restrict__ out, int M, int N, int K) {
+    __shared__ float as[BK][BM + 4];
+    __shared__ float ws[BK][BN + 4];
+    const int t = threadIdx.x;
+    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    const int tx = t % 16, ty = t / 16;
+    const int lrow = t / 4, lk = (t % 4) * 4;       // this thread stages row lrow, k lk..lk+3
+    float acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+
+    for (int k0 = 0; k0 < K; k0 += BK) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int k = k0 + lk + e;
+            const int am = m0 + lrow, wn = n0 + lrow;
+            as[lk + e][lrow] = (am < M && k < K) ? a[(size_t)am * K + k] : 0.f;
+            ws[lk + e][lrow] = (wn < N && k < K) ? w[(size_t)wn * K + k] : 0.f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < BK; ++k) {
+            float av[4], wv[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) av[i] = as[k][ty * 4 + i];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) wv[j] = ws[k][tx * 4 + j];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(av[i], wv[j], acc[i][j]);
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int m = m0 + ty * 4 + i;
+        if (m >= M) continue;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int n = n0 + tx * 4 + j;
+            if (n < N) out[(size_t)m * N + n] = acc[i][j];
+        }
+    }
+}
+
+extern "C" int mlr_gemm(const void* a, const void* w, void* out, int M, int N, int K, int out_float,
+                        hipStream_t stream) {
+    (void)out_float;                                   // the float engine's outputs are float
+    if (M <= 0 || N <= 0) return 0;
+    if (K <= 0) return -1;
+    dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM);
+    if (grid.y > 65535) return -2;
+    gemm_f32_kernel<<<grid, 256, 0, stream>>>((const float*)a, (const float*)w, (float*)out, M, N, K);
+    return (int)hipGetLastError();
+}
+
+#else
+// ------------------------------------------------------------------------------ bfloat16
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+
+#define BK 32
+#define LDS_STRIDE (BK + 8)      // in elements: rows 80 bytes apart
+
+// Eight consecutive k of one row as a 16-byte vector; zero beyond the matrix.
+__device__ __forceinline__ bf16x8 load_k8(const __bf16* base, int row, int rows, int k, int K,
+                                          bool vector_ok) {
+    bf16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (row < rows) {
+        const __bf16* p = base + (size_t)row * K + k;
+        if (vector_ok && k + 8 <= K) {
+            v = *reinterpret_cast<const bf16x8*>(p);
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                if (k + e < K) v[e] = p[e];
+        }
+    }
+    return v;
+}
+
+// Workgroup tile (WM * TM * 16) x (WN * TN * 16); WM x WN wavefronts, each TM x TN MFMA tiles.
+template <int WM, int WN, int TM, int TN, bool OUT_FLOAT>
+__global__ __launch_bounds__(WM * WN * 64) void gemm_bf16_kernel(
+    const __bf16* __restrict__ a, const __bf16* __restrict__ w, void* __restrict__ out_raw,
+    int M, int N, int K) {
+    constexpr int BM = WM * TM * 16, BN = WN * TN * 16, THREADS = WM * WN * 64;
+    __shared__ __bf16 as[BM * LDS_STRIDE];
+    __shared__ __bf16 ws[BN * LDS_STRIDE];
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int wm = wave / WN, wn = wave % WN;
+    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    const bool vector_ok = (K % 8) == 0;
+
+    floatx4 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    for (int k0 = 0; k0 < K; k0 += BK) {
+        for (int c = t; c < BM * 4; c += THREADS) {           // 4 chunks of 8 per row
+            const int r = c >> 2, kc = (c & 3) * 8;
+            *reinterpret_cast<bf16x8*>(&as[r * LDS_STRIDE + kc]) =
+                load_k8(a, m0 + r, M, k0 + kc, K, vector_ok);
+        }
+        for (int c = t; c < BN * 4; c += THREADS) {
+            const int r = c >> 2, kc = (c & 3) * 8;
+            *reinterpret_cast<bf16x8*>(&ws[r * LDS_STRIDE + kc]) =
+                load_k8(w, n0 + r, N, k0 + kc, K, vector_ok);
+        }
+        __syncthreads();
+        bf16x8 af[TM], wf[TN];
+        const int frag_row = lane & 15, frag_k = (lane >> 4) * 8;
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+            af[i] = *reinterpret_cast<const bf16x8*>(
+                &as[((wm * TM + i) * 16 + frag_row) * LDS_STRIDE + frag_k]);
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+            wf[j] = *reinterpret_cast<const bf16x8*>(
+                &ws[((wn * TN + j) * 16 + frag_row) * LDS_STRIDE + frag_k]);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[i], wf[j], acc[i][j], 0, 0, 0);
+        __syncthreads();
+    }
+
+    // accumulator element r of a lane: row (lane / 16) * 4 + r, column lane % 16
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const int n = n0 + (wn * TN + j) * 16 + (lane & 15);
+            if (n >= N) continue;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int m = m0 + (wm * TM + i) * 16 + (lane >> 4) * 4 + r;
+                if (m >= M) continue;
+                if (OUT_FLOAT) ((float*)out_raw)[(size_t)m * N + n] = acc[i][j][r];
+                else ((__bf16*)out_raw)[(size_t)m * N + n] = (__bf16)acc[i][j][r];
+            }
+        }
+    }
+}
+
+template <int WM, int WN, int TM, int TN>
+static int launch(const void* a, const void* w, void* out, int M, int N, int K, int out_float,
+                  hipStream_t stream) {
+    constexpr int BM = WM * TM * 16, BN = WN * TN * 16;
+    dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM);
+    if (grid.y > 65535) return -2;
+    if (out_float)
+        gemm_bf16_kernel<WM, WN, TM, TN, true><<<grid, WM * WN * 64, 0, stream>>>(
+            (const __bf16*)a, (const __bf16*)w, out, M, N, K);
+    else
+        gemm_bf16_kernel<WM, WN, TM, TN, false><<<grid, WM * WN * 64, 0, stream>>>(
+            (const __bf16*)a, (const __bf16*)w, out, M, N, K);
+    return (int)hipGetLastError();
+}
+
+extern "C" int mlr_gemm(const void* a, const void* w, void* out, int M, int N, int K, int out_float,
+                        hipStream_t stream) {
+    if (M <= 0 || N <= 0) return 0;
+    if (K <= 0) return -1;
+    if (M <= 16) return launch<1, 4, 1, 1>(a, w, out, M, N, K, out_float, stream);   // 16 x 64
+    if (M <= 64) return launch<2, 2, 2, 2>(a, w, out, M, N, K, out_float, stream);   // 64 x 64
+    return launch<2, 2, 4, 4>(a, w, out, M, N, K, out_float, stream);                // 128 x 128
+}
+#endif

@@ -1,0 +1,109 @@
+// Per-head RMSNorm of q and k, split-half rotation by position, and the write of k and v
+// into their pages of the cache: one kernel, one pass over the projection's output.
+//
+// Cache layout of one layer: pages[num_pages][kv_heads][page_size][head_dim]; token
+// position p of the request in slot s lies in page block_table[s][p / page_size] at row
+// p % page_size.  Norm sums and the rotation are computed in 32-bit; cos/sin come from a
+// float table [max_positions][head_dim] (first half cos, second half sin).
+#include "common.h"
+
+#define MAX_PAIRS 4   // head_dim / 2 <= 64 * MAX_PAIRS
+
+__global__ void qk_norm_rope_kv_kernel(
+    const elem_t* __restrict__ qkv, int ld, elem_t* __restrict__ q_out,
+    elem_t* __restrict__ k_pages, elem_t* __restrict__ v_pages,
+    const int32_t* __restrict__ block_table, int max_blocks,
+    const int32_t* __restrict__ slots, const int32_t* __restrict__ positions,
+    const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w, float eps,
+    const float* __restrict__ rope, int q_heads, int kv_heads, int head_dim, int page_size,
+    int write_cache) {
+    const int m = blockIdx.x;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
+    const int half = head_dim >> 1;
+    const int pos = positions[m];
+    const int slot = slots[m];
+    const elem_t* row = qkv + (size_t)m * ld;
+    const float* cs = rope ? rope + (size_t)pos * head_dim : nullptr;
+
+    size_t cache_row = 0;
+    bool cache_ok = false;
+    if (write_cache) {
+        const int page = block_table[(size_t)slot * max_blocks + pos / page_size];
+        cache_ok = page >= 0;
+        cache_row = (size_t)(page < 0 ? 0 : page) * kv_heads * page_size + (pos % page_size);
+    }
+
+    const int total = q_heads + 2 * kv_heads;
+    for (int head = wave; head < total; head += waves) {
+        const elem_t* src = row + (size_t)head * head_dim;
+        if (head >= q_heads + kv_heads) {            // a value head: copy into its page
+            if (cache_ok) {
+                const int kvh = head - q_heads - kv_heads;
+                elem_t* dst = v_pages + (cache_row + (size_t)kvh * page_size) * head_dim;
+                for (int d = lane; d < head_dim; d += 64) dst[d] = src[d];
+            }
+            continue;
+        }
+        const bool is_q = head < q_heads;
+        const float* w = is_q ? q_norm_w : k_norm_w;
+        float a[MAX_PAIRS], b[MAX_PAIRS];
+        float sum = 0.f;
+#pragma unroll
+        for (int i = 0; i < MAX_PAIRS; ++i) {
+            const int j = lane + 64 * i;
+            a[i] = b[i] = 0.f;
+            if (j < half) {
+                a[i] = to_float(src[j]);
+                b[i] = to_float(src[j + half]);
+                sum += a[i] * a[i] + b[i] * b[i];
+            }
+        }
+        if (w) {
+            sum = wave_sum(sum);
+            const float scale = 1.0f / sqrtf(sum / (float)head_dim + eps);
+#pragma unroll
+            for (int i = 0; i < MAX_PAIRS; ++i) {
+                const int j = lane + 64 * i;
+                if (j < half) {
+                    a[i] = (a[i] * scale) * w[j];
+                    b[i] = (b[i] * scale) * w[j + half];
+                }
+            }
+        }
+        elem_t* dst;
+        if (is_q) {
+            dst = q_out + ((size_t)m * q_heads + head) * head_dim;
+        } else {
+            if (!cache_ok) continue;
+            dst = k_pages + (cache_row + (size_t)(head - q_heads) * page_size) * head_dim;
+        }
+#pragma unroll
+        for (int i = 0; i < MAX_PAIRS; ++i) {
+            const int j = lane + 64 * i;
+            if (j < half) {
+                float x = a[i], y = b[i];
+                if (cs) {
+                    const float c = cs[j], s = cs[j + half];
+                    x = a[i] * c - b[i] * s;
+                    y = a[i] * s + b[i] * c;
+                }
+                dst[j] = from_float<elem_t>(x);
+                dst[j + half] = from_float<elem_t>(y);
+            }
+        }
+    }
+}
+
+extern "C" int mlr_qk_norm_rope_kv(
+    const void* qkv, int ld, void* q_out, void* k_pages, void* v_pages, const int32_t* block_table,
+    int max_blocks, const int32_t* slots, const int32_t* positions, const float* q_norm_w,
+    const float* k_norm_w, float eps, const float* rope, int rows, int q_heads, int kv_heads,
+    int head_dim, int page_size, int write_cache, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    if (head_dim % 2 != 0 || head_dim / 2 > 64 * MAX_PAIRS) return -1;
+    qk_norm_rope_kv_kernel<<<rows, 256, 0, stream>>>(
+        (const elem_t*)qkv, ld, (elem_t*)q_out, (elem_t*)k_pages, (elem_t*)v_pages, block_table,
+        max_blocks, slots, positions, q_norm_w, k_norm_w, eps, rope, q_heads, kv_heads, head_dim,
+        page_size, write_cache);
+    return (int)hipGetLastError();
+}

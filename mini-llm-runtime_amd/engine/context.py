@@ -1,0 +1,56 @@
+"""What a part may see of the running step, and the scratch memory it may use."""
+from __future__ import annotations
+
+import torch
+
+
+class Workspace:
+    """Named scratch buffers that live as long as the runner: a buffer is allocated when a name
+    is first asked for and grows only when a larger size is asked, so steady steps allocate
+    nothing."""
+
+    def __init__(self, device):
+        self.device = torch.device(device)
+        self._buffers = {}
+
+    def get(self, name, shape, dtype):
+        count = 1
+        for extent in shape:
+            count *= int(extent)
+        key = (name, dtype)
+        buf = self._buffers.get(key)
+        if buf is None or buf.numel() < count:
+            buf = torch.empty(max(count, 1), dtype=dtype, device=self.device)
+            self._buffers[key] = buf
+        return buf[:count].view(shape)
+
+    def reserve(self, name, shape, dtype):
+        self.get(name, shape, dtype)
+
+    def bytes(self):
+        return sum(b.numel() * b.element_size() for b in self._buffers.values())
+
+
+class StepContext:
+    """One step's view for the parts: the tokens with their positions and slots (device int32
+    vectors of equal length), the segments they form (host), the cache, the kernels and the
+    scratch memory."""
+
+    def __init__(self, kernels, cache, workspace, dtype, max_positions, split_keys, split_max_tokens):
+        self.kernels, self.cache, self.workspace, self.dtype = kernels, cache, workspace, dtype
+        self.max_positions = max_positions
+        self.split_keys, self.split_max_tokens = split_keys, split_max_tokens
+        self.n_tokens = 0
+        self.token_ids = self.positions = self.slots = None
+        self.segments = []            # (slot, first row, number of tokens, first position)
+        self.max_context = 0          # largest position + 1 among the step's tokens
+
+    def attention_split(self, rows, q_heads, head_dim):
+        """(split_keys, max_splits, partial buffer): small batches over long contexts split the
+        keys of a token over several workgroups.  The splits are ranges of absolute key
+        positions, so what a token's result is does not depend on this choice beyond rounding."""
+        if self.split_keys <= 0 or rows > self.split_max_tokens or self.max_context <= self.split_keys:
+            return 0, 1, None
+        max_splits = (self.max_context + self.split_keys - 1) // self.split_keys
+        numel = self.kernels.attention_partial_numel(rows, q_heads, head_dim, max_splits)
+        return self.split_keys, max_splits, self.workspace.get("attn_partial", (numel,), torch.float32)

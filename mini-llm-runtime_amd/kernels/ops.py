@@ -1,0 +1,230 @@
+"""Python side of the HIP kernels: one `Kernels` object per element type.
+
+Every method checks on the host that its operands lie on the GPU, are contiguous, have the
+element type and the shapes that the kernel and its grid assume, and only then launches on
+torch's current stream.  A kernel that cannot take a size refuses it here with a clear error.
+There is no other implementation behind these methods: without the compiled extension, or
+without a GPU, they raise.
+"""
+from __future__ import annotations
+
+import ctypes
+
+import torch
+
+from . import build
+
+_c_int = ctypes.c_int
+_c_float = ctypes.c_float
+_c_size_t = ctypes.c_size_t
+_ptr = ctypes.c_void_p
+
+MAX_HEAD_DIM = 256          # the attention and rotation kernels keep head_dim / 64 values per lane
+ATTENTION_TILE_KEYS = 64
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _p(t):
+    return _ptr(t.data_ptr()) if t is not None else _ptr(0)
+
+
+def _stream():
+    return _ptr(torch.cuda.current_stream().cuda_stream)
+
+
+def _need(cond, message):
+    if not cond:
+        raise KernelError(message)
+
+
+def _tensor(t, name, dtype, shape=None, ndim=None):
+    _need(isinstance(t, torch.Tensor), f"{name}: expected a tensor")
+    _need(t.is_cuda, f"{name}: must lie on the GPU (there is no CPU path)")
+    _need(t.dtype == dtype, f"{name}: expected {dtype}, got {t.dtype}")
+    _need(t.is_contiguous(), f"{name}: must be contiguous")
+    if ndim is not None:
+        _need(t.dim() == ndim, f"{name}: expected {ndim} dimensions, got {tuple(t.shape)}")
+    if shape is not None:
+        _need(tuple(t.shape) == tuple(shape), f"{name}: expected shape {tuple(shape)}, got {tuple(t.shape)}")
+    return t
+
+
+def _ok(code, what):
+    if code != 0:
+        raise KernelError(f"{what}: launch failed with code {code}")
+
+
+class Kernels:
+    def __init__(self, dtype):
+        _need(dtype in (torch.float32, torch.bfloat16), f"no kernels for element type {dtype}")
+        if not torch.cuda.is_available():
+            raise KernelError("no GPU is visible: the engine's kernels are HIP only")
+        self.dtype = dtype
+        self._libs = {}
+
+    # -- libraries ---------------------------------------------------------------------------
+    @staticmethod
+    def libraries_for(parts=("elementwise", "rope_kv", "attention", "gemm")):
+        return list(parts)
+
+    def prepare(self, names):
+        """Build (if need be) and load several libraries at once."""
+        typed = [n for n in names if build.HIP_LIBRARIES[n][2]]
+        untyped = [n for n in names if not build.HIP_LIBRARIES[n][2]]
+        if typed:
+            build.ensure_built(typed, self.dtype)
+        if untyped:
+            build.ensure_built(untyped)
+        for n in names:
+            self._lib(n)
+
+    def _lib(self, name):
+        lib = self._libs.get(name)
+        if lib is None:
+            lib = build.load(name, self.dtype)
+            self._libs[name] = lib
+        return lib
+
+    # -- row-wise ----------------------------------------------------------------------------
+    def embed_gather(self, ids, table, h):
+        """h[m] = float(table[ids[m]])."""
+        rows = ids.numel()
+        _tensor(ids, "ids", torch.int32, ndim=1)
+        _tensor(table, "table", self.dtype, ndim=2)
+        vocab, width = table.shape
+        _tensor(h, "h", torch.float32, (rows, width))
+        fn = self._lib("elementwise").mlr_embed_gather
+        _ok(fn(_p(ids), _p(table), _p(h), _c_int(rows), _c_int(width), _c_int(vocab), _stream()),
+            "embed_gather")
+
+    def add_rmsnorm(self, h, delta, weight, out, eps, rows=None, write_h=True):
+        """x = h[src] + delta[src] (delta may be None); h[src] = x when write_h; out[r] =
+        rmsnorm(x) * weight, src = rows[r] or r."""
+        _tensor(h, "h", torch.float32, ndim=2)
+        m, width = h.shape
+        if delta is not None:
+            _tensor(delta, "delta", self.dtype, (m, width))
+        _tensor(weight, "weight", torch.float32, (width,))
+        if rows is not None:
+            _tensor(rows, "rows", torch.int32, ndim=1)
+            n_out = rows.numel()
+        else:
+            n_out = m
+        _tensor(out, "out", self.dtype, (n_out, width))
+        fn = self._lib("elementwise").mlr_add_rmsnorm
+        _ok(fn(_p(h), _p(delta), _p(weight), _p(out), _p(rows), _c_int(n_out), _c_int(width),
+               _c_float(eps), _c_int(1 if (write_h and delta is not None) else 0), _stream()),
+            "add_rmsnorm")
+
+    def residual_add(self, h, delta):
+        _tensor(h, "h", torch.float32, ndim=2)
+        _tensor(delta, "delta", self.dtype, tuple(h.shape))
+        fn = self._lib("elementwise").mlr_residual_add
+        _ok(fn(_p(h), _p(delta), _c_size_t(h.numel()), _stream()), "residual_add")
+
+    def silu_mul(self, gate_up, act):
+        """act[m, f] = silu(gate_up[m, f]) * gate_up[m, F + f]."""
+        _tensor(gate_up, "gate_up", self.dtype, ndim=2)
+        m, two_f = gate_up.shape
+        _need(two_f % 2 == 0, "gate_up: the width must be even")
+        _tensor(act, "act", self.dtype, (m, two_f // 2))
+        fn = self._lib("elementwise").mlr_silu_mul
+        _ok(fn(_p(gate_up), _p(act), _c_int(m), _c_int(two_f // 2), _stream()), "silu_mul")
+
+    # -- projections -------------------------------------------------------------------------
+    def gemm(self, a, w, out):
+        """out[M, N] = a[M, K] . w[N, K]^T; out has the element type or is float32."""
+        _tensor(a, "a", self.dtype, ndim=2)
+        _tensor(w, "w", self.dtype, ndim=2)
+        m, k = a.shape
+        n, k2 = w.shape
+        _need(k == k2, f"gemm: inner sizes differ ({k} and {k2})")
+        _need(out.dtype in (self.dtype, torch.float32), f"gemm: output type {out.dtype} not supported")
+        _tensor(out, "out", out.dtype, (m, n))
+        fn = self._lib("gemm").mlr_gemm
+        _ok(fn(_p(a), _p(w), _p(out), _c_int(m), _c_int(n), _c_int(k),
+               _c_int(1 if out.dtype == torch.float32 else 0), _stream()), "gemm")
+
+    # -- attention ---------------------------------------------------------------------------
+    def _check_cache(self, k_pages, v_pages, kv_heads, head_dim, page_size):
+        _tensor(k_pages, "k_pages", self.dtype, ndim=4)
+        _need(tuple(k_pages.shape[1:]) == (kv_heads, page_size, head_dim),
+              f"k_pages: expected [pages, {kv_heads}, {page_size}, {head_dim}], got {tuple(k_pages.shape)}")
+        _tensor(v_pages, "v_pages", self.dtype, tuple(k_pages.shape))
+
+    def qk_norm_rope_kv(self, qkv, q_out, k_pages, v_pages, block_table, slots, positions, q_norm_w,
+                        k_norm_w, eps, rope, q_heads, kv_heads, head_dim, page_size, write_cache=True):
+        """Per head: RMSNorm of q and k (weights may be None), rotation by `rope`
+        [max_positions, head_dim] (may be None), q into q_out, k and v into their pages."""
+        _need(head_dim % 2 == 0 and 2 <= head_dim <= MAX_HEAD_DIM,
+              f"head_dim {head_dim}: the rotation kernel takes even sizes up to {MAX_HEAD_DIM}")
+        width = (q_heads + 2 * kv_heads) * head_dim
+        _tensor(qkv, "qkv", self.dtype, ndim=2)
+        m = qkv.shape[0]
+        _need(qkv.shape[1] == width, f"qkv: expected width {width}, got {qkv.shape[1]}")
+        _tensor(q_out, "q_out", self.dtype, (m, q_heads * head_dim))
+        self._check_cache(k_pages, v_pages, kv_heads, head_dim, page_size)
+        _tensor(block_table, "block_table", torch.int32, ndim=2)
+        _tensor(slots, "slots", torch.int32, (m,))
+        _tensor(positions, "positions", torch.int32, (m,))
+        if q_norm_w is not None:
+            _tensor(q_norm_w, "q_norm_w", torch.float32, (head_dim,))
+            _tensor(k_norm_w, "k_norm_w", torch.float32, (head_dim,))
+        if rope is not None:
+            _tensor(rope, "rope", torch.float32, ndim=2)
+            _need(rope.shape[1] == head_dim, "rope: table width must equal head_dim")
+        fn = self._lib("rope_kv").mlr_qk_norm_rope_kv
+        _ok(fn(_p(qkv), _c_int(width), _p(q_out), _p(k_pages), _p(v_pages), _p(block_table),
+               _c_int(block_table.shape[1]), _p(slots), _p(positions), _p(q_norm_w), _p(k_norm_w),
+               _c_float(eps), _p(rope), _c_int(m), _c_int(q_heads), _c_int(kv_heads), _c_int(head_dim),
+               _c_int(page_size), _c_int(1 if write_cache else 0), _stream()), "qk_norm_rope_kv")
+
+    def attention_partial_numel(self, rows, q_heads, head_dim, max_splits):
+        return rows * q_heads * max_splits * (head_dim + 2)
+
+    def paged_attention(self, q, k_pages, v_pages, block_table, slots, positions, out, q_heads,
+                        kv_heads, head_dim, page_size, scale, window=None, split_keys=0, max_splits=1,
+                        partial=None):
+        """out[m, h] = softmax over the keys seen by token m (positions <= its own, within the
+        window) of q.k * scale, times v; keys and values from the pages of slots[m]."""
+        _need(1 <= head_dim <= MAX_HEAD_DIM, f"head_dim {head_dim}: the attention kernel takes up to {MAX_HEAD_DIM}")
+        _need(q_heads % kv_heads == 0, "q_heads must be a multiple of kv_heads")
+        _tensor(q, "q", self.dtype, ndim=2)
+        m = q.shape[0]
+        _need(q.shape[1] == q_heads * head_dim, "q: wrong width")
+        _tensor(out, "out", self.dtype, (m, q_heads * head_dim))
+        self._check_cache(k_pages, v_pages, kv_heads, head_dim, page_size)
+        _tensor(block_table, "block_table", torch.int32, ndim=2)
+        _tensor(slots, "slots", torch.int32, (m,))
+        _tensor(positions, "positions", torch.int32, (m,))
+        _need(kv_heads <= 65535, "too many kv heads for the grid")
+        if max_splits > 1:
+            _need(split_keys > 0 and split_keys % ATTENTION_TILE_KEYS == 0,
+                  f"split_keys must be a multiple of {ATTENTION_TILE_KEYS}")
+            _need(partial is not None, "partial buffer needed for split attention")
+            _tensor(partial, "partial", torch.float32, ndim=1)
+            _need(partial.numel() >= self.attention_partial_numel(m, q_heads, head_dim, max_splits),
+                  "partial buffer too small")
+            group = q_heads // kv_heads
+            _need(((group + 7) // 8) * max_splits <= 65535, "too many key splits for the grid")
+        fn = self._lib("attention").mlr_paged_attention
+        _ok(fn(_p(q), _p(k_pages), _p(v_pages), _p(block_table), _c_int(block_table.shape[1]), _p(slots),
+               _p(positions), _p(out), _p(partial), _c_int(m), _c_int(q_heads), _c_int(kv_heads),
+               _c_int(head_dim), _c_int(page_size), _c_int(window or 0), _c_float(scale),
+               _c_int(split_keys), _c_int(max_splits), _stream()), "paged_attention")
+
+    # -- sampling ----------------------------------------------------------------------------
+    def sample(self, logits, temperature, uniform, tokens, status):
+        """tokens[r] = argmax (temperature <= 0) or the inverse-CDF draw at uniform[r]."""
+        _tensor(logits, "logits", torch.float32, ndim=2)
+        rows, vocab = logits.shape
+        _tensor(temperature, "temperature", torch.float32, (rows,))
+        _tensor(uniform, "uniform", torch.float32, (rows,))
+        _tensor(tokens, "tokens", torch.int32, (rows,))
+        _tensor(status, "status", torch.int32, (2,))
+        fn = self._lib("sampling").mlr_sample
+        _ok(fn(_p(logits), _c_int(rows), _c_int(vocab), _p(temperature), _p(uniform), _p(tokens),
+               _p(status), _stream()), "sample")

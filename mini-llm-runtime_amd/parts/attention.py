@@ -1,0 +1,85 @@
+"""Grouped-query attention over the paged cache: fused q/k/v projection, per-head RMSNorm of q
+and k before the rotation, rotation, write of k and v into their pages, attention of every
+token of the step over the keys at positions <= its own (optionally only a window of them),
+output projection.  Order of operations as in the reference (src/minillm/runtime.cpp:250-319,
+src/minillm/cuda/layer.cpp:42-63).  Consecutive query heads share a kv head."""
+from __future__ import annotations
+
+import torch
+
+from ..cache.manager import KvSpec
+from ..weights.loader import WeightSpec
+from .registry import PartError, build_part, register_part
+
+
+@register_part("mixer", "gqa_attention")
+class GqaAttention:
+    def __init__(self, spec):
+        self.spec = spec
+        s = spec
+        if s.q_heads % s.kv_heads != 0:
+            raise PartError(f"q_heads {s.q_heads} is no multiple of kv_heads {s.kv_heads}")
+        if s.head_dim % 16 != 0 or s.head_dim > 256:
+            raise PartError(f"head_dim {s.head_dim}: the attention kernels take multiples of 16 up to 256")
+        if s.window is not None and s.window < 1:
+            raise PartError("window must be positive")
+        self.q_norm = build_part("norm", s.qk_norm) if s.qk_norm is not None else None
+        self.k_norm = build_part("norm", s.qk_norm) if s.qk_norm is not None else None
+        if s.qk_norm is not None and s.qk_norm.size != s.head_dim:
+            raise PartError("the q/k norm must span one head")
+        self.position = build_part("position", s.position) if s.position is not None else None
+        if s.position is not None and s.position.dim != s.head_dim:
+            raise PartError("the rotation must span the whole head")
+        self.qkv = None
+        self.o = None
+
+    def weight_specs(self):
+        s = self.spec
+        specs = {
+            "q_proj": WeightSpec((s.q_heads * s.head_dim, s.hidden)),
+            "k_proj": WeightSpec((s.kv_heads * s.head_dim, s.hidden)),
+            "v_proj": WeightSpec((s.kv_heads * s.head_dim, s.hidden)),
+            "o_proj": WeightSpec((s.hidden, s.q_heads * s.head_dim)),
+        }
+        if self.q_norm is not None:
+            specs["q_norm.weight"] = self.q_norm.weight_specs()["weight"]
+            specs["k_norm.weight"] = self.k_norm.weight_specs()["weight"]
+        return specs
+
+    def bind(self, weights):
+        # rows of a projection are independent sums, so stacking q, k, v changes no result
+        self.qkv = torch.cat([weights["q_proj"], weights["k_proj"], weights["v_proj"]], dim=0).contiguous()
+        self.o = weights["o_proj"]
+        if self.q_norm is not None:
+            self.q_norm.bind({"weight": weights["q_norm.weight"]})
+            self.k_norm.bind({"weight": weights["k_norm.weight"]})
+
+    def cache_spec(self):
+        return KvSpec(self.spec.kv_heads, self.spec.head_dim, self.spec.window)
+
+    def libraries(self):
+        return ["gemm", "rope_kv", "attention"]
+
+    def forward(self, ctx, x, cache_id, write_cache=True):
+        s = self.spec
+        k = ctx.kernels
+        m = x.shape[0]
+        view = ctx.cache.kv_view(cache_id)
+        qkv = ctx.workspace.get("qkv", (m, (s.q_heads + 2 * s.kv_heads) * s.head_dim), x.dtype)
+        k.gemm(x, self.qkv, qkv)
+        q = ctx.workspace.get("q", (m, s.q_heads * s.head_dim), x.dtype)
+        rope = self.position.rotation_table(ctx.max_positions, x.device) if self.position is not None else None
+        k.qk_norm_rope_kv(
+            qkv, q, view.k_pages, view.v_pages, view.block_table, ctx.slots, ctx.positions,
+            self.q_norm.weight if self.q_norm is not None else None,
+            self.k_norm.weight if self.k_norm is not None else None,
+            self.q_norm.eps if self.q_norm is not None else 0.0, rope,
+            s.q_heads, s.kv_heads, s.head_dim, view.page_size, write_cache)
+        attn = ctx.workspace.get("attn", (m, s.q_heads * s.head_dim), x.dtype)
+        split_keys, max_splits, partial = ctx.attention_split(m, s.q_heads, s.head_dim)
+        k.paged_attention(q, view.k_pages, view.v_pages, view.block_table, ctx.slots, ctx.positions, attn,
+                          s.q_heads, s.kv_heads, s.head_dim, view.page_size, float(s.scale),
+                          window=s.window, split_keys=split_keys, max_splits=max_splits, partial=partial)
+        out = ctx.workspace.get("mixer_out", (m, s.hidden), x.dtype)
+        k.gemm(attn, self.o, out)
+        return out

@@ -1,0 +1,26 @@
+"""Arrangement of the parts in a layer.  Pre-norm residual block (src/minillm/runtime.cpp:245-337):
+h += mixer(norm1(h)); h += ffn(norm2(h)).  The residual stream h is float; every add into it is
+fused with the norm that follows, so a block hands its last output on as `pending` instead of
+adding it itself."""
+from __future__ import annotations
+
+from .registry import build_part, register_part
+
+
+@register_part("block", "prenorm")
+class PreNormBlock:
+    def __init__(self, spec):
+        self.norm1 = build_part("norm", spec.norm1)
+        self.mixer = build_part("mixer", spec.mixer)
+        self.norm2 = build_part("norm", spec.norm2)
+        self.ffn = build_part("ffn", spec.ffn)
+
+    def parts(self):
+        return {"norm1": self.norm1, "mixer": self.mixer, "norm2": self.norm2, "ffn": self.ffn}
+
+    def forward(self, ctx, h, pending, cache_id, write_cache=True):
+        normed = ctx.workspace.get("normed", tuple(h.shape), ctx.dtype)
+        self.norm1.forward(ctx, h, pending, normed)
+        mixed = self.mixer.forward(ctx, normed, cache_id, write_cache)
+        self.norm2.forward(ctx, h, mixed, normed)
+        return self.ffn.forward(ctx, normed)

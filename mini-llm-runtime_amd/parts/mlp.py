@@ -1,0 +1,42 @@
+"""SwiGLU feed-forward: out = (silu(x Wgate^T) * (x Wup^T)) Wdown^T with silu(g) = g / (1 + exp(-g))
+(src/minillm/runtime.cpp:323-336).  Gate and up are one stacked projection."""
+from __future__ import annotations
+
+import torch
+
+from ..weights.loader import WeightSpec
+from .registry import PartError, register_part
+
+
+@register_part("ffn", "swiglu")
+class SwiGluMlp:
+    def __init__(self, spec):
+        if spec.activation != "silu":
+            raise PartError(f"activation {spec.activation!r} is not built (silu)")
+        self.spec = spec
+        self.gate_up = None
+        self.down = None
+
+    def weight_specs(self):
+        s = self.spec
+        return {"gate_proj": WeightSpec((s.intermediate, s.hidden)),
+                "up_proj": WeightSpec((s.intermediate, s.hidden)),
+                "down_proj": WeightSpec((s.hidden, s.intermediate))}
+
+    def bind(self, weights):
+        self.gate_up = torch.cat([weights["gate_proj"], weights["up_proj"]], dim=0).contiguous()
+        self.down = weights["down_proj"]
+
+    def libraries(self):
+        return ["gemm", "elementwise"]
+
+    def forward(self, ctx, x):
+        s = self.spec
+        m = x.shape[0]
+        gate_up = ctx.workspace.get("gate_up", (m, 2 * s.intermediate), x.dtype)
+        ctx.kernels.gemm(x, self.gate_up, gate_up)
+        act = ctx.workspace.get("act", (m, s.intermediate), x.dtype)
+        ctx.kernels.silu_mul(gate_up, act)
+        out = ctx.workspace.get("ffn_out", (m, s.hidden), x.dtype)
+        ctx.kernels.gemm(act, self.down, out)
+        return out

@@ -1,0 +1,135 @@
+"""A decoder model put together from a `ModelSpec`: embedding, the layers (blocks of parts) in
+the order the schedule gives, a final norm on the wanted rows and the output projection.
+
+Which class builds which part is decided by the specs' `kind`s through the parts registry;
+which tensor of the file feeds which part is decided by the architecture's configuration
+class (`global_tensor_name`, `layer_tensor_name`).  The model itself knows no architecture.
+"""
+from __future__ import annotations
+
+import torch
+
+from ..config import load_config
+from ..weights.loader import WeightSpec, load_weights
+from .registry import PartError, build_part
+
+
+def build_blocks(spec):
+    return [build_part("block", layer) for layer in spec.layers]
+
+
+def _tensor_plan(config, spec, blocks):
+    """[(global name, WeightSpec, owner, local name)] for every tensor of the model; owner is
+    "embed", "lm_head", ("final_norm",) or (layer index, part name)."""
+    plan = [(config.global_tensor_name("embed"), WeightSpec((spec.vocab_size, spec.hidden)), "embed", None)]
+    final = build_part("norm", spec.final_norm)
+    for local, ws in final.weight_specs().items():
+        plan.append((config.global_tensor_name(f"final_norm.{local}"), ws, ("final_norm",), local))
+    plan.append((config.global_tensor_name("lm_head"),
+                 WeightSpec((spec.vocab_size, spec.hidden), optional=spec.tie_embeddings), "lm_head", None))
+    for i, block in enumerate(blocks):
+        for part_name, part in block.parts().items():
+            for local, ws in part.weight_specs().items():
+                plan.append((config.layer_tensor_name(i, part_name, local), ws, (i, part_name), local))
+    names = [p[0] for p in plan]
+    if len(set(names)) != len(names):
+        raise PartError("two parts claim the same tensor name")
+    return plan, final
+
+
+def expected_tensors(config):
+    """{tensor name: WeightSpec} of the architecture described by `config`."""
+    spec = config.model_spec()
+    plan, _ = _tensor_plan(config, spec, build_blocks(spec))
+    return {name: ws for name, ws, _, _ in plan}
+
+
+class DecoderModel:
+    def __init__(self, config, weights, dtype, device):
+        """`weights`: {tensor name: device tensor} as `load_weights` returns them."""
+        self.config = config
+        self.spec = spec = config.model_spec()
+        self.dtype, self.device = dtype, torch.device(device)
+        if len(spec.schedule) == 0:
+            raise PartError("the schedule runs no layer")
+        for run in spec.schedule:
+            if not 0 <= run.layer < len(spec.layers):
+                raise PartError(f"the schedule names layer {run.layer} of {len(spec.layers)}")
+        self.blocks = build_blocks(spec)
+        plan, self.final_norm = _tensor_plan(config, spec, self.blocks)
+        by_owner = {}
+        for name, ws, owner, local in plan:
+            if name not in weights:
+                continue
+            if owner == "embed":
+                self.embed = weights[name]
+            elif owner == "lm_head":
+                self.lm_head = weights[name]
+            else:
+                by_owner.setdefault(owner, {})[local] = weights[name]
+        if not hasattr(self, "lm_head"):
+            self.lm_head = self.embed          # tied: the same memory, no copy
+        self.final_norm.bind(by_owner[("final_norm",)])
+        for i, block in enumerate(self.blocks):
+            for part_name, part in block.parts().items():
+                part.bind(by_owner.get((i, part_name), {}))
+        # cache entries: one per cache id the schedule names
+        n_entries = 1 + max(run.cache for run in spec.schedule)
+        self.cache_entry_specs = [None] * n_entries
+        writers = set()
+        for run in spec.schedule:
+            cs = self.blocks[run.layer].mixer.cache_spec()
+            if self.cache_entry_specs[run.cache] is None:
+                self.cache_entry_specs[run.cache] = cs
+            elif self.cache_entry_specs[run.cache] != cs:
+                raise PartError(f"cache entry {run.cache} is shared by mixers with different needs")
+            if run.write_cache:
+                writers.add(run.cache)
+        for cid in range(n_entries):
+            if self.cache_entry_specs[cid] is not None and cid not in writers:
+                raise PartError(f"cache entry {cid} is read but never written")
+
+    @classmethod
+    def load(cls, folder, dtype, device="cuda:0"):
+        config = load_config(folder)
+        weights = load_weights(folder, expected_tensors(config), dtype, device)
+        return cls(config, weights, dtype, device)
+
+    def libraries(self):
+        names = {"elementwise", "gemm"}
+        for block in self.blocks:
+            for part in block.parts().values():
+                if hasattr(part, "libraries"):
+                    names.update(part.libraries())
+        return sorted(names)
+
+    def weight_bytes(self):
+        seen, total = set(), 0
+        tensors = [self.embed, self.lm_head, self.final_norm.weight]
+        for block in self.blocks:
+            for part in block.parts().values():
+                tensors += [v for v in vars(part).values() if isinstance(v, torch.Tensor)]
+        for t in tensors:
+            if t.data_ptr() not in seen:
+                seen.add(t.data_ptr())
+                total += t.numel() * t.element_size()
+        return total
+
+    def forward(self, ctx, want_rows):
+        """Run the step's tokens through every scheduled layer; logits float [R, V] at the rows
+        `want_rows` (device int32, indices into the step's tokens), or None when R = 0."""
+        k = ctx.kernels
+        m = ctx.n_tokens
+        h = ctx.workspace.get("hidden", (m, self.spec.hidden), torch.float32)
+        k.embed_gather(ctx.token_ids, self.embed, h)
+        pending = None
+        for run in self.spec.schedule:
+            pending = self.blocks[run.layer].forward(ctx, h, pending, run.cache, run.write_cache)
+        r = 0 if want_rows is None else want_rows.numel()
+        if r == 0:
+            return None
+        final = ctx.workspace.get("final", (r, self.spec.hidden), self.dtype)
+        self.final_norm.forward(ctx, h, pending, final, rows=want_rows, write_h=False)
+        logits = ctx.workspace.get("logits", (r, self.spec.vocab_size), torch.float32)
+        k.gemm(final, self.lm_head, logits)
+        return logits

@@ -1,0 +1,51 @@
+"""Registries of the parts a layer is put together from.  A spec's `kind` picks the class; a
+class is registered with a decorator and may live anywhere (a test can register a toy part
+without touching this package).
+
+Interfaces (B = the tokens of a step, E = the model width, T = the engine's element type):
+
+  norm            weight_specs() -> {local name: WeightSpec};  bind({local name: tensor});
+                  forward(ctx, h, delta, out, rows=None, write_h=True): h is the float residual
+                  stream [B, E]; x = h + delta (delta may be None) is written back to h when
+                  write_h; out[r] = norm(x[rows[r] or r]) as T.
+  position        rotation_table(max_positions, device) -> float [max_positions, dim] with cos
+                  in the first half and sin in the second, or None for "no rotation".
+  mixer           weight_specs(), bind();  cache_spec() -> KvSpec | StateSpec | None;
+                  libraries() -> names of the kernel libraries it launches;
+                  forward(ctx, x, cache_id, write_cache) -> T [B, E], x being the normed input.
+  feed-forward    weight_specs(), bind(), libraries();  forward(ctx, x) -> T [B, E].
+  block           built from (norm1, mixer, norm2, ffn);  forward(ctx, h, pending, cache_id,
+                  write_cache) -> the next pending delta: a block adds `pending` (the previous
+                  block's last output) into h itself, fused with its first norm.
+
+No part is told which model it is in; sizes and constants arrive through its spec.
+"""
+from __future__ import annotations
+
+_REGISTRIES = {"norm": {}, "position": {}, "mixer": {}, "ffn": {}, "block": {}}
+
+
+class PartError(ValueError):
+    pass
+
+
+def register_part(family, kind):
+    if family not in _REGISTRIES:
+        raise PartError(f"unknown part family {family!r}")
+
+    def add(cls):
+        _REGISTRIES[family][kind] = cls
+        return cls
+    return add
+
+
+def part_class(family, kind):
+    try:
+        return _REGISTRIES[family][kind]
+    except KeyError:
+        known = ", ".join(sorted(_REGISTRIES.get(family, {}))) or "none"
+        raise PartError(f"no {family} part of kind {kind!r}; known: {known}") from None
+
+
+def build_part(family, spec, **kwargs):
+    return part_class(family, spec.kind)(spec, **kwargs)

@@ -1,0 +1,383 @@
+"""Each HIP kernel alone against a plain formula in float64, at sizes other than the tiny
+models' (the reference tests each op against a host formula in the same way,
+tests/cuda_ops_tests.cu:38-72)."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def tol(dtype):
+    return dict(atol=2e-4, rtol=2e-4) if dtype == torch.float32 else dict(atol=2e-2, rtol=2e-2)
+
+
+def kernels(dtype):
+    from mini_llm_runtime_amd.kernels import Kernels
+    return Kernels(dtype)
+
+
+def rnd(shape, dtype, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (scale * torch.randn(shape, generator=g)).to(dtype).cuda()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("width", [1, 17, 76, 128, 1000, 3072])
+def test_embed_gather(dtype, width):
+    k = kernels(dtype)
+    table = rnd((37, width), dtype, 1)
+    ids = torch.tensor([0, 36, 5, 5, 17], dtype=torch.int32).cuda()
+    h = torch.full((5, width), 7.0, device="cuda")
+    k.embed_gather(ids, table, h)
+    assert torch.equal(h, table.float()[ids.long()])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("width", [1, 17, 31, 32, 33, 128, 1024, 3072])
+def test_add_rmsnorm(dtype, width):
+    k = kernels(dtype)
+    rows = 5
+    h0 = rnd((rows, width), torch.float32, 2, 3.0)
+    delta = rnd((rows, width), dtype, 3)
+    w = rnd((width,), torch.float32, 4)
+    eps = 1e-5
+    x = h0.double() + delta.double()
+    want = x * torch.rsqrt((x * x).mean(-1, keepdim=True) + eps) * w.double()
+    # fused add: h is updated
+    h = h0.clone()
+    out = torch.empty((rows, width), dtype=dtype, device="cuda")
+    k.add_rmsnorm(h, delta, w, out, eps)
+    torch.testing.assert_close(h.double(), x, atol=1e-6, rtol=1e-6)
+    torch.testing.assert_close(out.double(), want, **tol(dtype))
+    # gathered rows, h untouched
+    h = h0.clone()
+    idx = torch.tensor([4, 0, 4], dtype=torch.int32).cuda()
+    out = torch.empty((3, width), dtype=dtype, device="cuda")
+    k.add_rmsnorm(h, delta, w, out, eps, rows=idx, write_h=False)
+    assert torch.equal(h, h0)
+    torch.testing.assert_close(out.double(), want[idx.long()], **tol(dtype))
+    # no delta
+    out = torch.empty((rows, width), dtype=dtype, device="cuda")
+    k.add_rmsnorm(h, None, w, out, eps)
+    x = h0.double()
+    torch.testing.assert_close(out.double(), x * torch.rsqrt((x * x).mean(-1, keepdim=True) + eps) * w.double(),
+                               **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rmsnorm_extremes(dtype):
+    """Amplitudes from 0 to 1e15 (tests/cuda_ops_tests.cu:274-301) stay finite."""
+    k = kernels(dtype)
+    width = 257
+    amps = [0.0, 1e-15, 1.0, 1e15]
+    h = torch.zeros((len(amps), width))
+    for r, a in enumerate(amps):
+        h[r, 0::3] = -a
+        h[r, 1::3] = 0.5 * a
+        h[r, 2::3] = 0.5 * a
+    h = h.cuda()
+    w = torch.ones(width, device="cuda")
+    out = torch.empty((len(amps), width), dtype=dtype, device="cuda")
+    k.add_rmsnorm(h, None, w, out, 1e-6)
+    x = h.double()
+    want = x * torch.rsqrt((x * x).mean(-1, keepdim=True) + 1e-6)
+    assert torch.isfinite(out.float()).all()
+    torch.testing.assert_close(out.double(), want, **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_silu_mul_and_residual(dtype):
+    k = kernels(dtype)
+    inter = 100
+    gate_up = rnd((7, 2 * inter), dtype, 5, 3.0)
+    gate_up[0, :9] = torch.tensor([0, 1, -1, 80, -80, 1e4, -1e4, 30, -30], dtype=dtype)
+    act = torch.empty((7, inter), dtype=dtype, device="cuda")
+    k.silu_mul(gate_up, act)
+    g, u = gate_up.double()[:, :inter], gate_up.double()[:, inter:]
+    want = g / (1 + torch.exp(-g)) * u
+    assert torch.isfinite(act.float()).all()
+    torch.testing.assert_close(act.double(), want, **tol(dtype))
+    h0 = rnd((7, inter), torch.float32, 6)
+    h = h0.clone()
+    k.residual_add(h, act)
+    torch.testing.assert_close(h, h0 + act.float())
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("mnk", [(7, 19, 33), (5, 37, 131), (1, 311, 80), (16, 64, 64), (17, 130, 100),
+                                 (64, 200, 76), (65, 257, 256), (200, 300, 1024), (2, 2048, 1024)])
+def test_gemm(dtype, mnk):
+    """Odd shapes as in the reference's GEMM test (tests/cuda_unit_tests.cu:207-209)."""
+    m, n, kk = mnk
+    k = kernels(dtype)
+    a = rnd((m, kk), dtype, 7)
+    w = rnd((n, kk), dtype, 8)
+    want = a.double() @ w.double().T
+    for out_dtype in {dtype, torch.float32}:
+        out = torch.full((m, n), float("nan"), dtype=out_dtype, device="cuda")
+        k.gemm(a, w, out)
+        t = dict(atol=1e-4 * math.sqrt(kk), rtol=1e-5) if out_dtype == torch.float32 else \
+            dict(atol=2e-2 * math.sqrt(kk) / 4, rtol=2e-2)
+        torch.testing.assert_close(out.double(), want, **t)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_gemm_rows_do_not_depend_on_the_batch(dtype):
+    k = kernels(dtype)
+    a = rnd((200, 264), dtype, 9)
+    w = rnd((150, 264), dtype, 10)
+    full = torch.empty((200, 150), dtype=dtype, device="cuda")
+    k.gemm(a, w, full)
+    for lo, hi in [(0, 1), (3, 20), (100, 164), (130, 200)]:
+        part = torch.empty((hi - lo, 150), dtype=dtype, device="cuda")
+        k.gemm(a[lo:hi].contiguous(), w, part)
+        assert torch.equal(part, full[lo:hi])
+
+
+def plain_rope(x, pos, base):
+    """x [T, H, D] float64 by the plain implementation's rotation (angles held in 32-bit, as the
+    reference computes them)."""
+    from plain.qwen3_plain import rope_cos_sin, rope_rotate
+    cos, sin = rope_cos_sin(pos.numpy(), x.shape[-1], base)
+    return torch.from_numpy(rope_rotate(x.numpy(), cos, sin))
+
+
+def rope_table(max_pos, dim, base):
+    from mini_llm_runtime_amd.config import PositionSpec
+    from mini_llm_runtime_amd.parts.rope import RopeSplitHalf
+    return RopeSplitHalf(PositionSpec("rope_split_half", dim, base)).rotation_table(max_pos, "cuda")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", [(1, 1, 16, 4), (8, 2, 128, 16), (6, 3, 48, 8), (16, 16, 256, 32), (5, 1, 32, 1)])
+def test_qk_norm_rope_kv(dtype, shape):
+    """Positions around page edges and far ones (tests/cuda_ops_tests.cu:326); shuffled pages."""
+    hq, hkv, d, page = shape
+    k = kernels(dtype)
+    positions = [0, 1, page - 1, page, page + 1, 2 * page + 3, 1535, 2047]
+    positions = sorted(set(p for p in positions))
+    m = len(positions)
+    max_blocks = 2048 // page + 1
+    # two slots: even rows in slot 1, odd rows in slot 0; pages handed out in a shuffled order
+    slots = torch.tensor([1 - (i % 2) for i in range(m)], dtype=torch.int32)
+    n_pages = 2 * m + 3
+    perm = torch.randperm(n_pages, generator=torch.Generator().manual_seed(11)).tolist()
+    table = torch.full((2, max_blocks), -1, dtype=torch.int32)
+    for i, p in enumerate(positions):
+        table[slots[i], p // page] = perm.pop()
+    qkv = rnd((m, (hq + 2 * hkv) * d), dtype, 12)
+    qw, kw = rnd((d,), torch.float32, 13) + 1, rnd((d,), torch.float32, 14) + 1
+    eps, base = 1e-5, 1e6
+    rope = rope_table(2048, d, base)
+    k_pages = torch.full((n_pages, hkv, page, d), float("nan"), dtype=dtype, device="cuda")
+    v_pages = torch.full((n_pages, hkv, page, d), float("nan"), dtype=dtype, device="cuda")
+    q_out = torch.empty((m, hq * d), dtype=dtype, device="cuda")
+    pos_t = torch.tensor(positions, dtype=torch.int32)
+    k.qk_norm_rope_kv(qkv, q_out, k_pages, v_pages, table.cuda(), slots.cuda(), pos_t.cuda(), qw, kw, eps,
+                      rope, hq, hkv, d, page)
+    x = qkv.double().cpu()
+    q = x[:, :hq * d].view(m, hq, d)
+    kk = x[:, hq * d:(hq + hkv) * d].view(m, hkv, d)
+    v = x[:, (hq + hkv) * d:].view(m, hkv, d)
+
+    def norm(t, w):
+        return t * torch.rsqrt((t * t).mean(-1, keepdim=True) + eps) * w.double().cpu()
+    q_want = plain_rope(norm(q, qw), pos_t, base)
+    k_want = plain_rope(norm(kk, kw), pos_t, base)
+    torch.testing.assert_close(q_out.double().cpu().view(m, hq, d), q_want, **tol(dtype))
+    written = torch.zeros((n_pages, page), dtype=torch.bool)
+    for i, p in enumerate(positions):
+        pg = table[slots[i], p // page].item()
+        written[pg, p % page] = True
+        torch.testing.assert_close(k_pages[pg, :, p % page].double().cpu(), k_want[i], **tol(dtype))
+        assert torch.equal(v_pages[pg, :, p % page].cpu(), qkv[i, (hq + hkv) * d:].view(hkv, d).cpu())
+    # nothing else was touched
+    untouched = ~written[:, None, :, None].expand(n_pages, hkv, page, d)
+    assert torch.isnan(k_pages.float().cpu()[untouched]).all()
+    assert torch.isnan(v_pages.float().cpu()[untouched]).all()
+    # no norm, no rotation, no cache write
+    k2 = torch.full_like(k_pages, float("nan"))
+    k.qk_norm_rope_kv(qkv, q_out, k2, v_pages, table.cuda(), slots.cuda(), pos_t.cuda(), None, None, 0.0,
+                      None, hq, hkv, d, page, write_cache=False)
+    assert torch.equal(q_out.cpu(), qkv[:, :hq * d].cpu())
+    assert torch.isnan(k2.float()).all()
+
+
+def plain_attention(q, keys, values, scale, window):
+    """One query row over its visible keys, float64.  q [Hq, D]; keys, values [L, Hkv, D]."""
+    hq, hkv = q.shape[0], keys.shape[1]
+    g = hq // hkv
+    L = keys.shape[0]
+    lo = 0 if window is None else max(0, L - window)
+    out = torch.zeros_like(q)
+    for h in range(hq):
+        s = (keys[lo:, h // g] @ q[h]) * scale
+        a = torch.softmax(s, dim=0)
+        out[h] = a @ values[lo:, h // g]
+    return out
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("case", [
+    # (q heads, kv heads, head_dim, page, lengths of the requests, window, split_keys)
+    (4, 1, 16, 16, [1, 17, 33], None, 0),
+    (4, 2, 128, 16, [15, 16, 17, 127, 128, 129], None, 0),
+    (16, 8, 128, 16, [300, 1], None, 64),
+    (6, 3, 48, 8, [70, 131], None, 64),
+    (20, 1, 32, 32, [100], None, 0),
+    (4, 4, 256, 16, [65], None, 0),
+    (4, 2, 64, 16, [200, 40], 33, 0),
+    (4, 2, 64, 16, [200, 40], 64, 128),
+    (2, 1, 16, 4, [1000], None, 256),
+])
+def test_paged_attention(dtype, case):
+    """Every length is one request whose LAST token is the query (a decoded token) plus, for the
+    first request, a query at every position (a whole prompt); pages shuffled.  Shapes after
+    tests/cuda_layer_tests.cpp:528-536."""
+    hq, hkv, d, page, lengths, window, split_keys = case
+    k = kernels(dtype)
+    g = torch.Generator().manual_seed(20)
+    max_len = max(lengths)
+    max_blocks = (max_len + page - 1) // page
+    n_pages = sum((L + page - 1) // page for L in lengths) + 2
+    perm = torch.randperm(n_pages, generator=g).tolist()
+    table = torch.full((len(lengths), max_blocks), -1, dtype=torch.int32)
+    k_pages = torch.full((n_pages, hkv, page, d), float("nan"), dtype=dtype)
+    v_pages = torch.full((n_pages, hkv, page, d), float("nan"), dtype=dtype)
+    keys, values = [], []
+    for s, L in enumerate(lengths):
+        kk = torch.randn((L, hkv, d), generator=g).to(dtype)
+        vv = torch.randn((L, hkv, d), generator=g).to(dtype)
+        keys.append(kk)
+        values.append(vv)
+        for b in range((L + page - 1) // page):
+            pg = perm.pop()
+            table[s, b] = pg
+            n = min(page, L - b * page)
+            k_pages[pg, :, :n] = kk[b * page:b * page + n].transpose(0, 1)
+            v_pages[pg, :, :n] = vv[b * page:b * page + n].transpose(0, 1)
+    rows = [(0, p) for p in range(lengths[0])] + [(s, L - 1) for s, L in enumerate(lengths) if s > 0]
+    m = len(rows)
+    q = (torch.randn((m, hq, d), generator=g) * 2).to(dtype)
+    scale = 1 / math.sqrt(d)
+    out = torch.full((m, hq * d), float("nan"), dtype=dtype, device="cuda")
+    slots = torch.tensor([r[0] for r in rows], dtype=torch.int32).cuda()
+    pos = torch.tensor([r[1] for r in rows], dtype=torch.int32).cuda()
+    max_splits, partial = 1, None
+    if split_keys:
+        max_splits = (max_len + split_keys - 1) // split_keys
+        partial = torch.full((k.attention_partial_numel(m, hq, d, max_splits),), float("nan"), device="cuda")
+    k.paged_attention(q.view(m, hq * d).cuda(), k_pages.cuda(), v_pages.cuda(), table.cuda(), slots, pos, out,
+                      hq, hkv, d, page, scale, window=window, split_keys=split_keys, max_splits=max_splits,
+                      partial=partial)
+    got = out.double().cpu().view(m, hq, d)
+    for i, (s, p) in enumerate(rows):
+        want = plain_attention(q[i].double(), keys[s][:p + 1].double(), values[s][:p + 1].double(), scale, window)
+        torch.testing.assert_close(got[i], want, **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_finds_one_far_key(dtype):
+    """One key among a thousand matches the query (scaled so that its score stands out): the
+    output must be that key's value, wherever in the pages it lies."""
+    k = kernels(dtype)
+    hq = hkv = 1
+    d, page, L = 64, 16, 1000
+    g = torch.Generator().manual_seed(21)
+    for far in [0, 15, 16, 63, 64, 511, 512, 998, 999]:
+        kk = 0.05 * torch.randn((L, 1, d), generator=g)
+        vv = torch.randn((L, 1, d), generator=g)
+        q = torch.randn((1, d), generator=g)
+        kk[far, 0] = 40 * q[0] / q[0].norm()
+        n_blocks = (L + page - 1) // page
+        table = torch.arange(n_blocks - 1, -1, -1, dtype=torch.int32)[None, :].contiguous()
+        k_pages = torch.zeros((n_blocks, 1, page, d))
+        v_pages = torch.zeros((n_blocks, 1, page, d))
+        for b in range(n_blocks):
+            n = min(page, L - b * page)
+            k_pages[table[0, b], 0, :n] = kk[b * page:b * page + n, 0]
+            v_pages[table[0, b], 0, :n] = vv[b * page:b * page + n, 0]
+        out = torch.empty((1, d), dtype=dtype, device="cuda")
+        for split_keys in (0, 128):
+            max_splits = (L + split_keys - 1) // split_keys if split_keys else 1
+            partial = torch.empty(k.attention_partial_numel(1, 1, d, max_splits), device="cuda") if split_keys else None
+            k.paged_attention(q.to(dtype).cuda(), k_pages.to(dtype).cuda(), v_pages.to(dtype).cuda(), table.cuda(),
+                              torch.zeros(1, dtype=torch.int32).cuda(), torch.tensor([L - 1], dtype=torch.int32).cuda(),
+                              out, 1, 1, d, page, 1.0, split_keys=split_keys, max_splits=max_splits, partial=partial)
+            torch.testing.assert_close(out.float().cpu()[0], vv[far, 0].to(dtype).float(), atol=3e-2, rtol=3e-2)
+
+
+@pytest.mark.parametrize("vocab", [1, 31, 32, 33, 257, 1024, 1025, 151936])
+def test_sample_greedy(vocab):
+    """Ties -> lowest id; a NaN or infinity -> -1 and the status names the row
+    (tests/cuda_ops_tests.cu:408-435)."""
+    k = kernels(torch.float32)
+    g = torch.Generator().manual_seed(vocab)
+    logits = torch.randn((4, vocab), generator=g)
+    if vocab > 2:
+        logits[1, vocab - 1] = 50.0
+        logits[1, vocab // 2] = 50.0
+        logits[2, 0] = 60.0
+    if vocab > 40:
+        logits[3, 37] = float("nan")
+    temp = torch.zeros(4).cuda()
+    u = torch.zeros(4).cuda()
+    tokens = torch.full((4,), -7, dtype=torch.int32).cuda()
+    status = torch.zeros(2, dtype=torch.int32).cuda()
+    k.sample(logits.cuda(), temp, u, tokens, status)
+    got = tokens.cpu().tolist()
+    for r in range(4):
+        row = logits[r]
+        if not torch.isfinite(row).all():
+            assert got[r] == -1
+        else:
+            assert got[r] == int(np.argmax(row.numpy()))
+    if vocab > 40:
+        assert status.cpu().tolist() == [1, 3]
+    else:
+        assert status.cpu().tolist() == [0, 2 ** 31 - 1]
+    if vocab > 2:
+        assert got[1] == vocab // 2 and got[2] == 0
+
+
+@pytest.mark.parametrize("vocab", [5, 311, 4099, 151936])
+def test_sample_temperature(vocab):
+    """The drawn token's slice of the CDF of softmax(logits / T) (float64) holds u."""
+    from plain.qwen3_plain import temperature_cdf
+    k = kernels(torch.float32)
+    g = torch.Generator().manual_seed(vocab + 1)
+    rows = 64
+    logits = 3 * torch.randn((rows, vocab), generator=g)
+    temp = torch.rand(rows, generator=g) * 1.5 + 0.2
+    u = torch.rand(rows, generator=g)
+    u[0], u[1] = 0.0, 0.9999999
+    tokens = torch.empty(rows, dtype=torch.int32).cuda()
+    status = torch.zeros(2, dtype=torch.int32).cuda()
+    k.sample(logits.cuda(), temp.cuda(), u.cuda(), tokens, status)
+    got = tokens.cpu().tolist()
+    for r in range(rows):
+        cdf = temperature_cdf(logits[r].numpy(), float(temp[r]))
+        t = got[r]
+        lo = cdf[t - 1] if t > 0 else 0.0
+        assert lo - 1e-4 <= float(u[r]) <= cdf[t] + 1e-4, (r, t, lo, float(u[r]), cdf[t])
+
+
+def test_sample_frequencies():
+    """Empirical frequencies over many draws follow softmax(logits / T)."""
+    k = kernels(torch.float32)
+    logits = torch.tensor([0.0, 1.0, 2.0, -1.0, 0.5, 3.0, -2.0])
+    temp_value = 0.8
+    rows = 20000
+    g = torch.Generator().manual_seed(5)
+    u = torch.rand(rows, generator=g).cuda()
+    tokens = torch.empty(rows, dtype=torch.int32).cuda()
+    k.sample(logits[None, :].repeat(rows, 1).cuda().contiguous(), torch.full((rows,), temp_value).cuda(), u, tokens,
+             torch.zeros(2, dtype=torch.int32).cuda())
+    freq = torch.bincount(tokens.cpu().long(), minlength=7).double() / rows
+    want = torch.softmax(logits.double() / temp_value, 0)
+    assert (freq - want).abs().max() < 0.015
