@@ -1,0 +1,302 @@
+"""The scheduler above the step function: admission, portions of prompts under a token budget,
+decoding, finishing and freeing.  It follows the reference's engine loop
+(src/engine.cpp:295-355 admission, 392-580 iteration; src/scheduler.cpp:11-49 batch forming):
+
+  * submit refuses what can never run: an empty prompt, ids outside the vocabulary,
+    max_tokens < 1, prompt + max_tokens beyond max_model_len or beyond the whole pool;
+  * admission is first-come within aged priority; a request is admitted when a slot is free
+    and pages for its WHOLE life, ceil((prompt + max_tokens) / page_size), can be set aside.
+    Because everything is set aside up front, pages cannot run out in the middle of a
+    request: a request that does not fit waits until others finish and free theirs;
+    after `admission_reserve_ms` of waiting the oldest request may no longer be overtaken;
+  * each iteration gives every decoding request one token and fills the rest of the token
+    budget with portions of prompts (policy mixed), or runs prompts first (prefill_first);
+    the batch-forming decision itself is native (csrc/host/scheduler.cpp);
+  * the last token of a prompt and every decoded token ask for logits; a request ends on an
+    end-of-sequence id (unless ignore_eos) or at max_tokens, and its pages and slot are
+    given back at once.
+"""
+from __future__ import annotations
+
+import ctypes
+import time
+from dataclasses import dataclass, field
+from typing import List, Optional
+
+from ..kernels import build
+from ..sampling import RequestRng, Sampler
+from .step import Entry, Runner
+
+
+class _Item(ctypes.Structure):
+    _fields_ = [("key", ctypes.c_int64), ("prefill_remaining", ctypes.c_int64), ("priority", ctypes.c_int32),
+                ("wait_ms", ctypes.c_int64), ("order", ctypes.c_uint64)]
+
+
+class _Slice(ctypes.Structure):
+    _fields_ = [("key", ctypes.c_int64), ("tokens", ctypes.c_int64), ("prefill", ctypes.c_int32)]
+
+
+POLICIES = {"mixed": 0, "prefill_first": 1}
+
+
+def _lib():
+    lib = build.load("host")
+    if not getattr(lib, "_mlr_sched_typed", False):
+        lib.mlr_schedule_batch.argtypes = [ctypes.POINTER(_Item), ctypes.c_int, ctypes.c_int64, ctypes.c_int64,
+                                           ctypes.c_int, ctypes.c_int, ctypes.POINTER(_Slice)]
+        lib.mlr_effective_priority.argtypes = [ctypes.c_int, ctypes.c_int64, ctypes.c_int]
+        lib.mlr_effective_priority.restype = ctypes.c_int64
+        lib._mlr_sched_typed = True
+    return lib
+
+
+def effective_priority(priority, wait_ms, aging_ms):
+    return _lib().mlr_effective_priority(priority, int(wait_ms), aging_ms)
+
+
+def schedule_batch(items, batch_tokens, prefill_chunk, policy="mixed", aging_ms=250):
+    """items: (key, prefill_remaining, priority, wait_ms, order) each.  Returns the slices
+    [(key, tokens, is_prefill)] of the next batch."""
+    if policy not in POLICIES:
+        raise ValueError(f"policy must be one of {sorted(POLICIES)}")
+    n = len(items)
+    arr = (_Item * max(n, 1))()
+    for i, (key, remaining, priority, wait_ms, order) in enumerate(items):
+        arr[i] = _Item(key, remaining, priority, int(wait_ms), order)
+    out = (_Slice * max(n, 1))()
+    count = _lib().mlr_schedule_batch(arr, n, batch_tokens, prefill_chunk, POLICIES[policy], aging_ms, out)
+    if count < 0:
+        raise ValueError("batch_tokens, prefill_chunk and aging_ms must be positive")
+    return [(out[i].key, out[i].tokens, bool(out[i].prefill)) for i in range(count)]
+
+
+@dataclass
+class EngineOptions:
+    """Names and defaults after the reference's EngineConfig (include/llmserve/config.h:15-33)."""
+    context_tokens: int = 8192        # tokens the page pool holds
+    max_model_len: int = 2048         # longest prompt + output of one request
+    max_active: int = 8               # request slots
+    batch_tokens: int = 256           # token budget of one step
+    prefill_chunk: int = 128          # longest portion of one prompt in a step
+    block_size: int = 16              # tokens in a page
+    aging_ms: int = 250
+    admission_reserve_ms: int = 2000
+    policy: str = "mixed"
+    queue_capacity: int = 65536
+
+    def validate(self):
+        """src/config.cpp:8-36."""
+        if self.block_size <= 0 or self.context_tokens <= 0 or self.context_tokens % self.block_size != 0:
+            raise ValueError("context_tokens must be a positive multiple of block_size")
+        if self.max_model_len < 2 or self.max_model_len > self.context_tokens:
+            raise ValueError("max_model_len must be in [2, context_tokens]")
+        if self.max_active <= 0 or self.batch_tokens < self.max_active or self.batch_tokens > self.context_tokens:
+            raise ValueError("require 1 <= max_active <= batch_tokens <= context_tokens")
+        if self.prefill_chunk <= 0 or self.prefill_chunk > self.batch_tokens or self.queue_capacity <= 0:
+            raise ValueError("invalid prefill or queue limit")
+        if self.aging_ms <= 0 or self.admission_reserve_ms <= 0:
+            raise ValueError("invalid aging interval")
+        if self.policy not in POLICIES:
+            raise ValueError(f"policy must be one of {sorted(POLICIES)}")
+
+
+@dataclass
+class Request:
+    id: int
+    prompt: List[int]
+    max_tokens: int
+    temperature: float = 0.0
+    seed: int = 0
+    ignore_eos: bool = False
+    priority: int = 0
+    # state
+    order: int = 0
+    created: float = 0.0
+    last_scheduled: float = 0.0
+    slot: Optional[int] = None
+    pages: int = 0                    # pages set aside for its whole life
+    processed: int = 0                # prompt tokens already run
+    generated: List[int] = field(default_factory=list)
+    rng: Optional[RequestRng] = None
+    finish_reason: Optional[str] = None
+
+
+class Engine:
+    """Continuous batching over one `Runner`.  Single-threaded: the caller drives `step()`."""
+
+    def __init__(self, model, options: EngineOptions = None, clock=time.monotonic, runner=None, sampler=None):
+        self.options = options or EngineOptions()
+        self.options.validate()
+        o = self.options
+        self.model = model
+        self.runner = runner or Runner(model, max_tokens=o.context_tokens, max_slots=o.max_active,
+                                       max_length=min(o.max_model_len, model.spec.max_positions),
+                                       max_batch_tokens=o.batch_tokens, page_size=o.block_size)
+        self.sampler = sampler or Sampler(self.runner.kernels, self.runner.device, max_rows=o.max_active)
+        self.clock = clock
+        self.total_pages = o.context_tokens // o.block_size
+        self.free_credits = self.total_pages
+        self.waiting: List[Request] = []
+        self.active: List[Request] = []
+        self.finished = {}
+        self._next_id = 0
+        self._order = 0
+        self.failed = False
+        self.stats = dict(batches=0, mixed_batches=0, prefill_tokens=0, decode_tokens=0, generated_tokens=0,
+                          max_batch_tokens=0, max_batch_sequences=0, admission_waits=0)
+
+    # -- submit ----------------------------------------------------------------------------------
+    def submit(self, prompt, max_tokens=64, temperature=0.0, seed=None, ignore_eos=False, priority=0):
+        o = self.options
+        if self.failed:
+            raise RuntimeError("the engine stopped after a failed step")
+        prompt = [int(t) for t in prompt]
+        vocab = self.model.spec.vocab_size
+        if not prompt:
+            raise ValueError("empty prompt")
+        if any(t < 0 or t >= vocab for t in prompt):
+            raise ValueError("prompt holds a token id outside the vocabulary")
+        if max_tokens < 1:
+            raise ValueError("max_tokens must be at least 1")
+        if len(prompt) + max_tokens > min(o.max_model_len, self.model.spec.max_positions):
+            raise ValueError("prompt + max_tokens exceed max_model_len")
+        if self._pages_for(len(prompt) + max_tokens) > self.total_pages:
+            raise ValueError("the request does not fit an otherwise idle page pool")
+        if not 0 <= priority <= 3:
+            raise ValueError("priority must be in 0..3")
+        if temperature < 0:
+            raise ValueError("temperature must not be negative")
+        if len(self.waiting) >= o.queue_capacity:
+            raise RuntimeError("the waiting queue is full")
+        now = self.clock()
+        rid = self._next_id
+        self._next_id += 1
+        req = Request(rid, prompt, max_tokens, float(temperature), rid if seed is None else int(seed),
+                      bool(ignore_eos), priority, order=self._order, created=now, last_scheduled=now)
+        req.rng = RequestRng(req.seed)
+        self._order += 1
+        self.waiting.append(req)
+        return rid
+
+    def _pages_for(self, tokens):
+        return (tokens + self.options.block_size - 1) // self.options.block_size
+
+    # -- admission -------------------------------------------------------------------------------
+    def _admit(self, req):
+        pages = self._pages_for(len(req.prompt) + req.max_tokens)
+        if pages > self.free_credits or self.runner.free_slots() == 0:
+            return False
+        req.slot = self.runner.open_request()
+        req.pages = pages
+        self.free_credits -= pages
+        self.active.append(req)
+        return True
+
+    def _admit_waiting(self):
+        o = self.options
+        now = self.clock()
+        ms = lambda t: int((now - t) * 1000)
+        self.waiting.sort(key=lambda r: (-effective_priority(r.priority, ms(r.created), o.aging_ms), r.order))
+        i = 0
+        while i < len(self.waiting) and self.runner.free_slots() > 0:
+            req = self.waiting[i]
+            if self._admit(req):
+                self.waiting.pop(i)
+            elif ms(req.created) >= o.admission_reserve_ms:
+                self.stats["admission_waits"] += 1
+                break
+            else:
+                self.stats["admission_waits"] += 1
+                i += 1
+
+    def _finish(self, req, reason):
+        req.finish_reason = reason
+        self.runner.close_request(req.slot)
+        self.free_credits += req.pages
+        req.slot, req.pages = None, 0
+        self.active.remove(req)
+        self.finished[req.id] = req
+
+    # -- one iteration ---------------------------------------------------------------------------
+    def step(self):
+        """Admit, form one batch, run it, sample, finish.  Returns the events of this iteration:
+        [(request id, token, finish reason or None)]."""
+        if self.failed:
+            raise RuntimeError("the engine stopped after a failed step")
+        o = self.options
+        self._admit_waiting()
+        if not self.active:
+            if self.waiting:
+                raise RuntimeError("no request fits an otherwise idle KV pool")
+            return []
+        now = self.clock()
+        items = [(i, len(r.prompt) - r.processed, r.priority, int((now - r.last_scheduled) * 1000), r.order)
+                 for i, r in enumerate(self.active)]
+        slices = schedule_batch(items, o.batch_tokens, o.prefill_chunk, o.policy, o.aging_ms)
+        if not slices:
+            raise RuntimeError("scheduler made no progress")
+        entries, sampled = [], []
+        prefill_tokens = decode_tokens = 0
+        for key, count, is_prefill in slices:
+            req = self.active[key]
+            if is_prefill:
+                tokens = req.prompt[req.processed:req.processed + count]
+                last = req.processed + count == len(req.prompt)
+                entries.append(Entry(req.slot, tokens, [count - 1] if last else []))
+                if last:
+                    sampled.append(req)
+                prefill_tokens += count
+            else:
+                entries.append(Entry(req.slot, [req.generated[-1]], [0]))
+                sampled.append(req)
+                decode_tokens += 1
+        try:
+            logits = self.runner.step(entries)
+            tokens = []
+            if sampled:
+                tokens = self.sampler.sample(logits, [r.temperature for r in sampled],
+                                             [r.rng.uniform() if r.temperature > 0 else 0.0 for r in sampled])
+            vocab = self.model.spec.vocab_size
+            if len(tokens) != len(sampled) or any(t < 0 or t >= vocab for t in tokens):
+                raise RuntimeError("the step returned an invalid sample")
+        except Exception:
+            self.failed = True            # nothing of this batch is published
+            raise
+        s = self.stats
+        s["batches"] += 1
+        s["mixed_batches"] += int(prefill_tokens > 0 and decode_tokens > 0)
+        s["prefill_tokens"] += prefill_tokens
+        s["decode_tokens"] += decode_tokens
+        s["max_batch_tokens"] = max(s["max_batch_tokens"], prefill_tokens + decode_tokens)
+        s["max_batch_sequences"] = max(s["max_batch_sequences"], len(slices))
+        done_at = self.clock()
+        for key, count, is_prefill in slices:
+            req = self.active[key]
+            req.last_scheduled = done_at
+            if is_prefill:
+                req.processed += count
+        events = []
+        eos = set(self.model.spec.eos_token_ids)
+        for req, token in zip(sampled, tokens):
+            req.generated.append(token)
+            s["generated_tokens"] += 1
+            reason = None
+            if token in eos and not req.ignore_eos:
+                reason = "stop"
+            elif len(req.generated) >= req.max_tokens:
+                reason = "length"
+            events.append((req.id, token, reason))
+        for rid, _, reason in events:
+            if reason is not None:
+                self._finish(next(r for r in self.active if r.id == rid), reason)
+        return events
+
+    def has_work(self):
+        return bool(self.waiting or self.active)
+
+    def run_until_done(self):
+        """Drive steps until nothing waits or runs; {request id: generated tokens}."""
+        while self.has_work():
+            self.step()
+        return {rid: list(r.generated) for rid, r in self.finished.items()}

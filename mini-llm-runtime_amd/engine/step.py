@@ -58,6 +58,9 @@ class Runner:
     def length(self, slot):
         return self.cache.length(slot)
 
+    def free_slots(self):
+        return self.cache.book.free_slots()
+
     # -- the step ------------------------------------------------------------------------------
     def _validate(self, entries):
         if self.poisoned:

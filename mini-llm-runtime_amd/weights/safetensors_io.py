@@ -9,6 +9,7 @@ import json
 import mmap
 import os
 import struct
+import warnings
 
 import torch
 
@@ -74,7 +75,14 @@ class SafetensorsFile:
         begin, count = self._ranges[name]
         if count == 0:
             return torch.empty(shape, dtype=dtype)
-        flat = torch.frombuffer(self._map, dtype=dtype, count=count, offset=self._data_start + begin)
+        start = self._data_start + begin
+        width = _DTYPES[_NAMES[dtype]][1]
+        if start % width == 0:
+            with warnings.catch_warnings():
+                warnings.simplefilter("ignore", UserWarning)      # the mapping is read-only; nobody writes
+                flat = torch.frombuffer(self._map, dtype=dtype, count=count, offset=start)
+        else:                                                     # misaligned in the file: copy out
+            flat = torch.frombuffer(bytearray(self._map[start:start + count * width]), dtype=dtype, count=count)
         return flat.view(shape)
 
     def close(self):
@@ -87,22 +95,23 @@ class SafetensorsFile:
 
 
 def write_safetensors(path, tensors, metadata=None):
-    """Write {name: CPU tensor} in sorted name order, each tensor's bytes aligned to 8."""
+    """Write {name: CPU tensor}: widest element types first, then by name, bytes back to back
+    (every tensor then starts at a multiple of its element size)."""
     header = {}
     if metadata:
         header["__metadata__"] = {str(k): str(v) for k, v in metadata.items()}
     offset = 0
     blobs = []
-    for name in sorted(tensors):
-        t = tensors[name].detach().contiguous().cpu()
+    for t in tensors.values():
         if t.dtype not in _NAMES:
             raise SafetensorsError(f"cannot write dtype {t.dtype}")
+    for name in sorted(tensors, key=lambda n: (-tensors[n].element_size(), n)):
+        t = tensors[name].detach().contiguous().cpu()
         raw = t.view(torch.uint8).numpy().tobytes() if t.numel() else b""
-        pad = (-len(raw)) % 8
         header[name] = {"dtype": _NAMES[t.dtype], "shape": list(t.shape),
                         "data_offsets": [offset, offset + len(raw)]}
-        blobs.append(raw + b"\0" * pad)
-        offset += len(raw) + pad
+        blobs.append(raw)
+        offset += len(raw)
     text = json.dumps(header, separators=(",", ":")).encode("utf-8")
     text += b" " * ((-len(text)) % 8)
     with open(path, "wb") as f:

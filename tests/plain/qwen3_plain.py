@@ -69,11 +69,10 @@ def causal_attention(q, k, v, positions, scale, window=None):
     return out
 
 
-def attention_block(x, w, cfg, positions, window=None):
+def project_qkv(x, w, cfg, positions):
     """q = n Wq^T, k = n Wk^T, v = n Wv^T (no bias); per head RMSNorm over D with q_norm /
-    k_norm and the layer's eps, BEFORE the rotation; v is neither normed nor rotated; then
-    attention and the output projection.  x is the already normed input [T, E].
-    src/minillm/runtime.cpp:250-319."""
+    k_norm and the layer's eps, BEFORE the rotation; v is neither normed nor rotated.
+    Returns q [T, Hq, D], k and v [T, Hkv, D].  src/minillm/runtime.cpp:250-277."""
     T = x.shape[0]
     Hq, Hkv, D = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
     q = (x @ w["q_proj"].T).reshape(T, Hq, D)
@@ -82,10 +81,16 @@ def attention_block(x, w, cfg, positions, window=None):
     q = rms_norm(q, w["q_norm"], cfg["rms_norm_eps"])
     k = rms_norm(k, w["k_norm"], cfg["rms_norm_eps"])
     cos, sin = rope_cos_sin(positions, D, cfg["rope_theta"])
-    q = rope_rotate(q, cos, sin)
-    k = rope_rotate(k, cos, sin)
-    o = causal_attention(q, k, v, positions, 1.0 / np.sqrt(D), window)
-    return o.reshape(T, Hq * D) @ w["o_proj"].T
+    return rope_rotate(q, cos, sin), rope_rotate(k, cos, sin), v
+
+
+def attention_block(x, w, cfg, positions, window=None):
+    """The mixer of a layer on its already normed input x [T, E]: projections, attention with
+    scale 1/sqrt(D), output projection.  src/minillm/runtime.cpp:250-319."""
+    T = x.shape[0]
+    q, k, v = project_qkv(x, w, cfg, positions)
+    o = causal_attention(q, k, v, positions, 1.0 / np.sqrt(cfg["head_dim"]), window)
+    return o.reshape(T, -1) @ w["o_proj"].T
 
 
 def swiglu_mlp(x, w):

@@ -1,0 +1,156 @@
+"""The engine against the plain implementation, in 32-bit and in bfloat16, for every way of cutting
+the same requests into steps: whole; most in one step and the last 32 tokens one by one; portions
+of changing size down to two tokens; mixed, up to four live requests with so few pages that freed
+pages are used again; long decoding; the first tokens of a sequence.  (The reference's counterpart:
+240 teacher-forcing cases over chunk sizes and sequence counts, tests/cuda_validation_support.h:53-70.)
+"""
+import numpy as np
+import pytest
+import torch
+
+from conftest import PAGE_SIZE, TINY
+from helpers import (compare, last_one_by_one, make_requests, max_difference, mixed, plain_logits, portions,
+                     run_steps, whole)
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+LENGTHS = [70, 33, 100, 17, 64, 129, 2, 45]
+_models = {}
+
+
+def load(model_folders, name, dtype_name):
+    from mini_llm_runtime_amd.parts import DecoderModel
+    key = (name, dtype_name)
+    if key not in _models:
+        _models[key] = DecoderModel.load(model_folders[name], DTYPES[dtype_name])
+    return _models[key]
+
+
+def runner_for(model, name, max_tokens, **kwargs):
+    from mini_llm_runtime_amd.engine import Runner
+    return Runner(model, max_tokens=max_tokens, max_slots=4, page_size=PAGE_SIZE[name], **kwargs)
+
+
+@pytest.fixture(scope="module")
+def expected(plain_models):
+    out = {}
+    for name in TINY:
+        reqs = make_requests(TINY[name]["vocab_size"], LENGTHS, seed=11)
+        out[name] = (reqs, plain_logits(plain_models[name], reqs))
+    return out
+
+
+@pytest.mark.parametrize("dtype_name", DTYPES)
+@pytest.mark.parametrize("name", TINY)
+def test_every_way_of_cutting_gives_the_plain_logits(model_folders, expected, name, dtype_name):
+    reqs, want = expected[name]
+    model = load(model_folders, name, dtype_name)
+    results = {}
+    r = runner_for(model, name, max_tokens=192)          # one request at a time: 129 tokens -> 192
+    for mode, steps in [("whole", whole(reqs)), ("last32", last_one_by_one(reqs)), ("portions", portions(reqs))]:
+        results[mode] = run_steps(r, steps)
+        compare(results[mode], want, dtype_name)
+        r.cache.check()
+        assert r.cache.free_pages() == r.cache.num_pages
+    steps, peak = mixed(reqs, seed=5)
+    assert max(len(s["entries"]) for s in steps) == 4
+    # some step holds a portion of a prompt beside a single (decoded) token of another request
+    assert any(min(len(e["tokens"]) for e in s["entries"]) == 1 and max(len(e["tokens"]) for e in s["entries"]) > 1
+               for s in steps)
+    total = sum(-(-n // 64) * 64 for n in LENGTHS)
+    assert peak < total                                   # the pool is smaller than all requests together
+    r = runner_for(model, name, max_tokens=peak)
+    results["mixed"] = run_steps(r, steps)
+    compare(results["mixed"], want, dtype_name)
+    r.cache.check()
+    assert r.cache.free_pages() == r.cache.num_pages
+    # the same position, however it was cut and batched, agrees far inside the tolerance
+    limit = 2e-5 if dtype_name == "float32" else 0.05
+    for mode in ("last32", "portions", "mixed"):
+        assert max_difference(results["whole"], results[mode]) <= limit, mode
+
+
+@pytest.mark.parametrize("dtype_name", DTYPES)
+@pytest.mark.parametrize("split_keys,split_max_tokens", [(64, 10 ** 6), (0, 0)])
+def test_key_splits_do_not_change_the_result(model_folders, expected, dtype_name, split_keys, split_max_tokens):
+    """Attention over key ranges split across workgroups (forced on for every batch, and off)."""
+    reqs, want = expected["B"]
+    model = load(model_folders, "B", dtype_name)
+    r = runner_for(model, "B", max_tokens=192, split_keys=split_keys, split_max_tokens=split_max_tokens)
+    compare(run_steps(r, last_one_by_one(reqs)), want, dtype_name)
+
+
+@pytest.mark.parametrize("dtype_name", DTYPES)
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_long_decoding(model_folders, plain_models, name, dtype_name):
+    """A five-token prompt, then 600 tokens one by one (teacher-forced): crosses many pages and key tiles."""
+    toks = make_requests(TINY[name]["vocab_size"], [605], seed=3)["r0"]
+    want = plain_logits(plain_models[name], {"r0": toks})
+    model = load(model_folders, name, dtype_name)
+    r = runner_for(model, name, max_tokens=640)
+    steps = [dict(step=0, entries=[dict(id="r0", tokens=toks[:5], want=[0, 1, 2, 3, 4])], end=[])]
+    steps += [dict(step=i, entries=[dict(id="r0", tokens=[toks[i]], want=[0])], end=[]) for i in range(5, 605)]
+    steps[-1]["end"] = ["r0"]
+    compare(run_steps(r, steps), want, dtype_name)
+
+
+@pytest.mark.parametrize("dtype_name", DTYPES)
+@pytest.mark.parametrize("name", TINY)
+def test_first_tokens_of_a_sequence(model_folders, plain_models, name, dtype_name):
+    """Positions 0 and 1: a key set of one; four single-token prompts in one batch, then their second tokens."""
+    vocab = TINY[name]["vocab_size"]
+    reqs = {f"r{i}": [(17 * i + 3) % vocab, (5 * i + 1) % vocab] for i in range(4)}
+    want = plain_logits(plain_models[name], reqs)
+    model = load(model_folders, name, dtype_name)
+    r = runner_for(model, name, max_tokens=256)
+    steps = [dict(step=0, entries=[dict(id=rid, tokens=t[:1], want=[0]) for rid, t in reqs.items()], end=[]),
+             dict(step=1, entries=[dict(id=rid, tokens=t[1:], want=[0]) for rid, t in reqs.items()], end=list(reqs))]
+    compare(run_steps(r, steps), want, dtype_name)
+
+
+def test_refused_batches_change_nothing(model_folders, plain_models):
+    """The reference's list of invalid batches (tests/cuda_layer_tests.cpp:88-95) and an overcommitted pool:
+    each is refused before anything is written, and the request goes on as if nothing had happened."""
+    from mini_llm_runtime_amd.cache import CacheError, CacheFull
+    from mini_llm_runtime_amd.engine import Entry, Runner, StepError
+    model = load(model_folders, "A", "float32")
+    r = Runner(model, max_tokens=64, max_slots=2, max_length=48, max_batch_tokens=40, page_size=16)
+    toks = make_requests(256, [40], seed=9)["r0"]
+    want = plain_models["A"].logits(toks)
+    s = r.open_request()
+    r.step([Entry(s, toks[:20], [])])                    # nothing wanted: the cache is written all the same
+    other = r.open_request()
+    bad = [[], [Entry(s, [], [])], [Entry(s, [256], [0])], [Entry(s, [-1], [0])], [Entry(s, [1, 2], [2])],
+           [Entry(s, [1], [-1])], [Entry(7, [1], [0])], [Entry(s, [1], [0]), Entry(s, [2], [0])],
+           [Entry(s, [1] * 41, [])], [Entry(s, [1] * 29, [])],            # beyond the step's limit; beyond max_length
+           [Entry(s, [1] * 10, []), Entry(other, [1] * 40, [])]]          # `other` needs 3 pages, 2 are free
+    for batch in bad:
+        with pytest.raises((StepError, CacheError, CacheFull)):
+            r.step(batch)
+        assert r.length(s) == 20 and r.length(other) == 0 and not r.poisoned
+        r.cache.check()
+    got = r.step([Entry(s, toks[20:], list(range(20)))]).double().cpu().numpy()
+    np.testing.assert_allclose(got, want[20:], atol=2e-4, rtol=2e-4)
+    # a slot used again after its request ended behaves like a fresh one
+    r.close_request(s)
+    s2 = r.open_request()
+    again = r.step([Entry(s2, toks, list(range(40)))]).double().cpu().numpy()
+    np.testing.assert_allclose(again, want, atol=2e-4, rtol=2e-4)
+
+
+def test_steady_steps_allocate_nothing(model_folders):
+    """After the first steps have sized the scratch memory, a step allocates no device memory (the
+    reference asserts the same of its hot path, tests/cuda_runtime_tests.cpp:81-84)."""
+    from mini_llm_runtime_amd.engine import Entry
+    model = load(model_folders, "B", "bfloat16")
+    r = runner_for(model, "B", max_tokens=256)
+    s = r.open_request()
+    r.step([Entry(s, list(range(40)), [39])])
+    r.step([Entry(s, [1], [0])])
+    torch.cuda.synchronize()
+    before = torch.cuda.memory_stats()["allocation.all.allocated"]
+    for t in range(30):
+        r.step([Entry(s, [t], [0])])
+    torch.cuda.synchronize()
+    assert torch.cuda.memory_stats()["allocation.all.allocated"] == before

@@ -1,0 +1,137 @@
+"""Generation through the entry points: the Python API over the scheduler, and the command line.
+Greedy generation must give the plain implementation's tokens; temperature sampling must give, for a
+request, the same tokens whatever else runs beside it."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+from conftest import PAGE_SIZE, ROOT, TINY
+from helpers import make_requests
+
+pytestmark = pytest.mark.gpu
+
+
+def prompts_for(name, lengths=(7, 13, 5, 1, 30)):
+    return list(make_requests(TINY[name]["vocab_size"], lengths, seed=31).values())
+
+
+def check_greedy(plain, prompt, got, dtype):
+    """Token by token; in bfloat16 a step may differ only where the plain top two are nearly tied, and the
+    comparison stops there (the continuations differ legitimately)."""
+    tokens = list(prompt)
+    for i, t in enumerate(got):
+        row = plain.logits(tokens, [len(tokens) - 1])[0]
+        best = int(np.argmax(row))
+        if t != best:
+            top = np.sort(row)[-2:]
+            assert dtype == "bfloat16" and top[1] - top[0] < 0.05 * np.abs(row).max(), (i, t, best)
+            return
+        tokens.append(t)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_greedy_generation_through_the_python_entry_point(model_folders, plain_models, name, dtype):
+    from mini_llm_runtime_amd.api import LLM
+    llm = LLM(model_folders[name], dtype=dtype, context_tokens=256, max_model_len=128, max_active=4,
+              batch_tokens=16, prefill_chunk=8, block_size=PAGE_SIZE[name])
+    prompts = prompts_for(name)
+    outs = llm.generate(prompts, max_tokens=8)
+    assert [len(o) for o in outs] == [8] * len(prompts)
+    for prompt, out in zip(prompts, outs):
+        check_greedy(plain_models[name], prompt, out, dtype)
+    assert llm.engine.stats["mixed_batches"] > 0                   # prompts ran in portions beside decoding requests
+    assert llm.engine.runner.cache.free_pages() == llm.engine.total_pages
+    one = llm.generate(prompts[0], max_tokens=8)                    # one prompt in, one list out
+    if dtype == "float32":
+        assert one == outs[0] == plain_models[name].greedy(prompts[0], 8)
+
+
+def test_temperature_sampling_is_per_request(model_folders, plain_models):
+    """Same seed, same tokens, alone or beside others; each token is the inverse-CDF draw of the plain
+    distribution at the request's own uniform number."""
+    from mini_llm_runtime_amd.api import LLM
+    from mini_llm_runtime_amd.sampling import RequestRng
+    from plain.qwen3_plain import temperature_cdf
+    llm = LLM(model_folders["B"], dtype="float32", context_tokens=512, max_model_len=128, max_active=4,
+              batch_tokens=32, prefill_chunk=16, block_size=8)
+    prompts = prompts_for("B", (1, 9, 17, 30))
+    together = llm.generate(prompts, max_tokens=6, temperature=0.8, seed=100)
+    for i, prompt in enumerate(prompts):
+        alone = llm.generate(prompt, max_tokens=6, temperature=0.8, seed=100 + i)
+        assert alone == together[i]
+        rng = RequestRng(100 + i)
+        tokens = list(prompt)
+        for t in together[i]:
+            u = rng.uniform()
+            cdf = temperature_cdf(plain_models["B"].logits(tokens, [len(tokens) - 1])[0], 0.8)
+            lo = cdf[t - 1] if t > 0 else 0.0
+            assert lo - 1e-4 <= u <= cdf[t] + 1e-4
+            tokens.append(t)
+    assert llm.generate(prompts[1], max_tokens=6, temperature=0.8, seed=5) != \
+        llm.generate(prompts[1], max_tokens=6, temperature=0.8, seed=6)
+
+
+def test_end_of_sequence_stops_generation(model_folders, plain_models):
+    """Configuration C names token 5 as end of sequence: generation stops there unless told to go on."""
+    from mini_llm_runtime_amd.api import LLM
+    plain = plain_models["C"]
+    llm = LLM(model_folders["C"], dtype="float32", context_tokens=512, max_model_len=256, max_active=2,
+              batch_tokens=64, prefill_chunk=64, block_size=32)
+    # find a prompt whose greedy continuation reaches token 5 early
+    vocab = TINY["C"]["vocab_size"]
+    found = None
+    for first in range(vocab):
+        out = plain.greedy([first], 4)
+        if 5 in out[:3]:
+            found = ([first], out)
+            break
+    if found is None:
+        pytest.skip("no short greedy path to the end-of-sequence id with these weights")
+    prompt, out = found
+    stop = out.index(5)
+    assert llm.generate(prompt, max_tokens=4) == out[:stop + 1]
+    assert llm.generate(prompt, max_tokens=4, ignore_eos=True) == out
+
+
+def run_cli(args):
+    return subprocess.run([sys.executable, os.path.join(ROOT, "bin", "mini-llm")] + args, capture_output=True,
+                          text=True, timeout=300)
+
+
+def test_command_line(model_folders, plain_models, tmp_path):
+    prompt = prompts_for("A")[1]
+    ids = ",".join(str(t) for t in prompt)
+    report_path = str(tmp_path / "report.json")
+    done = run_cli(["--model", model_folders["A"], "--prompt-ids", ids, "--tokens", "6", "--dtype", "float32",
+                    "--chunk", "4", "--context", "64", "--sequences", "1", "--output", report_path, "--device-time"])
+    assert done.returncode == 0, done.stderr
+    report = json.loads(done.stdout)
+    assert report == json.load(open(report_path))
+    assert report["token_ids"] == plain_models["A"].greedy(prompt, 6)
+    assert report["prompt_tokens"] == 13 and report["completion_tokens"] == 6
+    phases = [f["phase"] for f in report["forwards"]]
+    assert phases == ["prefill"] * 4 + ["decode"] * 5               # 13 tokens in portions of 4; the last token is not fed back
+    assert [f["input_tokens"] for f in report["forwards"][:4]] == [4, 4, 4, 1]
+    assert report["used_kv_pages_before_release"] == 2 and report["used_kv_pages_after_release"] == 0
+    assert report["forwards"][0]["device_elapsed_ms"] > 0
+    # random-weights mode from a configuration file, seeded
+    cfg_path = str(tmp_path / "cfg.json")
+    json.dump(TINY["B"], open(cfg_path, "w"))
+    a = run_cli(["--random-weights", cfg_path, "--seed", "3", "--prompt-ids", "1,2,3", "--tokens", "5"])
+    b = run_cli(["--random-weights", cfg_path, "--seed", "3", "--prompt-ids", "1,2,3", "--tokens", "5"])
+    assert a.returncode == 0 and json.loads(a.stdout)["token_ids"] == json.loads(b.stdout)["token_ids"]
+    # errors: one line on stderr, exit code 1
+    for args, text in [(["--model", model_folders["A"], "--prompt-ids", ids, "--output", report_path], "new file"),
+                       (["--model", model_folders["A"], "--prompt-ids", "1,2", "--tokens", "0"], "out-of-range"),
+                       (["--model", model_folders["A"], "--prompt-ids", "999"], "vocabulary"),
+                       (["--model", model_folders["A"], "--prompt-ids", ids, "--context", "15", "--tokens", "4"], "exceed"),
+                       (["--model", model_folders["A"], "--bogus"], "unknown option"),
+                       (["--model", str(tmp_path), "--prompt-ids", "1"], "config.json")]:
+        bad = run_cli(args)
+        assert bad.returncode == 1 and text in bad.stderr, (args, bad.stderr)
+    assert run_cli(["--help"]).returncode == 0 and run_cli([]).returncode == 1

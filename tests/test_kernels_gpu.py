@@ -381,3 +381,35 @@ def test_sample_frequencies():
     freq = torch.bincount(tokens.cpu().long(), minlength=7).double() / rows
     want = torch.softmax(logits.double() / temp_value, 0)
     assert (freq - want).abs().max() < 0.015
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("window", [1, 16, 17, 64, 100])
+def test_attention_window_edge(dtype, window):
+    """The key just outside the window matches the query strongly and must not be seen; then the key
+    just inside does and must be seen."""
+    k = kernels(dtype)
+    d, page, L = 32, 16, 300
+    g = torch.Generator().manual_seed(31)
+    q = torch.randn((1, d), generator=g)
+    for inside in (False, True):
+        kk = 0.05 * torch.randn((L, d), generator=g)
+        vv = torch.randn((L, d), generator=g)
+        hot = L - window + (0 if inside else -1)
+        kk[hot] = 40 * q[0] / q[0].norm()
+        n_blocks = (L + page - 1) // page
+        table = torch.arange(n_blocks, dtype=torch.int32)[None, :].contiguous()
+        k_pages = torch.zeros((n_blocks, 1, page, d))
+        v_pages = torch.zeros((n_blocks, 1, page, d))
+        k_pages.view(-1, d)[:L] = kk
+        v_pages.view(-1, d)[:L] = vv
+        out = torch.empty((1, d), dtype=dtype, device="cuda")
+        k.paged_attention(q.to(dtype).cuda(), k_pages.to(dtype).cuda(), v_pages.to(dtype).cuda(), table.cuda(),
+                          torch.zeros(1, dtype=torch.int32).cuda(), torch.tensor([L - 1], dtype=torch.int32).cuda(),
+                          out, 1, 1, d, page, 1.0, window=window)
+        lo = L - window
+        want = plain_attention(q.to(dtype).double(), kk[:, None, :].to(dtype).double(), vv[:, None, :].to(dtype).double(),
+                               1.0, window)
+        torch.testing.assert_close(out.double().cpu(), want, **tol(dtype))
+        close_to_hot = (out.float().cpu()[0] - vv[hot].to(dtype).float()).abs().max() < 0.05
+        assert bool(close_to_hot) == inside, (window, inside, lo)

@@ -1,0 +1,279 @@
+"""The scheduler's decisions without a GPU.  The batch-forming vectors are the reference's own
+(tests/core_tests.cpp:123-146).  The engine runs against a fake step function whose "logits" are
+a hash of the request's token history, so any wrong position, order or mixing of requests changes
+the output (the reference's FakeRunner idea, tests/core_tests.cpp:518-594)."""
+import pytest
+
+from mini_llm_runtime_amd.cache import CacheFull, PageBook
+from mini_llm_runtime_amd.engine import Engine, EngineOptions, effective_priority, schedule_batch
+from mini_llm_runtime_amd.options import OptionError, Options
+
+
+def test_mixed_budget_and_decode_protection():
+    plan = schedule_batch([(0, 0, 0, 0, 0), (1, 10, 3, 0, 1), (2, 10, 0, 0, 2)], batch_tokens=8, prefill_chunk=4)
+    assert plan == [(0, 1, False), (1, 4, True), (2, 3, True)]
+
+
+def test_prefill_first_and_aging():
+    plan = schedule_batch([(0, 0, 0, 0, 0), (1, 20, 3, 0, 1), (2, 20, 0, 2000, 2)], 8, 8, "prefill_first", 250)
+    assert plan == [(2, 8, True)]                       # priority 0 + 2000/250 beats 3; no decode beside a prefill
+    assert effective_priority(0, 2000, 250) == 8 and effective_priority(3, -5, 250) == 3
+
+
+def test_decodes_first_then_prompts_in_order():
+    items = [(0, 5, 0, 0, 3), (1, 0, 0, 0, 2), (2, 0, 0, 0, 1), (3, 100, 0, 0, 0)]
+    assert schedule_batch(items, 16, 8) == [(2, 1, False), (1, 1, False), (3, 8, True), (0, 5, True)]
+    assert schedule_batch(items, 2, 8) == [(2, 1, False), (1, 1, False)]           # budget spent on decodes
+    assert schedule_batch(items, 3, 8) == [(2, 1, False), (1, 1, False), (3, 1, True)]
+    assert schedule_batch([(7, 3, 0, 0, 0)], 100, 2) == [(7, 2, True)]
+    assert schedule_batch([], 4, 4) == []
+    with pytest.raises(ValueError):
+        schedule_batch(items, 0, 8)
+    with pytest.raises(ValueError):
+        schedule_batch(items, 8, 8, "fastest")
+
+
+def test_options_validation():
+    """src/config.cpp:8-36; tests/core_tests.cpp:148-158."""
+    EngineOptions().validate()
+    for change in [dict(max_active=0), dict(batch_tokens=4), dict(context_tokens=65), dict(max_model_len=1),
+                   dict(prefill_chunk=0), dict(prefill_chunk=1000), dict(aging_ms=0), dict(policy="x"),
+                   dict(max_model_len=10000)]:
+        with pytest.raises(ValueError):
+            EngineOptions(**change).validate()
+
+
+# ------------------------------------------------------------------------------- fake step function
+class FakeSpec:
+    vocab_size = 1000
+    max_positions = 4096
+    eos_token_ids = (999,)
+
+
+class FakeModel:
+    spec = FakeSpec()
+
+
+def next_token(history):
+    h = 1469598103934665603
+    for i, t in enumerate(history):
+        h = ((h ^ (t + 31 * i)) * 1099511628211) % (1 << 64)
+    return h % 998                                          # never the end-of-sequence id
+
+
+class FakeRunner:
+    """Keeps the page bookkeeping real (native PageBook) and the model fake."""
+
+    def __init__(self, options, eos_after=None):
+        self.book = PageBook(options.max_active, options.max_model_len)
+        self.book.add_group(options.block_size, options.context_tokens // options.block_size)
+        self.history = {}
+        self.batches = []
+        self.max_batch_tokens = options.batch_tokens
+        self.eos_after = eos_after or {}
+        self.kernels = self.device = None
+
+    def free_slots(self):
+        return self.book.free_slots()
+
+    def open_request(self):
+        s = self.book.acquire_slot()
+        self.history[s] = []
+        return s
+
+    def close_request(self, slot):
+        self.book.release_slot(slot)
+        del self.history[slot]
+
+    def step(self, entries):
+        assert sum(len(e.tokens) for e in entries) <= self.max_batch_tokens
+        self.book.commit([e.slot for e in entries], [len(e.tokens) for e in entries])
+        self.book.check()
+        self.batches.append([(e.slot, len(e.tokens), list(e.want)) for e in entries])
+        out = []
+        for e in entries:
+            for i, t in enumerate(e.tokens):
+                self.history[e.slot].append(t)
+                if i in e.want:
+                    hist = self.history[e.slot]
+                    out.append(999 if self.eos_after.get(tuple(hist[:2])) == len(hist) else next_token(hist))
+        return out
+
+
+class FakeSampler:
+    def sample(self, logits, temperatures, uniforms):
+        return list(logits)
+
+
+def serial(prompt, n):
+    hist, out = list(prompt), []
+    for _ in range(n):
+        out.append(next_token(hist))
+        hist.append(out[-1])
+    return out
+
+
+def engine(clock=None, eos_after=None, **changes):
+    opts = EngineOptions(**{**dict(context_tokens=256, max_model_len=128, max_active=4, batch_tokens=16,
+                                   prefill_chunk=8, block_size=16), **changes})
+    now = [0.0]
+    eng = Engine(FakeModel(), opts, clock=clock or (lambda: now[0]), runner=FakeRunner(opts, eos_after),
+                 sampler=FakeSampler())
+    return eng, now
+
+
+def test_batched_equals_serial():
+    eng, _ = engine()
+    prompts = [[1, 2, 3], list(range(10, 33)), [7], list(range(50, 59)), [4, 4, 4, 4], list(range(100, 140))]
+    ids = [eng.submit(p, max_tokens=5 + i) for i, p in enumerate(prompts)]
+    out = eng.run_until_done()
+    for i, (rid, p) in enumerate(zip(ids, prompts)):
+        assert out[rid] == serial(p, 5 + i)
+        assert eng.finished[rid].finish_reason == "length"
+    assert eng.stats["mixed_batches"] > 0 and eng.stats["max_batch_sequences"] > 1
+    assert eng.stats["max_batch_tokens"] <= 16
+    assert eng.free_credits == eng.total_pages and eng.runner.book.free_pages() == eng.total_pages
+    assert eng.runner.book.free_slots() == 4
+
+
+def test_prompt_portions_and_wanted_places():
+    eng, _ = engine(batch_tokens=8, prefill_chunk=5)
+    eng.submit(list(range(12)), max_tokens=3)
+    eng.run_until_done()
+    # 12 prompt tokens in portions of 5, 5, 2; logits only at the prompt's last token, then decode steps
+    assert eng.runner.batches == [[(0, 5, [])], [(0, 5, [])], [(0, 2, [1])], [(0, 1, [0])], [(0, 1, [0])]]
+
+
+def test_decode_runs_beside_a_long_prompt():
+    eng, _ = engine(batch_tokens=8, prefill_chunk=8)
+    a = eng.submit([1, 2], max_tokens=6)
+    eng.step()                                       # a: whole prompt, first token sampled
+    b = eng.submit(list(range(30)), max_tokens=2)
+    eng.step()
+    assert eng.runner.batches[-1] == [(0, 1, [0]), (1, 7, [])]      # the decode first, the rest of the budget to b
+    out = eng.run_until_done()
+    assert out[a] == serial([1, 2], 6) and out[b] == serial(list(range(30)), 2)
+
+
+def test_stops_on_end_of_sequence_unless_ignored():
+    eng, _ = engine(eos_after={(1, 2): 5})
+    a = eng.submit([1, 2, 3], max_tokens=10)
+    b = eng.submit([1, 2, 3], max_tokens=4, ignore_eos=True)
+    out = eng.run_until_done()
+    assert out[a][-1] == 999 and len(out[a]) == 3 and eng.finished[a].finish_reason == "stop"
+    assert len(out[b]) == 4 and out[b][2] == 999 and eng.finished[b].finish_reason == "length"
+
+
+def test_submit_refuses_what_can_never_run():
+    eng, _ = engine()
+    for kwargs in [dict(prompt=[]), dict(prompt=[1000]), dict(prompt=[-1]), dict(prompt=[1], max_tokens=0),
+                   dict(prompt=[1] * 100, max_tokens=29), dict(prompt=[1], priority=4), dict(prompt=[1], temperature=-1.0)]:
+        with pytest.raises(ValueError):
+            eng.submit(**kwargs)
+    small, _ = engine(context_tokens=64, max_model_len=64, batch_tokens=16)
+    small.submit([1] * 30, max_tokens=34)            # exactly the whole pool
+    big, _ = engine(context_tokens=64, max_model_len=64, batch_tokens=16)
+    with pytest.raises(ValueError):
+        big.submit([1] * 40, max_tokens=30)
+
+
+def test_when_pages_run_out_requests_wait():
+    """Every request sets aside the pages of its whole life at admission, so a running request can
+    never be short of pages; one that does not fit waits for others to finish."""
+    eng, _ = engine(context_tokens=64, max_model_len=64, max_active=4, batch_tokens=16)   # 4 pages
+    a = eng.submit([1] * 20, max_tokens=12)          # 2 pages
+    b = eng.submit([2] * 10, max_tokens=20)          # 2 pages
+    c = eng.submit([3] * 5, max_tokens=5)            # 1 page: has to wait
+    eng.step()
+    assert [r.id for r in eng.active] == [a, b] and [r.id for r in eng.waiting] == [c]
+    assert eng.free_credits == 0
+    live_when_c_started = None
+    while eng.has_work():
+        eng.step()
+        if live_when_c_started is None and any(r.id == c for r in eng.active):
+            live_when_c_started = {r.id for r in eng.active}
+        assert eng.runner.book.free_pages() >= eng.free_credits >= 0     # held pages never exceed what was set aside
+    assert live_when_c_started is not None and len(live_when_c_started) <= 2
+    out = {rid: r.generated for rid, r in eng.finished.items()}
+    assert out[a] == serial([1] * 20, 12) and out[b] == serial([2] * 10, 20) and out[c] == serial([3] * 5, 5)
+    assert eng.stats["admission_waits"] > 0 and eng.free_credits == 4
+
+
+def test_the_step_function_refuses_an_overcommitted_batch_untouched():
+    """Below the scheduler (as the trace tool drives it) a batch that needs more pages than are free
+    is refused before anything changes."""
+    opts = EngineOptions(context_tokens=32, max_model_len=32, max_active=2, batch_tokens=32, prefill_chunk=32)
+    r = FakeRunner(opts)
+    s0, s1 = r.open_request(), r.open_request()
+    from mini_llm_runtime_amd.engine import Entry
+    r.step([Entry(s0, [1] * 17, [])])
+    with pytest.raises(CacheFull):
+        r.step([Entry(s1, [1] * 5, [])])
+    assert r.book.length(s1) == 0 and r.book.free_pages() == 0
+    r.close_request(s0)
+    r.step([Entry(s1, [1] * 5, [])])
+
+
+def test_small_later_requests_overtake_until_the_reserve_time():
+    eng, now = engine(context_tokens=64, max_model_len=64, max_active=4, batch_tokens=16, admission_reserve_ms=2000)
+    a = eng.submit([1] * 30, max_tokens=18)          # 3 of 4 pages
+    eng.step()
+    big = eng.submit([2] * 20, max_tokens=20)        # 3 pages: waits
+    small = eng.submit([3] * 4, max_tokens=4)        # 1 page: may overtake
+    eng.step()
+    assert {r.id for r in eng.active} == {a, small}
+    eng.run_until_done()
+    # the same, but the big request has already waited the reserve time: nothing overtakes it
+    eng, now = engine(context_tokens=64, max_model_len=64, max_active=4, batch_tokens=16, admission_reserve_ms=2000)
+    a = eng.submit([1] * 30, max_tokens=18)
+    eng.step()
+    big = eng.submit([2] * 20, max_tokens=20)
+    now[0] = 2.5
+    small = eng.submit([3] * 4, max_tokens=4)
+    eng.step()
+    assert {r.id for r in eng.active} == {a}
+    out = eng.run_until_done()
+    assert out[big] == serial([2] * 20, 20) and out[small] == serial([3] * 4, 4)
+
+
+def test_priority_decides_who_is_admitted_first():
+    eng, _ = engine(max_active=1, batch_tokens=16)
+    low = eng.submit([1], max_tokens=2, priority=0)
+    high = eng.submit([2], max_tokens=2, priority=3)
+    eng.step()
+    assert [r.id for r in eng.active] == [high]
+    out = eng.run_until_done()
+    assert out[low] == serial([1], 2) and out[high] == serial([2], 2)
+
+
+def test_a_failed_step_stops_the_engine():
+    eng, _ = engine()
+    eng.submit([1, 2, 3], max_tokens=4)
+    eng.sampler.sample = lambda *a: [5000]           # outside the vocabulary
+    with pytest.raises(RuntimeError, match="invalid sample"):
+        eng.step()
+    with pytest.raises(RuntimeError, match="stopped"):
+        eng.step()
+    with pytest.raises(RuntimeError, match="stopped"):
+        eng.submit([1], max_tokens=1)
+
+
+# ------------------------------------------------------------------------------- command-line options
+def test_option_parser():
+    """apps/options.h:12-62: exact names, value or flag, duplicates and unknowns are errors."""
+    o = Options(["--model", "m", "--tokens", "8", "--ignore-eos", "--temperature", "0.5", "--prompt-ids", "1,2,3"],
+                {"--model", "--tokens", "--temperature", "--prompt-ids"}, {"--help", "--ignore-eos"})
+    assert o.get("--model") == "m" and o.has("--ignore-eos") and not o.has("--help")
+    assert o.integer("--tokens", 32, 1, 4096) == 8 and o.integer("--chunk", 7, 1, 10) == 7
+    assert o.number("--temperature", 0.0, 0.0, 10.0) == 0.5 and o.integers("--prompt-ids") == [1, 2, 3]
+    for argv in [["--model", "a", "--model", "b"], ["--bogus"], ["--model"], ["--tokens", "8", "extra"]]:
+        with pytest.raises(OptionError):
+            Options(argv, {"--model", "--tokens"}, {"--help"})
+    for text in ["0", "5000", "8x", "", " 8", "+8", "1e3"]:
+        with pytest.raises(OptionError):
+            Options(["--tokens", text], {"--tokens"}).integer("--tokens", 32, 1, 4096)
+    for text in ["nan", "inf", "-1", "x"]:
+        with pytest.raises(OptionError):
+            Options(["--t", text], {"--t"}).number("--t", 0.0, 0.0, 10.0)
+    with pytest.raises(OptionError):
+        Options(["--p", "1,a"], {"--p"}).integers("--p")
