@@ -1,0 +1,153 @@
+"""Decode throughput of the Qwen3-0.6B-sized model (random weights, synthetic token ids) on one MI355X.
+
+    python bench.py [--gpus 1] [--steps 64] [--warmup 8] [--layers 28] [--batch 8] [--context 4096]
+
+A "step" is one decode step of the whole batch: one token per request through the engine's step
+function and the greedy sampler.  Requests are first filled by real prefill (portions of 2048 tokens)
+so that the timed steps end at the context length.  One JSON line is printed with decoded tokens a
+second, the same at batch 1 and 64, the prefill of 2048 tokens and the decode step's share of the
+HBM roofline.
+"""
+import argparse
+import json
+import os
+import sys
+import tempfile
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK = 8.0e12              # bytes/s, MI355X
+MFMA_PEAK = {"bf16": 2.5e15, "fp32": 157.3e12}
+SIZES = dict(hidden_size=1024, num_attention_heads=16, num_key_value_heads=8, head_dim=128,
+             intermediate_size=3072, vocab_size=151936, max_position_embeddings=40960, rms_norm_eps=1e-6,
+             rope_theta=1000000.0, tie_word_embeddings=True)
+FULL_LAYERS = 28
+PREFILL_TOKENS = 2048
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--layers", type=int, default=FULL_LAYERS)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--context", type=int, default=4096)
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points and the prefill")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU; --gpus {args.gpus} is not built (single-GPU engine)")
+        return 2
+
+    import torch
+    from mini_llm_runtime_amd.api import parse_dtype
+    from mini_llm_runtime_amd.config import config_from_dict
+    from mini_llm_runtime_amd.engine import Entry, Runner
+    from mini_llm_runtime_amd.parts import DecoderModel
+    from mini_llm_runtime_amd.sampling import Sampler
+    from mini_llm_runtime_amd.weights import write_random_model
+
+    dtype = parse_dtype(args.dtype)
+    tag = "bf16" if dtype == torch.bfloat16 else "fp32"
+    cfg = config_from_dict(dict(SIZES, architectures=["Qwen3ForCausalLM"], num_hidden_layers=args.layers))
+    with tempfile.TemporaryDirectory(prefix="mlr-bench-") as folder:
+        write_random_model(folder, cfg, seed=0)
+        model = DecoderModel.load(folder, dtype)
+    c = cfg
+    layer_params = c.hidden_size * (c.num_attention_heads + 2 * c.num_key_value_heads) * c.head_dim \
+        + c.num_attention_heads * c.head_dim * c.hidden_size + 3 * c.hidden_size * c.intermediate_size
+    elem = 2 if dtype == torch.bfloat16 else 4
+    weight_bytes = (args.layers * layer_params + c.vocab_size * c.hidden_size) * elem
+    kv_bytes_per_token = args.layers * 2 * c.num_key_value_heads * c.head_dim * elem
+    g = torch.Generator().manual_seed(0)
+
+    def decode_run(batch, steps, warmup):
+        """Fill `batch` requests so that warmup + steps decode steps end at the context length; time `steps`."""
+        runner = Runner(model, max_tokens=batch * (-(-args.context // 64) * 64), max_slots=batch,
+                        max_length=args.context, max_batch_tokens=max(PREFILL_TOKENS, batch), page_size=16)
+        sampler = Sampler(runner.kernels, runner.device, max_rows=batch)
+        fill = args.context - steps - warmup
+        assert fill >= 1
+        slots = [runner.open_request() for _ in range(batch)]
+        for s in slots:
+            ids = torch.randint(0, c.vocab_size, (fill,), generator=g).tolist()
+            for at in range(0, fill, PREFILL_TOKENS):
+                runner.step([Entry(s, ids[at:at + PREFILL_TOKENS], [])])
+        tokens = torch.randint(0, c.vocab_size, (batch,), generator=g).tolist()
+        zeros = [0.0] * batch
+
+        def one(tokens):
+            logits = runner.step([Entry(s, [t], [0]) for s, t in zip(slots, tokens)])
+            return sampler.sample(logits, zeros, zeros)
+        for _ in range(warmup):
+            tokens = one(tokens)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            tokens = one(tokens)
+        torch.cuda.synchronize()
+        seconds = time.perf_counter() - t0
+        mean_context = args.context - steps / 2.0
+        for s in slots:
+            runner.close_request(s)
+        del runner
+        torch.cuda.empty_cache()
+        return seconds, mean_context
+
+    def prefill_run():
+        runner = Runner(model, max_tokens=PREFILL_TOKENS, max_slots=1, max_length=PREFILL_TOKENS,
+                        max_batch_tokens=PREFILL_TOKENS, page_size=16)
+        ids = torch.randint(0, c.vocab_size, (PREFILL_TOKENS,), generator=g).tolist()
+        times = []
+        for i in range(4):
+            s = runner.open_request()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            runner.step([Entry(s, ids, [PREFILL_TOKENS - 1])])
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t0)
+            runner.close_request(s)
+        seconds = min(times[1:])
+        t = PREFILL_TOKENS
+        flops = 2.0 * t * args.layers * layer_params \
+            + 2.0 * t * t * c.num_attention_heads * c.head_dim * args.layers \
+            + 2.0 * c.vocab_size * c.hidden_size
+        return dict(value=round(t / seconds, 1), tokens=t, ms=round(seconds * 1e3, 3),
+                    frac=round(flops / seconds / MFMA_PEAK[tag], 5))
+
+    seconds, mean_context = decode_run(args.batch, args.steps, args.warmup)
+    ms_per_step = seconds / args.steps * 1e3
+    value = args.batch * args.steps / seconds
+    step_bytes = weight_bytes + args.batch * mean_context * kv_bytes_per_token
+    achieved = step_bytes / (seconds / args.steps) / 1e9
+    line = {
+        "metric": "decode tok/s, Qwen3-0.6B sizes, batch 8, context 4096", "value": round(value, 1),
+        "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": tag, "data": "synthetic token ids, random weights N(0, 0.02)",
+        "config": {"model": "Qwen3-0.6B sizes", "layers": args.layers, "layers_full": FULL_LAYERS,
+                   "hidden_size": c.hidden_size, "q_heads": c.num_attention_heads,
+                   "kv_heads": c.num_key_value_heads, "head_dim": c.head_dim,
+                   "intermediate_size": c.intermediate_size, "vocab_size": c.vocab_size,
+                   "tied_embeddings": True, "rope_theta": c.rope_theta, "rms_norm_eps": c.rms_norm_eps,
+                   "global_batch": args.batch, "seq_len": args.context, "page_size": 16,
+                   "sampling": "greedy", "parallelism": "single GPU"},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                     "frac": round(achieved * 1e9 / HBM_PEAK, 5)},
+    }
+    if not args.no_points:
+        line["prefill"] = prefill_run()
+        points = {}
+        for batch in (1, 64):
+            s, _ = decode_run(batch, max(8, args.steps // 2), max(2, args.warmup // 2))
+            points[f"decode_b{batch}"] = round(batch * max(8, args.steps // 2) / s, 1)
+        line["points"] = points
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
