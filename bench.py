@@ -37,6 +37,11 @@ def main():
     ap.add_argument("--context", type=int, default=4096)
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points and the prefill")
+    ap.add_argument("--only", default="all", choices=["all", "decode", "prefill"],
+                    help="profiling aid: run just the decode steps or just the prefill")
+    ap.add_argument("--fill", default="prefill", choices=["prefill", "random"],
+                    help="how the requests' caches are filled before the timed steps: by real prefill "
+                         "(default) or, as a profiling aid, with random keys and values")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not built (single-GPU engine)")
@@ -72,10 +77,15 @@ def main():
         fill = args.context - steps - warmup
         assert fill >= 1
         slots = [runner.open_request() for _ in range(batch)]
-        for s in slots:
-            ids = torch.randint(0, c.vocab_size, (fill,), generator=g).tolist()
-            for at in range(0, fill, PREFILL_TOKENS):
-                runner.step([Entry(s, ids[at:at + PREFILL_TOKENS], [])])
+        if args.fill == "random":
+            runner.cache.commit(slots, [fill] * batch)
+            for slab in runner.cache._k + runner.cache._v:
+                slab.normal_()
+        else:
+            for s in slots:
+                ids = torch.randint(0, c.vocab_size, (fill,), generator=g).tolist()
+                for at in range(0, fill, PREFILL_TOKENS):
+                    runner.step([Entry(s, ids[at:at + PREFILL_TOKENS], [])])
         tokens = torch.randint(0, c.vocab_size, (batch,), generator=g).tolist()
         zeros = [0.0] * batch
 
@@ -118,6 +128,9 @@ def main():
         return dict(value=round(t / seconds, 1), tokens=t, ms=round(seconds * 1e3, 3),
                     frac=round(flops / seconds / MFMA_PEAK[tag], 5))
 
+    if args.only == "prefill":
+        print(json.dumps({"prefill": prefill_run()}))
+        return 0
     seconds, mean_context = decode_run(args.batch, args.steps, args.warmup)
     ms_per_step = seconds / args.steps * 1e3
     value = args.batch * args.steps / seconds
@@ -138,7 +151,7 @@ def main():
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                      "frac": round(achieved * 1e9 / HBM_PEAK, 5)},
     }
-    if not args.no_points:
+    if not args.no_points and args.only == "all":
         line["prefill"] = prefill_run()
         points = {}
         for batch in (1, 64):

@@ -10,7 +10,9 @@ window).  The bookkeeping itself (free lists, tables, lengths, invariants) is na
 csrc/host/cache_manager.cpp; this module owns the device memory and keeps the device copies
 of the block tables current.
 
-Device layout of a group: k and v slabs [entries, num_pages, kv_heads, page_size, head_dim];
+Device layout of a group: keys [entries, num_pages, kv_heads, page_size, head_dim]; values transposed
+within a page, [entries, num_pages, kv_heads, head_dim, page_size], so that the keys of one channel lie
+side by side for the matrix-core product of probabilities and values;
 block table int32 [max_slots, max_blocks], -1 where no page is mapped.  Unused memory is
 filled with NaN so that a read of a never-written key shows (the reference fills its cache
 with 0xFF for the same reason, src/minillm/cuda/storage.cpp:199-200).
@@ -51,7 +53,7 @@ class StateSpec:
 @dataclass
 class KvView:
     k_pages: torch.Tensor             # [num_pages, kv_heads, page_size, head_dim]
-    v_pages: torch.Tensor
+    v_pages: torch.Tensor             # [num_pages, kv_heads, head_dim, page_size]
     block_table: torch.Tensor         # device int32 [max_slots, max_blocks]
     page_size: int
     window: Optional[int]
@@ -221,8 +223,9 @@ class CacheManager:
         self._k, self._v, self._tables = [], [], []
         for g, spec in enumerate(self.group_specs):
             shape = (len(members[g]), self.num_pages, spec.kv_heads, page_size, spec.head_dim)
+            v_shape = (len(members[g]), self.num_pages, spec.kv_heads, spec.head_dim, page_size)
             self._k.append(torch.full(shape, float("nan"), dtype=dtype, device=self.device))
-            self._v.append(torch.full(shape, float("nan"), dtype=dtype, device=self.device))
+            self._v.append(torch.full(v_shape, float("nan"), dtype=dtype, device=self.device))
             self._tables.append(torch.full((max_slots, self.book.max_blocks(g)), -1, dtype=torch.int32,
                                            device=self.device))
         self._states = {}

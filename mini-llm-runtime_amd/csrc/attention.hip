@@ -13,7 +13,9 @@
 // With more than one split the workgroups write partial (max, sum, weighted values) and
 // `attention_combine_kernel` merges them in ascending order.
 //
-// Cache layout of one layer: pages[num_pages][kv_heads][page_size][head_dim].
+// Cache layout of one layer: keys pages[num_pages][kv_heads][page_size][head_dim]; values transposed,
+// pages[num_pages][kv_heads][head_dim][page_size], so that the keys of one channel lie side by side
+// (the layout the matrix cores want for probabilities x values).
 #include "common.h"
 
 #define TILE_KEYS 64
@@ -48,7 +50,8 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(AttnArgs a) {
     float* q_lds = lds;                                    // [HEADS_PER_BLOCK][D]
     float* k_lds = q_lds + HEADS_PER_BLOCK * D;            // [TILE_KEYS][DIM_CHUNK + 1]
     float* p_lds = k_lds + TILE_KEYS * (DIM_CHUNK + 1);    // [HEADS_PER_BLOCK][TILE_KEYS]
-    __shared__ long long row_off[TILE_KEYS];               // element offset of each key's row
+    __shared__ long long row_off[TILE_KEYS];               // element offset of each key's row in k_pages
+    __shared__ long long val_off[TILE_KEYS];               // element offset of each key's column in v_pages
 
     const int pos = a.positions[m];
     const int slot = a.slots[m];
@@ -79,14 +82,16 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(AttnArgs a) {
         __syncthreads();                       // previous tile's reads of row_off / p_lds are done
         if (threadIdx.x < TILE_KEYS) {
             const int kp = t0 + threadIdx.x;
-            long long off = -1;
+            long long off = -1, voff = -1;
             if (kp >= kbegin && kp < kend) {
                 const int page = table[kp / a.page_size];
                 if (page >= 0) {
                     off = (((long long)page * a.kv_heads + kvh) * a.page_size + kp % a.page_size) * D;
+                    voff = ((long long)page * a.kv_heads + kvh) * D * a.page_size + kp % a.page_size;
                 }
             }
             row_off[threadIdx.x] = off;
+            val_off[threadIdx.x] = voff;
         }
         float score[HEADS_PER_WAVE];
 #pragma unroll
@@ -132,13 +137,13 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(AttnArgs a) {
         __syncthreads();
         const int nkeys = min(TILE_KEYS, kend - t0);
         for (int key = 0; key < nkeys; ++key) {
-            const long long off = row_off[key];
+            const long long off = val_off[key];
             if (off < 0) continue;
             float v[MAX_DIM_REGS];
 #pragma unroll
             for (int i = 0; i < MAX_DIM_REGS; ++i) {
                 const int d = lane + 64 * i;
-                v[i] = d < D ? to_float(a.v_pages[off + d]) : 0.f;
+                v[i] = d < D ? to_float(a.v_pages[off + (long long)d * a.page_size]) : 0.f;
             }
 #pragma unroll
             for (int hh = 0; hh < HEADS_PER_WAVE; ++hh) {
@@ -230,3 +235,264 @@ extern "C" int mlr_paged_attention(
     }
     return err;
 }
+
+#if MLR_BF16
+// ------------------------------------------------------------------------------------------------
+// Matrix-core attention for the bfloat16 engine.
+//
+// A workgroup serves one GROUP of up to 16 query columns that share their keys: `ntok` consecutive
+// tokens of one request (rows row0 .. row0 + ntok - 1 of the batch, positions pos0 ..) times the
+// `g = q_heads / kv_heads` query heads of one kv head; column c is (token c / g, head c % g).  A decoded
+// token is a group of one token.  Keys are walked in tiles of 32 at absolute multiples of 32; the four
+// wavefronts of the workgroup take the tiles t with t % 4 == wave, keep (max, sum, weighted values) each
+// and are merged in the order 0..3 at the end, so a column's sums depend on its own position only.
+//
+// Per tile, with v_mfma_f32_16x16x32_bf16 (D = A x B, a lane holds row/column lane % 16 and the eight
+// k-slots (lane / 16, 0..7) of A and of B):
+//   scores^T[key][column] = K[key][:] . Q[column][:]      A = 16 keys of K (rows as they lie in the page),
+//                                                         B = Q; two such products cover the 32 keys;
+//   out^T[d][column]     += V^T[d][key] . P^T[key][column]  A = 16 channels of V^T (keys side by side in
+//                                                         the transposed page), B = the probabilities,
+//                                                         which already sit in B's register layout:
+//                                                         k-slot (b, e) is key 4b + e of the first 16 keys
+//                                                         for e < 4 and key 4b + e - 4 of the second 16.
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+
+#define MFMA_TILE_KEYS 32
+
+template <int NCH>   // ceil(head_dim / 32)
+__global__ __launch_bounds__(256) void attention_mfma_kernel(AttnArgs a, const int32_t* __restrict__ group_row0,
+                                                             const int32_t* __restrict__ group_ntok) {
+    extern __shared__ float lds[];
+    const int D = a.head_dim, P = a.page_size;
+    const int g = a.q_heads / a.kv_heads;
+    const int grp = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int col = lane & 15, b = lane >> 4;
+    const int row0 = group_row0[grp], ntok = group_ntok[grp];
+    const int slot = a.slots[row0], pos0 = a.positions[row0];
+    const int tok = col / g, hh = col % g;
+    const bool col_valid = tok < ntok;
+    const int kend_c = col_valid ? pos0 + tok + 1 : 0;
+    int kbegin_c = a.window > 0 ? max(0, kend_c - a.window) : 0;
+    int lo = a.window > 0 ? max(0, pos0 + 1 - a.window) : 0;      // the group's key range
+    const int ke = pos0 + ntok;                                     // keys below ke are written
+    int hi = ke;
+    if (a.max_splits > 1) {
+        lo = max(lo, split * a.split_keys);
+        hi = min(hi, (split + 1) * a.split_keys);
+    }
+    kbegin_c = max(kbegin_c, lo);
+    const int kstop_c = min(kend_c, hi);
+
+    const __bf16* q = reinterpret_cast<const __bf16*>(a.q);
+    const __bf16* kp_base = reinterpret_cast<const __bf16*>(a.k_pages);
+    const __bf16* vp_base = reinterpret_cast<const __bf16*>(a.v_pages);
+    const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+
+    bf16x8 qf[NCH];
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) {
+        const int d0 = 32 * c + 8 * b;
+        qf[c] = zero8;
+        if (col_valid && d0 < D)
+            qf[c] = *reinterpret_cast<const bf16x8*>(q + ((size_t)(row0 + tok) * a.q_heads + kvh * g + hh) * D + d0);
+    }
+
+    float m_run = -INFINITY, l_run = 0.f;
+    floatx4 o[2 * NCH];
+#pragma unroll
+    for (int i = 0; i < 2 * NCH; ++i) o[i] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    const int32_t* table = a.block_table + (size_t)slot * a.max_blocks;
+    for (int t = lo / MFMA_TILE_KEYS + wave; t * MFMA_TILE_KEYS < hi; t += 4) {
+        const int tb = t * MFMA_TILE_KEYS;
+        bool sub_ok[2];
+        size_t kbase[2], vbase[2];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int key0 = tb + 16 * j;
+            sub_ok[j] = key0 < ke;
+            int page = -1;
+            if (sub_ok[j]) page = table[key0 / P];
+            sub_ok[j] = page >= 0;
+            const size_t pk = (size_t)(page < 0 ? 0 : page) * a.kv_heads + kvh;
+            kbase[j] = (pk * P + key0 % P) * D;
+            vbase[j] = pk * D * P + key0 % P;
+        }
+        floatx4 s[2];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            s[j] = floatx4{0.f, 0.f, 0.f, 0.f};
+            if (sub_ok[j]) {
+#pragma unroll
+                for (int c = 0; c < NCH; ++c) {
+                    const int d0 = 32 * c + 8 * b;
+                    bf16x8 kf = zero8;
+                    if (d0 < D) kf = *reinterpret_cast<const bf16x8*>(kp_base + kbase[j] + (size_t)col * D + d0);
+                    s[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[c], s[j], 0, 0, 0);
+                }
+            }
+        }
+        // this lane: keys tb + 16 j + 4 b + r of column `col`
+        float sv[2][4];
+        float tile_max = -INFINITY;
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int key = tb + 16 * j + 4 * b + r;
+                const bool ok = sub_ok[j] && key >= kbegin_c && key < kstop_c;
+                sv[j][r] = ok ? s[j][r] * a.scale : -INFINITY;
+                tile_max = fmaxf(tile_max, sv[j][r]);
+            }
+        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, MLR_WAVE));
+        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, MLR_WAVE));
+        const float m_new = fmaxf(m_run, tile_max);
+        float corr = 1.f;
+        bf16x8 pf = zero8;
+        if (m_new > -INFINITY) {
+            corr = __expf(m_run - m_new);              // m_run = -inf gives 0
+            float psum = 0.f;
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const float p = sv[j][r] > -INFINITY ? __expf(sv[j][r] - m_new) : 0.f;
+                    psum += p;
+                    pf[4 * j + r] = (__bf16)p;
+                }
+            l_run = l_run * corr + psum;
+            m_run = m_new;
+        }
+        const bool tail = tb + MFMA_TILE_KEYS > ke;      // some keys of the tile are not written yet
+#pragma unroll
+        for (int db = 0; db < 2 * NCH; ++db) {
+            if (16 * db >= D) break;
+            o[db] *= corr;
+            const int d = 16 * db + col;                  // here `col` is the channel row of A
+            bf16x8 vf = zero8;
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                if (!sub_ok[j]) continue;
+                bf16x4 v4 = *reinterpret_cast<const bf16x4*>(vp_base + vbase[j] + (size_t)d * P + 4 * b);
+                if (tail) {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        if (tb + 16 * j + 4 * b + r >= ke) v4[r] = (__bf16)0.f;
+                }
+#pragma unroll
+                for (int r = 0; r < 4; ++r) vf[4 * j + r] = v4[r];
+            }
+            o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, o[db], 0, 0, 0);
+        }
+    }
+    // per column: the four lane blocks hold partial sums of the same column
+    l_run += __shfl_xor(l_run, 16, MLR_WAVE);
+    l_run += __shfl_xor(l_run, 32, MLR_WAVE);
+
+    // merge the wavefronts: 1..3 park their state in LDS, 0 merges in ascending order and writes
+    const int stride = 16 * D + 32;                        // floats per wavefront: out^T [D][16], max[16], sum[16]
+    if (wave > 0) {
+        float* dst = lds + (size_t)(wave - 1) * stride;
+#pragma unroll
+        for (int db = 0; db < 2 * NCH; ++db) {
+            if (16 * db >= D) break;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) dst[(16 * db + 4 * b + r) * 16 + col] = o[db][r];
+        }
+        if (b == 0) {
+            dst[16 * D + col] = m_run;
+            dst[16 * D + 16 + col] = l_run;
+        }
+    }
+    __syncthreads();
+    if (wave != 0) return;
+    float m_tot = m_run;
+    for (int w = 0; w < 3; ++w) m_tot = fmaxf(m_tot, lds[(size_t)w * stride + 16 * D + col]);
+    float l_tot = 0.f;
+    float own = 0.f;
+    if (m_tot > -INFINITY) {
+        own = m_run > -INFINITY ? __expf(m_run - m_tot) : 0.f;
+        l_tot = l_run * own;
+    }
+#pragma unroll
+    for (int db = 0; db < 2 * NCH; ++db) o[db] *= own;
+    for (int w = 0; w < 3; ++w) {
+        const float* src = lds + (size_t)w * stride;
+        const float mw = src[16 * D + col];
+        if (!(mw > -INFINITY)) continue;
+        const float f = __expf(mw - m_tot);
+        l_tot += src[16 * D + 16 + col] * f;
+#pragma unroll
+        for (int db = 0; db < 2 * NCH; ++db) {
+            if (16 * db >= D) break;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) o[db][r] += src[(16 * db + 4 * b + r) * 16 + col] * f;
+        }
+    }
+    if (!col_valid) return;
+    const size_t out_row = (size_t)(row0 + tok) * a.q_heads + kvh * g + hh;
+    if (a.max_splits > 1) {
+        float* dst = a.partial + (out_row * a.max_splits + split) * (D + 2);
+#pragma unroll
+        for (int db = 0; db < 2 * NCH; ++db) {
+            if (16 * db >= D) break;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) dst[16 * db + 4 * b + r] = o[db][r];
+        }
+        if (b == 0) {
+            dst[D] = m_tot;
+            dst[D + 1] = l_tot;
+        }
+    } else {
+        __bf16* dst = reinterpret_cast<__bf16*>(a.out) + out_row * D;
+#pragma unroll
+        for (int db = 0; db < 2 * NCH; ++db) {
+            if (16 * db >= D) break;
+            bf16x4 w4;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) w4[r] = (__bf16)(l_tot > 0.f ? o[db][r] / l_tot : 0.f);
+            *reinterpret_cast<bf16x4*>(dst + 16 * db + 4 * b) = w4;
+        }
+    }
+}
+
+// Groups: group_row0[i] = first batch row of group i, group_ntok[i] = its tokens (consecutive rows of one
+// request, ntok * (q_heads / kv_heads) <= 16); together the groups cover the batch rows 0 .. rows - 1.  Needs page_size % 16 == 0, head_dim % 16 == 0,
+// q_heads / kv_heads <= 16.
+extern "C" int mlr_attention_mfma(
+    const void* q, const void* k_pages, const void* v_pages, const int32_t* block_table, int max_blocks,
+    const int32_t* slots, const int32_t* positions, void* out, float* partial, const int32_t* group_row0,
+    const int32_t* group_ntok, int groups, int rows, int q_heads, int kv_heads, int head_dim, int page_size,
+    int window, float scale, int split_keys, int max_splits, hipStream_t stream) {
+    if (groups <= 0 || rows <= 0) return 0;
+    if (head_dim % 16 != 0 || head_dim > 256 || page_size % 16 != 0 || q_heads % kv_heads != 0 ||
+        q_heads / kv_heads > 16) return -1;
+    if (max_splits > 1 && (partial == nullptr || split_keys <= 0 || split_keys % MFMA_TILE_KEYS != 0)) return -2;
+    AttnArgs a{(const elem_t*)q, (const elem_t*)k_pages, (const elem_t*)v_pages, block_table, slots,
+               positions, (elem_t*)out, partial, max_blocks, q_heads, kv_heads, head_dim, page_size,
+               window, split_keys, max_splits < 1 ? 1 : max_splits, scale};
+    dim3 grid(groups, kv_heads, a.max_splits);
+    const size_t lds = sizeof(float) * 3 * (16 * (size_t)head_dim + 32);
+    const int nch = (head_dim + 31) / 32;
+    switch (nch) {
+        case 1: attention_mfma_kernel<1><<<grid, 256, lds, stream>>>(a, group_row0, group_ntok); break;
+        case 2: attention_mfma_kernel<2><<<grid, 256, lds, stream>>>(a, group_row0, group_ntok); break;
+        case 3: attention_mfma_kernel<3><<<grid, 256, lds, stream>>>(a, group_row0, group_ntok); break;
+        case 4: attention_mfma_kernel<4><<<grid, 256, lds, stream>>>(a, group_row0, group_ntok); break;
+        case 5: attention_mfma_kernel<5><<<grid, 256, lds, stream>>>(a, group_row0, group_ntok); break;
+        case 6: attention_mfma_kernel<6><<<grid, 256, lds, stream>>>(a, group_row0, group_ntok); break;
+        case 7: attention_mfma_kernel<7><<<grid, 256, lds, stream>>>(a, group_row0, group_ntok); break;
+        default: attention_mfma_kernel<8><<<grid, 256, lds, stream>>>(a, group_row0, group_ntok); break;
+    }
+    int err = (int)hipGetLastError();
+    if (err != 0) return err;
+    if (a.max_splits > 1) {
+        attention_combine_kernel<<<dim3(rows, q_heads), 64, 0, stream>>>(a);   // the groups cover rows 0 .. rows - 1
+    }
+    return (int)hipGetLastError();
+}
+#endif

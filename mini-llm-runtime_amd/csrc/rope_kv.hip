@@ -1,9 +1,9 @@
 // Per-head RMSNorm of q and k, split-half rotation by position, and the write of k and v
 // into their pages of the cache: one kernel, one pass over the projection's output.
 //
-// Cache layout of one layer: pages[num_pages][kv_heads][page_size][head_dim]; token
-// position p of the request in slot s lies in page block_table[s][p / page_size] at row
-// p % page_size.  Norm sums and the rotation are computed in 32-bit; cos/sin come from a
+// Cache layout of one layer: keys pages[num_pages][kv_heads][page_size][head_dim], values transposed
+// pages[num_pages][kv_heads][head_dim][page_size]; token position p of the request in slot s lies in
+// page block_table[s][p / page_size] at row (values: column) p % page_size.  Norm sums and the rotation are computed in 32-bit; cos/sin come from a
 // float table [max_positions][head_dim] (first half cos, second half sin).
 #include "common.h"
 
@@ -25,12 +25,13 @@ __global__ void qk_norm_rope_kv_kernel(
     const elem_t* row = qkv + (size_t)m * ld;
     const float* cs = rope ? rope + (size_t)pos * head_dim : nullptr;
 
-    size_t cache_row = 0;
+    size_t cache_row = 0, cache_page = 0;
     bool cache_ok = false;
     if (write_cache) {
         const int page = block_table[(size_t)slot * max_blocks + pos / page_size];
         cache_ok = page >= 0;
-        cache_row = (size_t)(page < 0 ? 0 : page) * kv_heads * page_size + (pos % page_size);
+        cache_page = (size_t)(page < 0 ? 0 : page) * kv_heads;
+        cache_row = cache_page * page_size + (pos % page_size);
     }
 
     const int total = q_heads + 2 * kv_heads;
@@ -39,8 +40,8 @@ __global__ void qk_norm_rope_kv_kernel(
         if (head >= q_heads + kv_heads) {            // a value head: copy into its page
             if (cache_ok) {
                 const int kvh = head - q_heads - kv_heads;
-                elem_t* dst = v_pages + (cache_row + (size_t)kvh * page_size) * head_dim;
-                for (int d = lane; d < head_dim; d += 64) dst[d] = src[d];
+                elem_t* dst = v_pages + (cache_page + kvh) * head_dim * page_size + (pos % page_size);
+                for (int d = lane; d < head_dim; d += 64) dst[(size_t)d * page_size] = src[d];
             }
             continue;
         }

@@ -1,4 +1,4 @@
-from .context import StepContext, Workspace
+from .context import StepContext, Uploader, Workspace
 from .scheduler import Engine, EngineOptions, Request, effective_priority, schedule_batch
 from .step import Entry, Runner, StepError
 

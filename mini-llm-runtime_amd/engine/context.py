@@ -31,6 +31,32 @@ class Workspace:
         return sum(b.numel() * b.element_size() for b in self._buffers.values())
 
 
+class Uploader:
+    """Small host-to-device copies through one pinned buffer.  The copy is asynchronous; an event
+    guards the buffer so that the next use waits until the previous copy has left it."""
+
+    def __init__(self, capacity, device):
+        self.device = torch.device(device)
+        self._host = torch.empty(capacity, dtype=torch.int32).pin_memory()
+        self._event = torch.cuda.Event()
+        self._busy = False
+
+    def send(self, values, dst):
+        """values: list of ints; dst: device int32 vector of at least that many elements."""
+        n = len(values)
+        if n > self._host.numel():
+            if self._busy:
+                self._event.synchronize()
+                self._busy = False
+            self._host = torch.empty(max(n, 2 * self._host.numel()), dtype=torch.int32).pin_memory()
+        if self._busy:
+            self._event.synchronize()
+        self._host[:n] = torch.tensor(values, dtype=torch.int32)
+        dst[:n].copy_(self._host[:n], non_blocking=True)
+        self._event.record()
+        self._busy = True
+
+
 class StepContext:
     """One step's view for the parts: the tokens with their positions and slots (device int32
     vectors of equal length), the segments they form (host), the cache, the kernels and the
@@ -44,6 +70,31 @@ class StepContext:
         self.token_ids = self.positions = self.slots = None
         self.segments = []            # (slot, first row, number of tokens, first position)
         self.max_context = 0          # largest position + 1 among the step's tokens
+        self._groups = {}
+        self._group_upload = None
+
+    def begin_step(self):
+        self._groups = {}
+
+    def token_groups(self, tokens_per_group):
+        """The step's rows cut into groups of at most `tokens_per_group` consecutive tokens of one request:
+        (first row of each group, tokens in each group) as device int32 vectors, and their number."""
+        hit = self._groups.get(tokens_per_group)
+        if hit is not None:
+            return hit
+        first, count = [], []
+        for _, row, n, _ in self.segments:
+            for i in range(0, n, tokens_per_group):
+                first.append(row + i)
+                count.append(min(tokens_per_group, n - i))
+        g = len(first)
+        dev = self.workspace.get(f"token_groups_{tokens_per_group}", (2 * g,), torch.int32)
+        if self._group_upload is None:
+            self._group_upload = Uploader(4096, dev.device)
+        self._group_upload.send(first + count, dev)
+        hit = (dev[:g], dev[g:2 * g], g)
+        self._groups[tokens_per_group] = hit
+        return hit
 
     def attention_split(self, rows, q_heads, head_dim):
         """(split_keys, max_splits, partial buffer): small batches over long contexts split the

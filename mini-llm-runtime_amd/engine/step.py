@@ -14,7 +14,7 @@ import torch
 
 from ..cache.manager import CacheManager
 from ..kernels import Kernels
-from .context import StepContext, Workspace
+from .context import StepContext, Uploader, Workspace
 
 
 class StepError(ValueError):
@@ -43,7 +43,7 @@ class Runner:
         self.workspace = Workspace(self.device)
         self.ctx = StepContext(self.kernels, self.cache, self.workspace, self.dtype, self.max_length,
                                split_keys, split_max_tokens)
-        self._staging = torch.empty(4 * self.max_batch_tokens, dtype=torch.int32).pin_memory()
+        self._upload = Uploader(4 * self.max_batch_tokens, self.device)
         self._meta = torch.empty(4 * self.max_batch_tokens, dtype=torch.int32, device=self.device)
         self.poisoned = False
         self.steps = 0
@@ -105,10 +105,9 @@ class Runner:
                 slot_of.extend([e.slot] * n)
                 rows.extend(base + int(w) for w in e.want)
             r = len(rows)
-            flat = torch.tensor(ids + pos + slot_of + rows, dtype=torch.int32)
-            self._staging[:flat.numel()].copy_(flat)
-            self._meta[:flat.numel()].copy_(self._staging[:flat.numel()], non_blocking=True)
+            self._upload.send(ids + pos + slot_of + rows, self._meta)
             ctx = self.ctx
+            ctx.begin_step()
             ctx.n_tokens = total
             ctx.token_ids = self._meta[0:total]
             ctx.positions = self._meta[total:2 * total]

@@ -153,7 +153,7 @@ class Kernels:
         _tensor(k_pages, "k_pages", self.dtype, ndim=4)
         _need(tuple(k_pages.shape[1:]) == (kv_heads, page_size, head_dim),
               f"k_pages: expected [pages, {kv_heads}, {page_size}, {head_dim}], got {tuple(k_pages.shape)}")
-        _tensor(v_pages, "v_pages", self.dtype, tuple(k_pages.shape))
+        _tensor(v_pages, "v_pages", self.dtype, (k_pages.shape[0], kv_heads, head_dim, page_size))
 
     def qk_norm_rope_kv(self, qkv, q_out, k_pages, v_pages, block_table, slots, positions, q_norm_w,
                         k_norm_w, eps, rope, q_heads, kv_heads, head_dim, page_size, write_cache=True):
@@ -215,6 +215,45 @@ class Kernels:
                _p(positions), _p(out), _p(partial), _c_int(m), _c_int(q_heads), _c_int(kv_heads),
                _c_int(head_dim), _c_int(page_size), _c_int(window or 0), _c_float(scale),
                _c_int(split_keys), _c_int(max_splits), _stream()), "paged_attention")
+
+    def mfma_attention_supported(self, q_heads, kv_heads, head_dim, page_size):
+        """The matrix-core attention kernel serves the bfloat16 engine for pages that are a multiple of
+        16 tokens, head sizes that are a multiple of 16 and up to 16 query heads per kv head."""
+        return (self.dtype == torch.bfloat16 and page_size % 16 == 0 and head_dim % 16 == 0
+                and head_dim <= MAX_HEAD_DIM and q_heads % kv_heads == 0 and q_heads // kv_heads <= 16)
+
+    def attention_mfma(self, q, k_pages, v_pages, block_table, slots, positions, out, group_row0, group_ntok,
+                       groups, q_heads, kv_heads, head_dim, page_size, scale, window=None, split_keys=0,
+                       max_splits=1, partial=None):
+        """As `paged_attention`, on the matrix cores.  The batch rows are covered by `groups` groups of
+        consecutive rows of one request each (group_row0[i], group_ntok[i]), at most 16 // (q_heads //
+        kv_heads) tokens a group."""
+        _need(self.mfma_attention_supported(q_heads, kv_heads, head_dim, page_size),
+              "attention_mfma: sizes not supported (bfloat16, page_size % 16 == 0, head_dim % 16 == 0, "
+              "at most 16 query heads per kv head)")
+        _tensor(q, "q", self.dtype, ndim=2)
+        m = q.shape[0]
+        _need(q.shape[1] == q_heads * head_dim, "q: wrong width")
+        _tensor(out, "out", self.dtype, (m, q_heads * head_dim))
+        self._check_cache(k_pages, v_pages, kv_heads, head_dim, page_size)
+        _tensor(block_table, "block_table", torch.int32, ndim=2)
+        _tensor(slots, "slots", torch.int32, (m,))
+        _tensor(positions, "positions", torch.int32, (m,))
+        _tensor(group_row0, "group_row0", torch.int32, (groups,))
+        _tensor(group_ntok, "group_ntok", torch.int32, (groups,))
+        _need(kv_heads <= 65535 and max_splits <= 65535, "too many kv heads or key splits for the grid")
+        if max_splits > 1:
+            _need(split_keys > 0 and split_keys % ATTENTION_TILE_KEYS == 0,
+                  f"split_keys must be a multiple of {ATTENTION_TILE_KEYS}")
+            _need(partial is not None, "partial buffer needed for split attention")
+            _tensor(partial, "partial", torch.float32, ndim=1)
+            _need(partial.numel() >= self.attention_partial_numel(m, q_heads, head_dim, max_splits),
+                  "partial buffer too small")
+        fn = self._lib("attention").mlr_attention_mfma
+        _ok(fn(_p(q), _p(k_pages), _p(v_pages), _p(block_table), _c_int(block_table.shape[1]), _p(slots),
+               _p(positions), _p(out), _p(partial), _p(group_row0), _p(group_ntok), _c_int(groups), _c_int(m),
+               _c_int(q_heads), _c_int(kv_heads), _c_int(head_dim), _c_int(page_size), _c_int(window or 0),
+               _c_float(scale), _c_int(split_keys), _c_int(max_splits), _stream()), "attention_mfma")
 
     # -- sampling ----------------------------------------------------------------------------
     def sample(self, logits, temperature, uniform, tokens, status):

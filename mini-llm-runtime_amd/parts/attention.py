@@ -77,9 +77,16 @@ class GqaAttention:
             s.q_heads, s.kv_heads, s.head_dim, view.page_size, write_cache)
         attn = ctx.workspace.get("attn", (m, s.q_heads * s.head_dim), x.dtype)
         split_keys, max_splits, partial = ctx.attention_split(m, s.q_heads, s.head_dim)
-        k.paged_attention(q, view.k_pages, view.v_pages, view.block_table, ctx.slots, ctx.positions, attn,
-                          s.q_heads, s.kv_heads, s.head_dim, view.page_size, float(s.scale),
-                          window=s.window, split_keys=split_keys, max_splits=max_splits, partial=partial)
+        if k.mfma_attention_supported(s.q_heads, s.kv_heads, s.head_dim, view.page_size):
+            first, count, groups = ctx.token_groups(max(1, 16 // (s.q_heads // s.kv_heads)))
+            k.attention_mfma(q, view.k_pages, view.v_pages, view.block_table, ctx.slots, ctx.positions, attn,
+                             first, count, groups, s.q_heads, s.kv_heads, s.head_dim, view.page_size,
+                             float(s.scale), window=s.window, split_keys=split_keys, max_splits=max_splits,
+                             partial=partial)
+        else:
+            k.paged_attention(q, view.k_pages, view.v_pages, view.block_table, ctx.slots, ctx.positions, attn,
+                              s.q_heads, s.kv_heads, s.head_dim, view.page_size, float(s.scale),
+                              window=s.window, split_keys=split_keys, max_splits=max_splits, partial=partial)
         out = ctx.workspace.get("mixer_out", (m, s.hidden), x.dtype)
         k.gemm(attn, self.o, out)
         return out

@@ -175,7 +175,7 @@ def test_qk_norm_rope_kv(dtype, shape):
     eps, base = 1e-5, 1e6
     rope = rope_table(2048, d, base)
     k_pages = torch.full((n_pages, hkv, page, d), float("nan"), dtype=dtype, device="cuda")
-    v_pages = torch.full((n_pages, hkv, page, d), float("nan"), dtype=dtype, device="cuda")
+    v_pages = torch.full((n_pages, hkv, d, page), float("nan"), dtype=dtype, device="cuda")
     q_out = torch.empty((m, hq * d), dtype=dtype, device="cuda")
     pos_t = torch.tensor(positions, dtype=torch.int32)
     k.qk_norm_rope_kv(qkv, q_out, k_pages, v_pages, table.cuda(), slots.cuda(), pos_t.cuda(), qw, kw, eps,
@@ -195,11 +195,11 @@ def test_qk_norm_rope_kv(dtype, shape):
         pg = table[slots[i], p // page].item()
         written[pg, p % page] = True
         torch.testing.assert_close(k_pages[pg, :, p % page].double().cpu(), k_want[i], **tol(dtype))
-        assert torch.equal(v_pages[pg, :, p % page].cpu(), qkv[i, (hq + hkv) * d:].view(hkv, d).cpu())
+        assert torch.equal(v_pages[pg, :, :, p % page].cpu(), qkv[i, (hq + hkv) * d:].view(hkv, d).cpu())
     # nothing else was touched
     untouched = ~written[:, None, :, None].expand(n_pages, hkv, page, d)
     assert torch.isnan(k_pages.float().cpu()[untouched]).all()
-    assert torch.isnan(v_pages.float().cpu()[untouched]).all()
+    assert torch.isnan(v_pages.float().cpu().transpose(2, 3)[untouched]).all()
     # no norm, no rotation, no cache write
     k2 = torch.full_like(k_pages, float("nan"))
     k.qk_norm_rope_kv(qkv, q_out, k2, v_pages, table.cuda(), slots.cuda(), pos_t.cuda(), None, None, 0.0,
@@ -234,6 +234,9 @@ def plain_attention(q, keys, values, scale, window):
     (4, 2, 64, 16, [200, 40], 33, 0),
     (4, 2, 64, 16, [200, 40], 64, 128),
     (2, 1, 16, 4, [1000], None, 256),
+    (6, 3, 48, 32, [100, 70], None, 0),
+    (32, 2, 64, 16, [130, 5], None, 64),
+    (8, 8, 80, 16, [77], 40, 0),
 ])
 def test_paged_attention(dtype, case):
     """Every length is one request whose LAST token is the query (a decoded token) plus, for the
@@ -248,7 +251,7 @@ def test_paged_attention(dtype, case):
     perm = torch.randperm(n_pages, generator=g).tolist()
     table = torch.full((len(lengths), max_blocks), -1, dtype=torch.int32)
     k_pages = torch.full((n_pages, hkv, page, d), float("nan"), dtype=dtype)
-    v_pages = torch.full((n_pages, hkv, page, d), float("nan"), dtype=dtype)
+    v_pages = torch.full((n_pages, hkv, d, page), float("nan"), dtype=dtype)
     keys, values = [], []
     for s, L in enumerate(lengths):
         kk = torch.randn((L, hkv, d), generator=g).to(dtype)
@@ -260,7 +263,7 @@ def test_paged_attention(dtype, case):
             table[s, b] = pg
             n = min(page, L - b * page)
             k_pages[pg, :, :n] = kk[b * page:b * page + n].transpose(0, 1)
-            v_pages[pg, :, :n] = vv[b * page:b * page + n].transpose(0, 1)
+            v_pages[pg, :, :, :n] = vv[b * page:b * page + n].permute(1, 2, 0)
     rows = [(0, p) for p in range(lengths[0])] + [(s, L - 1) for s, L in enumerate(lengths) if s > 0]
     m = len(rows)
     q = (torch.randn((m, hq, d), generator=g) * 2).to(dtype)
@@ -276,9 +279,26 @@ def test_paged_attention(dtype, case):
                       hq, hkv, d, page, scale, window=window, split_keys=split_keys, max_splits=max_splits,
                       partial=partial)
     got = out.double().cpu().view(m, hq, d)
-    for i, (s, p) in enumerate(rows):
-        want = plain_attention(q[i].double(), keys[s][:p + 1].double(), values[s][:p + 1].double(), scale, window)
-        torch.testing.assert_close(got[i], want, **tol(dtype))
+    wants = [plain_attention(q[i].double(), keys[s][:p + 1].double(), values[s][:p + 1].double(), scale, window)
+             for i, (s, p) in enumerate(rows)]
+    for i in range(m):
+        torch.testing.assert_close(got[i], wants[i], **tol(dtype))
+    if not k.mfma_attention_supported(hq, hkv, d, page):
+        return
+    # the matrix-core kernel: the first request's rows in groups of consecutive tokens, the others alone
+    tq = max(1, 16 // (hq // hkv))
+    first = list(range(0, lengths[0], tq)) + list(range(lengths[0], m))
+    count = [min(tq, lengths[0] - r) for r in range(0, lengths[0], tq)] + [1] * (m - lengths[0])
+    out2 = torch.full((m, hq * d), float("nan"), dtype=dtype, device="cuda")
+    if partial is not None:
+        partial.fill_(float("nan"))
+    k.attention_mfma(q.view(m, hq * d).cuda(), k_pages.cuda(), v_pages.cuda(), table.cuda(), slots, pos, out2,
+                     torch.tensor(first, dtype=torch.int32).cuda(), torch.tensor(count, dtype=torch.int32).cuda(),
+                     len(first), hq, hkv, d, page, scale, window=window, split_keys=split_keys,
+                     max_splits=max_splits, partial=partial)
+    got = out2.double().cpu().view(m, hq, d)
+    for i in range(m):
+        torch.testing.assert_close(got[i], wants[i], **tol(dtype))
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -297,11 +317,11 @@ def test_attention_finds_one_far_key(dtype):
         n_blocks = (L + page - 1) // page
         table = torch.arange(n_blocks - 1, -1, -1, dtype=torch.int32)[None, :].contiguous()
         k_pages = torch.zeros((n_blocks, 1, page, d))
-        v_pages = torch.zeros((n_blocks, 1, page, d))
+        v_pages = torch.zeros((n_blocks, 1, d, page))
         for b in range(n_blocks):
             n = min(page, L - b * page)
             k_pages[table[0, b], 0, :n] = kk[b * page:b * page + n, 0]
-            v_pages[table[0, b], 0, :n] = vv[b * page:b * page + n, 0]
+            v_pages[table[0, b], 0, :, :n] = vv[b * page:b * page + n, 0].T
         out = torch.empty((1, d), dtype=dtype, device="cuda")
         for split_keys in (0, 128):
             max_splits = (L + split_keys - 1) // split_keys if split_keys else 1
@@ -310,6 +330,14 @@ def test_attention_finds_one_far_key(dtype):
                               torch.zeros(1, dtype=torch.int32).cuda(), torch.tensor([L - 1], dtype=torch.int32).cuda(),
                               out, 1, 1, d, page, 1.0, split_keys=split_keys, max_splits=max_splits, partial=partial)
             torch.testing.assert_close(out.float().cpu()[0], vv[far, 0].to(dtype).float(), atol=3e-2, rtol=3e-2)
+            if k.mfma_attention_supported(1, 1, d, page):
+                out.fill_(float("nan"))
+                one = torch.ones(1, dtype=torch.int32).cuda()
+                k.attention_mfma(q.to(dtype).cuda(), k_pages.to(dtype).cuda(), v_pages.to(dtype).cuda(), table.cuda(),
+                                 torch.zeros(1, dtype=torch.int32).cuda(), torch.tensor([L - 1], dtype=torch.int32).cuda(),
+                                 out, torch.zeros(1, dtype=torch.int32).cuda(), one, 1, 1, 1, d, page, 1.0,
+                                 split_keys=split_keys, max_splits=max_splits, partial=partial)
+                torch.testing.assert_close(out.float().cpu()[0], vv[far, 0].to(dtype).float(), atol=3e-2, rtol=3e-2)
 
 
 @pytest.mark.parametrize("vocab", [1, 31, 32, 33, 257, 1024, 1025, 151936])
@@ -400,9 +428,10 @@ def test_attention_window_edge(dtype, window):
         n_blocks = (L + page - 1) // page
         table = torch.arange(n_blocks, dtype=torch.int32)[None, :].contiguous()
         k_pages = torch.zeros((n_blocks, 1, page, d))
-        v_pages = torch.zeros((n_blocks, 1, page, d))
         k_pages.view(-1, d)[:L] = kk
-        v_pages.view(-1, d)[:L] = vv
+        rows = torch.zeros((n_blocks * page, d))
+        rows[:L] = vv
+        v_pages = rows.view(n_blocks, 1, page, d).transpose(2, 3).contiguous()
         out = torch.empty((1, d), dtype=dtype, device="cuda")
         k.paged_attention(q.to(dtype).cuda(), k_pages.to(dtype).cuda(), v_pages.to(dtype).cuda(), table.cuda(),
                           torch.zeros(1, dtype=torch.int32).cuda(), torch.tensor([L - 1], dtype=torch.int32).cuda(),
@@ -413,3 +442,11 @@ def test_attention_window_edge(dtype, window):
         torch.testing.assert_close(out.double().cpu(), want, **tol(dtype))
         close_to_hot = (out.float().cpu()[0] - vv[hot].to(dtype).float()).abs().max() < 0.05
         assert bool(close_to_hot) == inside, (window, inside, lo)
+        if k.mfma_attention_supported(1, 1, d, page):
+            out.fill_(float("nan"))
+            k.attention_mfma(q.to(dtype).cuda(), k_pages.to(dtype).cuda(), v_pages.to(dtype).cuda(), table.cuda(),
+                             torch.zeros(1, dtype=torch.int32).cuda(), torch.tensor([L - 1], dtype=torch.int32).cuda(),
+                             out, torch.zeros(1, dtype=torch.int32).cuda(), torch.ones(1, dtype=torch.int32).cuda(),
+                             1, 1, 1, d, page, 1.0, window=window)
+            torch.testing.assert_close(out.double().cpu(), want, **tol(dtype))
+            assert bool((out.float().cpu()[0] - vv[hot].to(dtype).float()).abs().max() < 0.05) == inside
