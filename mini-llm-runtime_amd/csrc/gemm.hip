@@ -166,6 +166,71 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_bf16_kernel(
     }
 }
 
+// Few rows (M <= 64): the weight is streamed once, straight from memory into the matrix cores.  A
+// workgroup owns 16 output columns (16 rows of w); its four wavefronts each take a quarter of k, and
+// their partial sums are added in the order 0..3, so the result does not depend on M.  The weight
+// is the A operand (rows n), the activation the B operand (columns m): a lane ends up with four
+// consecutive n of one m.
+template <int MT, bool OUT_FLOAT>
+__global__ __launch_bounds__(256) void gemm_skinny_kernel(const __bf16* __restrict__ a,
+                                                          const __bf16* __restrict__ w,
+                                                          void* __restrict__ out_raw, int M, int N, int K) {
+    __shared__ float part[3][MT][64][4];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r16 = lane & 15, b = lane >> 4;
+    const int n0 = blockIdx.x * 16;
+    const bool vector_ok = (K % 8) == 0;
+    const int steps = (K + 31) / 32;
+    const int per_wave = (steps + 3) / 4;
+    const int s_begin = wave * per_wave, s_end = min(steps, s_begin + per_wave);
+    floatx4 acc[MT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i) acc[i] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+    for (int s = s_begin; s < s_end; ++s) {
+        const int k = s * 32 + b * 8;
+        const bf16x8 wf = load_k8(w, n0 + r16, N, k, K, vector_ok);
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+            const bf16x8 xf = load_k8(a, 16 * i + r16, M, k, K, vector_ok);
+            acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, xf, acc[i], 0, 0, 0);
+        }
+    }
+    if (wave > 0) {
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) part[wave - 1][i][lane][r] = acc[i][r];
+    }
+    __syncthreads();
+    if (wave != 0) return;
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+        const int m = 16 * i + r16;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            float v = acc[i][r];
+            for (int p = 0; p < 3; ++p) v += part[p][i][lane][r];
+            const int n = n0 + 4 * b + r;
+            if (m < M && n < N) {
+                if (OUT_FLOAT) ((float*)out_raw)[(size_t)m * N + n] = v;
+                else ((__bf16*)out_raw)[(size_t)m * N + n] = (__bf16)v;
+            }
+        }
+    }
+}
+
+template <int MT>
+static int launch_skinny(const void* a, const void* w, void* out, int M, int N, int K, int out_float,
+                         hipStream_t stream) {
+    dim3 grid((N + 15) / 16);
+    if (out_float)
+        gemm_skinny_kernel<MT, true><<<grid, 256, 0, stream>>>((const __bf16*)a, (const __bf16*)w, out, M, N, K);
+    else
+        gemm_skinny_kernel<MT, false><<<grid, 256, 0, stream>>>((const __bf16*)a, (const __bf16*)w, out, M, N, K);
+    return (int)hipGetLastError();
+}
+
 template <int WM, int WN, int TM, int TN>
 static int launch(const void* a, const void* w, void* out, int M, int N, int K, int out_float,
                   hipStream_t stream) {
@@ -185,8 +250,10 @@ extern "C" int mlr_gemm(const void* a, const void* w, void* out, int M, int N, i
                         hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
     if (K <= 0) return -1;
-    if (M <= 16) return launch<1, 4, 1, 1>(a, w, out, M, N, K, out_float, stream);   // 16 x 64
-    if (M <= 64) return launch<2, 2, 2, 2>(a, w, out, M, N, K, out_float, stream);   // 64 x 64
+    if (M <= 16) return launch_skinny<1>(a, w, out, M, N, K, out_float, stream);
+    if (M <= 32) return launch_skinny<2>(a, w, out, M, N, K, out_float, stream);
+    if (M <= 64) return launch_skinny<4>(a, w, out, M, N, K, out_float, stream);
+    if (M <= 128) return launch<2, 2, 2, 2>(a, w, out, M, N, K, out_float, stream);  // 64 x 64
     return launch<2, 2, 4, 4>(a, w, out, M, N, K, out_float, stream);                // 128 x 128
 }
 #endif

@@ -72,9 +72,11 @@ class StepContext:
         self.max_context = 0          # largest position + 1 among the step's tokens
         self._groups = {}
         self._group_upload = None
+        self.single_token_groups = None
 
     def begin_step(self):
         self._groups = {}
+        self.single_token_groups = None
 
     def token_groups(self, tokens_per_group):
         """The step's rows cut into groups of at most `tokens_per_group` consecutive tokens of one request:
@@ -82,6 +84,8 @@ class StepContext:
         hit = self._groups.get(tokens_per_group)
         if hit is not None:
             return hit
+        if self.single_token_groups is not None:      # a step of single tokens with fixed buffers
+            return self.single_token_groups
         first, count = [], []
         for _, row, n, _ in self.segments:
             for i in range(0, n, tokens_per_group):

@@ -30,7 +30,7 @@ class Entry:
 
 class Runner:
     def __init__(self, model, max_tokens, max_slots=4, max_length=None, max_batch_tokens=None,
-                 page_size=16, split_keys=256, split_max_tokens=256):
+                 page_size=16, split_keys=256, split_max_tokens=256, use_graphs=True, graph_max_batch=256):
         self.model = model
         self.dtype, self.device = model.dtype, model.device
         spec = model.spec
@@ -47,6 +47,11 @@ class Runner:
         self._meta = torch.empty(4 * self.max_batch_tokens, dtype=torch.int32, device=self.device)
         self.poisoned = False
         self.steps = 0
+        # steps of single tokens (decoding) are launch-bound: after a first eager run a batch size is
+        # captured once as a HIP graph over fixed buffers and replayed from then on
+        self.use_graphs = use_graphs and model.graph_safe()
+        self.graph_max_batch = graph_max_batch
+        self._decode_graphs = {}
 
     # -- requests ------------------------------------------------------------------------------
     def open_request(self):
@@ -60,6 +65,44 @@ class Runner:
 
     def free_slots(self):
         return self.cache.book.free_slots()
+
+    # -- decoding steps as graphs --------------------------------------------------------------
+    def _decode_step(self, entries, first):
+        """One token per request, logits wanted for each: the same kernels as any step, launched from a
+        captured graph.  The graph's buffers are fixed: token ids, positions, slots and wanted rows live
+        in a vector of their own per batch size, key splits are laid out for the longest context, and the
+        logits land in the usual scratch buffer."""
+        n = len(entries)
+        state = self._decode_graphs.get(n)
+        if state is None:
+            meta = torch.empty(4 * n + 2 * n, dtype=torch.int32, device=self.device)
+            meta[3 * n:4 * n] = torch.arange(n, dtype=torch.int32, device=self.device)      # wanted rows
+            meta[4 * n:5 * n] = torch.arange(n, dtype=torch.int32, device=self.device)      # groups: row i ...
+            meta[5 * n:6 * n] = 1                                                           # ... one token each
+            state = dict(meta=meta, upload=Uploader(3 * n, self.device), graph=None, logits=None, runs=0)
+            self._decode_graphs[n] = state
+        meta = state["meta"]
+        state["upload"].send([int(e.tokens[0]) for e in entries] + list(first) + [e.slot for e in entries], meta)
+        if state["graph"] is not None:
+            state["graph"].replay()
+            return state["logits"]
+        ctx = self.ctx
+        ctx.begin_step()
+        ctx.n_tokens = n
+        ctx.token_ids, ctx.positions, ctx.slots = meta[0:n], meta[n:2 * n], meta[2 * n:3 * n]
+        ctx.segments = [(e.slot, i, 1, p0) for i, (e, p0) in enumerate(zip(entries, first))]
+        ctx.max_context = self.max_length                 # the graph must serve every later context
+        ctx.single_token_groups = (meta[4 * n:5 * n], meta[5 * n:6 * n], n)
+        want_rows = meta[3 * n:4 * n]
+        state["runs"] += 1
+        if state["runs"] == 1:                            # first time: eager, sizes the scratch buffers
+            return self.model.forward(ctx, want_rows)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            logits = self.model.forward(ctx, want_rows)
+        state["graph"], state["logits"] = graph, logits
+        graph.replay()
+        return logits
 
     # -- the step ------------------------------------------------------------------------------
     def _validate(self, entries):
@@ -94,6 +137,12 @@ class Runner:
         first = [self.cache.length(s) for s in slots]
         self.cache.commit(slots, counts)
         try:
+            if (self.use_graphs and total == len(entries) <= self.graph_max_batch
+                    and all(list(e.want) == [0] for e in entries)):
+                logits = self._decode_step(entries, first)
+                self.cache.retire(slots)
+                self.steps += 1
+                return logits
             ids, pos, slot_of, rows = [], [], [], []
             segments = []
             for e, p0 in zip(entries, first):

@@ -14,6 +14,7 @@ from .registry import PartError, build_part, register_part
 
 @register_part("mixer", "gqa_attention")
 class GqaAttention:
+    graph_safe = True        # forward launches kernels over the step's device vectors only
     def __init__(self, spec):
         self.spec = spec
         s = spec

@@ -9,6 +9,7 @@ from .registry import build_part, register_part
 
 @register_part("block", "prenorm")
 class PreNormBlock:
+    graph_safe = True        # forward launches kernels over the step's device vectors only
     def __init__(self, spec):
         self.norm1 = build_part("norm", spec.norm1)
         self.mixer = build_part("mixer", spec.mixer)

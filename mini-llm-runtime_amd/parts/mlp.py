@@ -10,6 +10,7 @@ from .registry import PartError, register_part
 
 @register_part("ffn", "swiglu")
 class SwiGluMlp:
+    graph_safe = True        # forward launches kernels over the step's device vectors only
     def __init__(self, spec):
         if spec.activation != "silu":
             raise PartError(f"activation {spec.activation!r} is not built (silu)")

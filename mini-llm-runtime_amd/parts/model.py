@@ -103,6 +103,11 @@ class DecoderModel:
                     names.update(part.libraries())
         return sorted(names)
 
+    def graph_safe(self):
+        """True when every part of every layer may be captured in a graph."""
+        return all(getattr(part, "graph_safe", False) for block in self.blocks
+                   for part in [block, *block.parts().values()]) and getattr(self.final_norm, "graph_safe", False)
+
     def weight_bytes(self):
         seen, total = set(), 0
         tensors = [self.embed, self.lm_head, self.final_norm.weight]

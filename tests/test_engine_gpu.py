@@ -147,10 +147,14 @@ def test_steady_steps_allocate_nothing(model_folders):
     r = runner_for(model, "B", max_tokens=256)
     s = r.open_request()
     r.step([Entry(s, list(range(40)), [39])])
-    r.step([Entry(s, [1], [0])])
+    for t in range(3):                                   # eager, then captured as a graph, then replayed
+        r.step([Entry(s, [t], [0])])
+    r.step([Entry(s, [5, 6], [1])])
     torch.cuda.synchronize()
     before = torch.cuda.memory_stats()["allocation.all.allocated"]
     for t in range(30):
         r.step([Entry(s, [t], [0])])
+        if t % 7 == 0:
+            r.step([Entry(s, [t, t + 1], [1])])          # a portion between decoded tokens
     torch.cuda.synchronize()
     assert torch.cuda.memory_stats()["allocation.all.allocated"] == before
