@@ -186,27 +186,52 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(AttnArgs a) {
     }
 }
 
-// out[m, head, :] = sum_s w_s acc_s / sum_s w_s l_s with w_s = exp(max_s - max), over the
-// splits that hold keys of this token, in ascending order.
-__global__ void attention_combine_kernel(AttnArgs a) {
+// out[m, head, :] = sum_s w_s acc_s / sum_s w_s l_s with w_s = exp(max_s - max), over the splits
+// first_split .. last_split that hold keys of this token, in ascending order.  One wavefront per
+// (token, head); the splits' weights go through LDS, the channel loads are independent of each other.
+#define COMBINE_MAX_SPLITS 1024
+__global__ __launch_bounds__(64) void attention_combine_kernel(AttnArgs a) {
+    __shared__ float w_lds[COMBINE_MAX_SPLITS];
+    __shared__ float l_lds[COMBINE_MAX_SPLITS];
     const int m = blockIdx.x, head = blockIdx.y;
     const int D = a.head_dim;
     const int pos = a.positions[m];
-    const int nsplit = min(a.max_splits, pos / a.split_keys + 1);
-    const float* base = a.partial + ((size_t)m * a.q_heads + head) * a.max_splits * (D + 2);
+    const int first = a.window > 0 ? max(0, pos + 1 - a.window) / a.split_keys : 0;
+    const int last = min(a.max_splits - 1, pos / a.split_keys);
+    const int n = last - first + 1;
+    const float* base = a.partial + (((size_t)m * a.q_heads + head) * a.max_splits + first) * (D + 2);
     float gmax = -INFINITY;
-    for (int s = 0; s < nsplit; ++s) gmax = fmaxf(gmax, base[(size_t)s * (D + 2) + D]);
-    for (int d = threadIdx.x; d < D; d += blockDim.x) {
-        float num = 0.f, den = 0.f;
-        for (int s = 0; s < nsplit; ++s) {
-            const float* p = base + (size_t)s * (D + 2);
-            const float smax = p[D];
-            if (smax == -INFINITY) continue;
-            const float w = expf(smax - gmax);
-            num += w * p[d];
-            den += w * p[D + 1];
+    for (int s = threadIdx.x; s < n; s += 64) {
+        const float smax = base[(size_t)s * (D + 2) + D];
+        w_lds[s] = smax;
+        l_lds[s] = base[(size_t)s * (D + 2) + D + 1];
+        gmax = fmaxf(gmax, smax);
+    }
+    gmax = wave_max(gmax);
+    __syncthreads();
+    for (int s = threadIdx.x; s < n; s += 64) {
+        const float smax = w_lds[s];
+        w_lds[s] = smax > -INFINITY ? expf(smax - gmax) : 0.f;       // an empty split holds zeros
+    }
+    __syncthreads();
+    float den = 0.f;
+    for (int s = 0; s < n; ++s) den += w_lds[s] * l_lds[s];
+    float num[MAX_DIM_REGS];
+#pragma unroll
+    for (int i = 0; i < MAX_DIM_REGS; ++i) num[i] = 0.f;
+    for (int s = 0; s < n; ++s) {
+        const float w = w_lds[s];
+        const float* p = base + (size_t)s * (D + 2);
+#pragma unroll
+        for (int i = 0; i < MAX_DIM_REGS; ++i) {
+            const int d = threadIdx.x + 64 * i;
+            if (d < D) num[i] += w * p[d];
         }
-        a.out[((size_t)m * a.q_heads + head) * D + d] = from_float<elem_t>(den > 0.f ? num / den : 0.f);
+    }
+#pragma unroll
+    for (int i = 0; i < MAX_DIM_REGS; ++i) {
+        const int d = threadIdx.x + 64 * i;
+        if (d < D) a.out[((size_t)m * a.q_heads + head) * D + d] = from_float<elem_t>(den > 0.f ? num[i] / den : 0.f);
     }
 }
 
@@ -217,7 +242,8 @@ extern "C" int mlr_paged_attention(
     int split_keys, int max_splits, hipStream_t stream) {
     if (rows <= 0) return 0;
     if (head_dim > 64 * MAX_DIM_REGS || q_heads % kv_heads != 0) return -1;
-    if (max_splits > 1 && (partial == nullptr || split_keys <= 0 || split_keys % TILE_KEYS != 0)) return -2;
+    if (max_splits > 1 && (partial == nullptr || split_keys <= 0 || split_keys % TILE_KEYS != 0 ||
+                           max_splits > COMBINE_MAX_SPLITS)) return -2;
     AttnArgs a{(const elem_t*)q, (const elem_t*)k_pages, (const elem_t*)v_pages, block_table, slots,
                positions, (elem_t*)out, partial, max_blocks, q_heads, kv_heads, head_dim, page_size,
                window, split_keys, max_splits < 1 ? 1 : max_splits, scale};
@@ -246,6 +272,7 @@ extern "C" int mlr_paged_attention(
 // token is a group of one token.  Keys are walked in tiles of 32 at absolute multiples of 32; the four
 // wavefronts of the workgroup take the tiles t with t % 4 == wave, keep (max, sum, weighted values) each
 // and are merged in the order 0..3 at the end, so a column's sums depend on its own position only.
+// The loads of the next tile are issued before the current one is computed.
 //
 // Per tile, with v_mfma_f32_16x16x32_bf16 (D = A x B, a lane holds row/column lane % 16 and the eight
 // k-slots (lane / 16, 0..7) of A and of B):
@@ -256,14 +283,30 @@ extern "C" int mlr_paged_attention(
 //                                                         which already sit in B's register layout:
 //                                                         k-slot (b, e) is key 4b + e of the first 16 keys
 //                                                         for e < 4 and key 4b + e - 4 of the second 16.
+//
+// With key splits (max_splits > 1) every workgroup that holds keys writes its partial result and
+// `attention_combine_kernel` merges them (a second launch: on this GPU partial results of other
+// workgroups become visible cheaply at a kernel's end only).
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 
 #define MFMA_TILE_KEYS 32
 
+template <int NCH>
+struct KvTile {
+    bf16x8 k[2][NCH];
+    bf16x4 v[2 * NCH][2];
+    bool ok[2];
+    int tb;
+};
+
+struct TilePages {
+    int page[2];
+};
+
 template <int NCH>   // ceil(head_dim / 32)
-__global__ __launch_bounds__(256) void attention_mfma_kernel(AttnArgs a, const int32_t* __restrict__ group_row0,
+__global__ __launch_bounds__(256, (NCH <= 4 ? 2 : 1)) void attention_mfma_kernel(AttnArgs a, const int32_t* __restrict__ group_row0,
                                                              const int32_t* __restrict__ group_ntok) {
     extern __shared__ float lds[];
     const int D = a.head_dim, P = a.page_size;
@@ -277,10 +320,13 @@ __global__ __launch_bounds__(256) void attention_mfma_kernel(AttnArgs a, const i
     const bool col_valid = tok < ntok;
     const int kend_c = col_valid ? pos0 + tok + 1 : 0;
     int kbegin_c = a.window > 0 ? max(0, kend_c - a.window) : 0;
-    int lo = a.window > 0 ? max(0, pos0 + 1 - a.window) : 0;      // the group's key range
-    const int ke = pos0 + ntok;                                     // keys below ke are written
-    int hi = ke;
+    const int glo = a.window > 0 ? max(0, pos0 + 1 - a.window) : 0;   // the group's key range [glo, ke)
+    const int ke = pos0 + ntok;                                         // keys below ke are written
+    int lo = glo, hi = ke;
     if (a.max_splits > 1) {
+        const int first_split = glo / a.split_keys;
+        const int last_split = min(a.max_splits - 1, (ke - 1) / a.split_keys);
+        if (split < first_split || split > last_split) return;          // no keys here: the whole workgroup leaves
         lo = max(lo, split * a.split_keys);
         hi = min(hi, (split + 1) * a.split_keys);
     }
@@ -291,6 +337,8 @@ __global__ __launch_bounds__(256) void attention_mfma_kernel(AttnArgs a, const i
     const __bf16* kp_base = reinterpret_cast<const __bf16*>(a.k_pages);
     const __bf16* vp_base = reinterpret_cast<const __bf16*>(a.v_pages);
     const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+    const bf16x4 zero4 = {0, 0, 0, 0};
+    const int32_t* table = a.block_table + (size_t)slot * a.max_blocks;
 
     bf16x8 qf[NCH];
 #pragma unroll
@@ -306,34 +354,45 @@ __global__ __launch_bounds__(256) void attention_mfma_kernel(AttnArgs a, const i
 #pragma unroll
     for (int i = 0; i < 2 * NCH; ++i) o[i] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-    const int32_t* table = a.block_table + (size_t)slot * a.max_blocks;
-    for (int t = lo / MFMA_TILE_KEYS + wave; t * MFMA_TILE_KEYS < hi; t += 4) {
-        const int tb = t * MFMA_TILE_KEYS;
-        bool sub_ok[2];
-        size_t kbase[2], vbase[2];
+    auto lookup = [&](int t) {
+        TilePages tp;
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
-            const int key0 = tb + 16 * j;
-            sub_ok[j] = key0 < ke;
-            int page = -1;
-            if (sub_ok[j]) page = table[key0 / P];
-            sub_ok[j] = page >= 0;
-            const size_t pk = (size_t)(page < 0 ? 0 : page) * a.kv_heads + kvh;
-            kbase[j] = (pk * P + key0 % P) * D;
-            vbase[j] = pk * D * P + key0 % P;
+            const int key0 = t * MFMA_TILE_KEYS + 16 * j;
+            tp.page[j] = (key0 < hi) ? table[key0 / P] : -1;
         }
+        return tp;
+    };
+    auto load = [&](int t, const TilePages& tp, KvTile<NCH>& T) {
+        T.tb = t * MFMA_TILE_KEYS;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int key0 = T.tb + 16 * j;
+            T.ok[j] = tp.page[j] >= 0;
+            const size_t pk = (size_t)(T.ok[j] ? tp.page[j] : 0) * a.kv_heads + kvh;
+            const __bf16* kptr = kp_base + (pk * P + key0 % P + col) * D + 8 * b;
+            const __bf16* vptr = vp_base + pk * D * P + key0 % P + (size_t)col * P + 4 * b;
+#pragma unroll
+            for (int c = 0; c < NCH; ++c) {
+                T.k[j][c] = zero8;
+                if (T.ok[j] && 32 * c + 8 * b < D) T.k[j][c] = *reinterpret_cast<const bf16x8*>(kptr + 32 * c);
+            }
+#pragma unroll
+            for (int db = 0; db < 2 * NCH; ++db) {
+                T.v[db][j] = zero4;
+                if (T.ok[j] && 16 * db < D) T.v[db][j] = *reinterpret_cast<const bf16x4*>(vptr + (size_t)16 * db * P);
+            }
+        }
+    };
+    auto compute = [&](KvTile<NCH>& T) {
         floatx4 s[2];
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             s[j] = floatx4{0.f, 0.f, 0.f, 0.f};
-            if (sub_ok[j]) {
+            if (T.ok[j]) {
 #pragma unroll
-                for (int c = 0; c < NCH; ++c) {
-                    const int d0 = 32 * c + 8 * b;
-                    bf16x8 kf = zero8;
-                    if (d0 < D) kf = *reinterpret_cast<const bf16x8*>(kp_base + kbase[j] + (size_t)col * D + d0);
-                    s[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[c], s[j], 0, 0, 0);
-                }
+                for (int c = 0; c < NCH; ++c)
+                    s[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(T.k[j][c], qf[c], s[j], 0, 0, 0);
             }
         }
         // this lane: keys tb + 16 j + 4 b + r of column `col`
@@ -343,8 +402,8 @@ __global__ __launch_bounds__(256) void attention_mfma_kernel(AttnArgs a, const i
         for (int j = 0; j < 2; ++j)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const int key = tb + 16 * j + 4 * b + r;
-                const bool ok = sub_ok[j] && key >= kbegin_c && key < kstop_c;
+                const int key = T.tb + 16 * j + 4 * b + r;
+                const bool ok = T.ok[j] && key >= kbegin_c && key < kstop_c;
                 sv[j][r] = ok ? s[j][r] * a.scale : -INFINITY;
                 tile_max = fmaxf(tile_max, sv[j][r]);
             }
@@ -367,33 +426,55 @@ __global__ __launch_bounds__(256) void attention_mfma_kernel(AttnArgs a, const i
             l_run = l_run * corr + psum;
             m_run = m_new;
         }
-        const bool tail = tb + MFMA_TILE_KEYS > ke;      // some keys of the tile are not written yet
+        const bool tail = T.tb + MFMA_TILE_KEYS > ke;  // some keys of the tile are not written yet
 #pragma unroll
         for (int db = 0; db < 2 * NCH; ++db) {
             if (16 * db >= D) break;
             o[db] *= corr;
-            const int d = 16 * db + col;                  // here `col` is the channel row of A
-            bf16x8 vf = zero8;
+            bf16x8 vf;
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
-                if (!sub_ok[j]) continue;
-                bf16x4 v4 = *reinterpret_cast<const bf16x4*>(vp_base + vbase[j] + (size_t)d * P + 4 * b);
+                bf16x4 v4 = T.v[db][j];
                 if (tail) {
 #pragma unroll
                     for (int r = 0; r < 4; ++r)
-                        if (tb + 16 * j + 4 * b + r >= ke) v4[r] = (__bf16)0.f;
+                        if (T.tb + 16 * j + 4 * b + r >= ke) v4[r] = (__bf16)0.f;
                 }
 #pragma unroll
                 for (int r = 0; r < 4; ++r) vf[4 * j + r] = v4[r];
             }
             o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, o[db], 0, 0, 0);
         }
+    };
+
+    {
+        KvTile<NCH> ta, tb2;
+        int t = lo / MFMA_TILE_KEYS + wave;
+        const int t_end = (hi + MFMA_TILE_KEYS - 1) / MFMA_TILE_KEYS;
+        if (t < t_end) {
+            TilePages pa = lookup(t);
+            TilePages pb = lookup(t + 4);
+            load(t, pa, ta);
+            for (;;) {
+                const bool more_b = t + 4 < t_end;
+                pa = lookup(t + 8);
+                if (more_b) load(t + 4, pb, tb2);
+                compute(ta);
+                if (!more_b) break;
+                const bool more_a = t + 8 < t_end;
+                pb = lookup(t + 12);
+                if (more_a) load(t + 8, pa, ta);
+                compute(tb2);
+                if (!more_a) break;
+                t += 8;
+            }
+        }
     }
     // per column: the four lane blocks hold partial sums of the same column
     l_run += __shfl_xor(l_run, 16, MLR_WAVE);
     l_run += __shfl_xor(l_run, 32, MLR_WAVE);
 
-    // merge the wavefronts: 1..3 park their state in LDS, 0 merges in ascending order and writes
+    // merge the wavefronts: 1..3 park their state in LDS, 0 merges in ascending order
     const int stride = 16 * D + 32;                        // floats per wavefront: out^T [D][16], max[16], sum[16]
     if (wave > 0) {
         float* dst = lds + (size_t)(wave - 1) * stride;
@@ -409,69 +490,72 @@ __global__ __launch_bounds__(256) void attention_mfma_kernel(AttnArgs a, const i
         }
     }
     __syncthreads();
-    if (wave != 0) return;
-    float m_tot = m_run;
-    for (int w = 0; w < 3; ++w) m_tot = fmaxf(m_tot, lds[(size_t)w * stride + 16 * D + col]);
-    float l_tot = 0.f;
-    float own = 0.f;
-    if (m_tot > -INFINITY) {
-        own = m_run > -INFINITY ? __expf(m_run - m_tot) : 0.f;
-        l_tot = l_run * own;
-    }
-#pragma unroll
-    for (int db = 0; db < 2 * NCH; ++db) o[db] *= own;
-    for (int w = 0; w < 3; ++w) {
-        const float* src = lds + (size_t)w * stride;
-        const float mw = src[16 * D + col];
-        if (!(mw > -INFINITY)) continue;
-        const float f = __expf(mw - m_tot);
-        l_tot += src[16 * D + 16 + col] * f;
-#pragma unroll
-        for (int db = 0; db < 2 * NCH; ++db) {
-            if (16 * db >= D) break;
-#pragma unroll
-            for (int r = 0; r < 4; ++r) o[db][r] += src[(16 * db + 4 * b + r) * 16 + col] * f;
-        }
-    }
-    if (!col_valid) return;
     const size_t out_row = (size_t)(row0 + tok) * a.q_heads + kvh * g + hh;
-    if (a.max_splits > 1) {
-        float* dst = a.partial + (out_row * a.max_splits + split) * (D + 2);
-#pragma unroll
-        for (int db = 0; db < 2 * NCH; ++db) {
-            if (16 * db >= D) break;
-#pragma unroll
-            for (int r = 0; r < 4; ++r) dst[16 * db + 4 * b + r] = o[db][r];
+    if (wave == 0) {
+        float m_tot = m_run;
+        for (int w = 0; w < 3; ++w) m_tot = fmaxf(m_tot, lds[(size_t)w * stride + 16 * D + col]);
+        float l_tot = 0.f;
+        float own = 0.f;
+        if (m_tot > -INFINITY) {
+            own = m_run > -INFINITY ? __expf(m_run - m_tot) : 0.f;
+            l_tot = l_run * own;
         }
-        if (b == 0) {
-            dst[D] = m_tot;
-            dst[D + 1] = l_tot;
+#pragma unroll
+        for (int db = 0; db < 2 * NCH; ++db) o[db] *= own;
+        for (int w = 0; w < 3; ++w) {
+            const float* src = lds + (size_t)w * stride;
+            const float mw = src[16 * D + col];
+            if (!(mw > -INFINITY)) continue;
+            const float f = __expf(mw - m_tot);
+            l_tot += src[16 * D + 16 + col] * f;
+#pragma unroll
+            for (int db = 0; db < 2 * NCH; ++db) {
+                if (16 * db >= D) break;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) o[db][r] += src[(16 * db + 4 * b + r) * 16 + col] * f;
+            }
         }
-    } else {
-        __bf16* dst = reinterpret_cast<__bf16*>(a.out) + out_row * D;
+        if (col_valid) {
+            if (a.max_splits > 1) {
+                float* dst = a.partial + (out_row * a.max_splits + split) * (D + 2);
 #pragma unroll
-        for (int db = 0; db < 2 * NCH; ++db) {
-            if (16 * db >= D) break;
-            bf16x4 w4;
+                for (int db = 0; db < 2 * NCH; ++db) {
+                    if (16 * db >= D) break;
 #pragma unroll
-            for (int r = 0; r < 4; ++r) w4[r] = (__bf16)(l_tot > 0.f ? o[db][r] / l_tot : 0.f);
-            *reinterpret_cast<bf16x4*>(dst + 16 * db + 4 * b) = w4;
+                    for (int r = 0; r < 4; ++r) dst[16 * db + 4 * b + r] = o[db][r];
+                }
+                if (b == 0) {
+                    dst[D] = m_tot;
+                    dst[D + 1] = l_tot;
+                }
+            } else {
+                __bf16* dst = reinterpret_cast<__bf16*>(a.out) + out_row * D;
+#pragma unroll
+                for (int db = 0; db < 2 * NCH; ++db) {
+                    if (16 * db >= D) break;
+                    bf16x4 w4;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) w4[r] = (__bf16)(l_tot > 0.f ? o[db][r] / l_tot : 0.f);
+                    *reinterpret_cast<bf16x4*>(dst + 16 * db + 4 * b) = w4;
+                }
+            }
         }
     }
 }
 
 // Groups: group_row0[i] = first batch row of group i, group_ntok[i] = its tokens (consecutive rows of one
-// request, ntok * (q_heads / kv_heads) <= 16); together the groups cover the batch rows 0 .. rows - 1.  Needs page_size % 16 == 0, head_dim % 16 == 0,
-// q_heads / kv_heads <= 16.
+// request, ntok * (q_heads / kv_heads) <= 16); together the groups cover the batch rows 0 .. rows - 1.
+// Needs page_size % 16 == 0, head_dim % 16 == 0, q_heads / kv_heads <= 16.
 extern "C" int mlr_attention_mfma(
     const void* q, const void* k_pages, const void* v_pages, const int32_t* block_table, int max_blocks,
-    const int32_t* slots, const int32_t* positions, void* out, float* partial, const int32_t* group_row0,
-    const int32_t* group_ntok, int groups, int rows, int q_heads, int kv_heads, int head_dim, int page_size,
-    int window, float scale, int split_keys, int max_splits, hipStream_t stream) {
+    const int32_t* slots, const int32_t* positions, void* out, float* partial,
+    const int32_t* group_row0, const int32_t* group_ntok, int groups, int rows, int q_heads, int kv_heads,
+    int head_dim, int page_size, int window, float scale, int split_keys, int max_splits, hipStream_t stream) {
     if (groups <= 0 || rows <= 0) return 0;
     if (head_dim % 16 != 0 || head_dim > 256 || page_size % 16 != 0 || q_heads % kv_heads != 0 ||
         q_heads / kv_heads > 16) return -1;
-    if (max_splits > 1 && (partial == nullptr || split_keys <= 0 || split_keys % MFMA_TILE_KEYS != 0)) return -2;
+    if (max_splits > 1 && (partial == nullptr || split_keys <= 0 || split_keys % MFMA_TILE_KEYS != 0 ||
+                           max_splits > COMBINE_MAX_SPLITS)) return -2;
     AttnArgs a{(const elem_t*)q, (const elem_t*)k_pages, (const elem_t*)v_pages, block_table, slots,
                positions, (elem_t*)out, partial, max_blocks, q_heads, kv_heads, head_dim, page_size,
                window, split_keys, max_splits < 1 ? 1 : max_splits, scale};
@@ -492,7 +576,8 @@ extern "C" int mlr_attention_mfma(
     if (err != 0) return err;
     if (a.max_splits > 1) {
         attention_combine_kernel<<<dim3(rows, q_heads), 64, 0, stream>>>(a);   // the groups cover rows 0 .. rows - 1
+        err = (int)hipGetLastError();
     }
-    return (int)hipGetLastError();
+    return err;
 }
 #endif

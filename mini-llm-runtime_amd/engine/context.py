@@ -24,8 +24,18 @@ class Workspace:
             self._buffers[key] = buf
         return buf[:count].view(shape)
 
-    def reserve(self, name, shape, dtype):
-        self.get(name, shape, dtype)
+    def get_zeroed(self, name, shape, dtype):
+        """As `get`, for buffers whose users leave them zero after use (counters): the memory is zeroed
+        when it is allocated, never afterwards."""
+        count = 1
+        for extent in shape:
+            count *= int(extent)
+        key = (name, dtype)
+        buf = self._buffers.get(key)
+        if buf is None or buf.numel() < count:
+            buf = torch.zeros(max(count, 1), dtype=dtype, device=self.device)
+            self._buffers[key] = buf
+        return buf[:count].view(shape)
 
     def bytes(self):
         return sum(b.numel() * b.element_size() for b in self._buffers.values())
@@ -66,6 +76,7 @@ class StepContext:
         self.kernels, self.cache, self.workspace, self.dtype = kernels, cache, workspace, dtype
         self.max_positions = max_positions
         self.split_keys, self.split_max_tokens = split_keys, split_max_tokens
+        self.target_workgroups = 512      # about two workgroups per compute unit
         self.n_tokens = 0
         self.token_ids = self.positions = self.slots = None
         self.segments = []            # (slot, first row, number of tokens, first position)
@@ -100,12 +111,27 @@ class StepContext:
         self._groups[tokens_per_group] = hit
         return hit
 
-    def attention_split(self, rows, q_heads, head_dim):
-        """(split_keys, max_splits, partial buffer): small batches over long contexts split the
-        keys of a token over several workgroups.  The splits are ranges of absolute key
-        positions, so what a token's result is does not depend on this choice beyond rounding."""
-        if self.split_keys <= 0 or rows > self.split_max_tokens or self.max_context <= self.split_keys:
+    def attention_split(self, rows, kv_heads, q_heads, head_dim):
+        """(split_keys, max_splits, partial buffer).  A batch of many tokens fills the GPU with one
+        workgroup per (token group, kv head); a small batch over long contexts does not, so there the
+        keys of a token are split over several workgroups, in ranges [s * split_keys, (s + 1) *
+        split_keys) of absolute key positions, and merged in ascending order.  split_keys is the
+        largest of base, 2 base, 4 base, ... that still gives `target_workgroups`; what a token's
+        result is does not depend on the choice beyond rounding."""
+        base = self.split_keys
+        if base <= 0 or rows > self.split_max_tokens or self.max_context <= base:
             return 0, 1, None
-        max_splits = (self.max_context + self.split_keys - 1) // self.split_keys
+        units = max(1, rows * kv_heads)
+        keys = base
+        while keys * 2 < self.max_context and units * (-(-self.max_context // (keys * 2))) >= self.target_workgroups:
+            keys *= 2
+        if units >= self.target_workgroups:
+            return 0, 1, None
+        max_splits = -(-self.max_context // keys)
+        if max_splits <= 1:
+            return 0, 1, None
+        while max_splits > 1024:                     # the merge kernel's limit
+            keys *= 2
+            max_splits = -(-self.max_context // keys)
         numel = self.kernels.attention_partial_numel(rows, q_heads, head_dim, max_splits)
-        return self.split_keys, max_splits, self.workspace.get("attn_partial", (numel,), torch.float32)
+        return keys, max_splits, self.workspace.get("attn_partial", (numel,), torch.float32)

@@ -21,6 +21,7 @@ _ptr = ctypes.c_void_p
 
 MAX_HEAD_DIM = 256          # the attention and rotation kernels keep head_dim / 64 values per lane
 ATTENTION_TILE_KEYS = 64
+MAX_KEY_SPLITS = 1024         # the merge of key splits keeps one weight per split in LDS
 
 
 class KernelError(RuntimeError):
@@ -209,7 +210,8 @@ class Kernels:
             _need(partial.numel() >= self.attention_partial_numel(m, q_heads, head_dim, max_splits),
                   "partial buffer too small")
             group = q_heads // kv_heads
-            _need(((group + 7) // 8) * max_splits <= 65535, "too many key splits for the grid")
+            _need(((group + 7) // 8) * max_splits <= 65535 and max_splits <= MAX_KEY_SPLITS,
+                  "too many key splits for the grid")
         fn = self._lib("attention").mlr_paged_attention
         _ok(fn(_p(q), _p(k_pages), _p(v_pages), _p(block_table), _c_int(block_table.shape[1]), _p(slots),
                _p(positions), _p(out), _p(partial), _c_int(m), _c_int(q_heads), _c_int(kv_heads),
@@ -241,7 +243,7 @@ class Kernels:
         _tensor(positions, "positions", torch.int32, (m,))
         _tensor(group_row0, "group_row0", torch.int32, (groups,))
         _tensor(group_ntok, "group_ntok", torch.int32, (groups,))
-        _need(kv_heads <= 65535 and max_splits <= 65535, "too many kv heads or key splits for the grid")
+        _need(kv_heads <= 65535 and max_splits <= MAX_KEY_SPLITS, "too many kv heads or key splits for the grid")
         if max_splits > 1:
             _need(split_keys > 0 and split_keys % ATTENTION_TILE_KEYS == 0,
                   f"split_keys must be a multiple of {ATTENTION_TILE_KEYS}")

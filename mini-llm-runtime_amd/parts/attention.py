@@ -77,7 +77,7 @@ class GqaAttention:
             self.q_norm.eps if self.q_norm is not None else 0.0, rope,
             s.q_heads, s.kv_heads, s.head_dim, view.page_size, write_cache)
         attn = ctx.workspace.get("attn", (m, s.q_heads * s.head_dim), x.dtype)
-        split_keys, max_splits, partial = ctx.attention_split(m, s.q_heads, s.head_dim)
+        split_keys, max_splits, partial = ctx.attention_split(m, s.kv_heads, s.q_heads, s.head_dim)
         if k.mfma_attention_supported(s.q_heads, s.kv_heads, s.head_dim, view.page_size):
             first, count, groups = ctx.token_groups(max(1, 16 // (s.q_heads // s.kv_heads)))
             k.attention_mfma(q, view.k_pages, view.v_pages, view.block_table, ctx.slots, ctx.positions, attn,
