@@ -167,40 +167,53 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_bf16_kernel(
 }
 
 // Few rows (M <= 64): the weight is streamed once, straight from memory into the matrix cores.  A
-// workgroup owns 16 output columns (16 rows of w); its four wavefronts each take a quarter of k, and
-// their partial sums are added in the order 0..3, so the result does not depend on M.  The weight
+// workgroup owns 16 output columns (16 rows of w); its eight wavefronts each take an eighth of k, and
+// their partial sums are added in the order 0..7, so the result does not depend on M.  The weight
 // is the A operand (rows n), the activation the B operand (columns m): a lane ends up with four
 // consecutive n of one m.
-template <int MT, bool OUT_FLOAT>
-__global__ __launch_bounds__(256) void gemm_skinny_kernel(const __bf16* __restrict__ a,
-                                                          const __bf16* __restrict__ w,
-                                                          void* __restrict__ out_raw, int M, int N, int K) {
-    __shared__ float part[3][MT][64][4];
+// GATED: w holds two stacked matrices [gate; up] of N rows each; the workgroup computes the same 16
+// columns of both and writes silu(gate) * up (the feed-forward's activation fused into the projection).
+#define SKINNY_WAVES 8
+template <int MT, bool OUT_FLOAT, bool GATED>
+__global__ __launch_bounds__(SKINNY_WAVES * 64) void gemm_skinny_kernel(const __bf16* __restrict__ a,
+                                                                         const __bf16* __restrict__ w,
+                                                                         void* __restrict__ out_raw, int M, int N,
+                                                                         int K) {
+    constexpr int NW = GATED ? 2 : 1;
+    __shared__ float part[SKINNY_WAVES - 1][NW][MT][64][4];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r16 = lane & 15, b = lane >> 4;
     const int n0 = blockIdx.x * 16;
     const bool vector_ok = (K % 8) == 0;
     const int steps = (K + 31) / 32;
-    const int per_wave = (steps + 3) / 4;
+    const int per_wave = (steps + SKINNY_WAVES - 1) / SKINNY_WAVES;
     const int s_begin = wave * per_wave, s_end = min(steps, s_begin + per_wave);
-    floatx4 acc[MT];
+    floatx4 acc[NW][MT];
 #pragma unroll
-    for (int i = 0; i < MT; ++i) acc[i] = floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int g = 0; g < NW; ++g)
+#pragma unroll
+        for (int i = 0; i < MT; ++i) acc[g][i] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll 4
     for (int s = s_begin; s < s_end; ++s) {
         const int k = s * 32 + b * 8;
-        const bf16x8 wf = load_k8(w, n0 + r16, N, k, K, vector_ok);
+        bf16x8 wf[NW];
+#pragma unroll
+        for (int g = 0; g < NW; ++g) wf[g] = load_k8(w + (size_t)g * N * K, n0 + r16, N, k, K, vector_ok);
 #pragma unroll
         for (int i = 0; i < MT; ++i) {
             const bf16x8 xf = load_k8(a, 16 * i + r16, M, k, K, vector_ok);
-            acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, xf, acc[i], 0, 0, 0);
+#pragma unroll
+            for (int g = 0; g < NW; ++g)
+                acc[g][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[g], xf, acc[g][i], 0, 0, 0);
         }
     }
     if (wave > 0) {
 #pragma unroll
-        for (int i = 0; i < MT; ++i)
+        for (int g = 0; g < NW; ++g)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) part[wave - 1][i][lane][r] = acc[i][r];
+            for (int i = 0; i < MT; ++i)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) part[wave - 1][g][i][lane][r] = acc[g][i][r];
     }
     __syncthreads();
     if (wave != 0) return;
@@ -209,25 +222,33 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const __bf16* __restri
         const int m = 16 * i + r16;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            float v = acc[i][r];
-            for (int p = 0; p < 3; ++p) v += part[p][i][lane][r];
+            float v[NW];
+#pragma unroll
+            for (int g = 0; g < NW; ++g) {
+                v[g] = acc[g][i][r];
+                for (int p = 0; p < SKINNY_WAVES - 1; ++p) v[g] += part[p][g][i][lane][r];
+            }
+            float y = v[0];
+            if (GATED) y = (v[0] / (1.0f + expf(-v[0]))) * v[NW - 1];
             const int n = n0 + 4 * b + r;
             if (m < M && n < N) {
-                if (OUT_FLOAT) ((float*)out_raw)[(size_t)m * N + n] = v;
-                else ((__bf16*)out_raw)[(size_t)m * N + n] = (__bf16)v;
+                if (OUT_FLOAT) ((float*)out_raw)[(size_t)m * N + n] = y;
+                else ((__bf16*)out_raw)[(size_t)m * N + n] = (__bf16)y;
             }
         }
     }
 }
 
-template <int MT>
+template <int MT, bool GATED>
 static int launch_skinny(const void* a, const void* w, void* out, int M, int N, int K, int out_float,
                          hipStream_t stream) {
     dim3 grid((N + 15) / 16);
     if (out_float)
-        gemm_skinny_kernel<MT, true><<<grid, 256, 0, stream>>>((const __bf16*)a, (const __bf16*)w, out, M, N, K);
+        gemm_skinny_kernel<MT, true, GATED><<<grid, SKINNY_WAVES * 64, 0, stream>>>(
+            (const __bf16*)a, (const __bf16*)w, out, M, N, K);
     else
-        gemm_skinny_kernel<MT, false><<<grid, 256, 0, stream>>>((const __bf16*)a, (const __bf16*)w, out, M, N, K);
+        gemm_skinny_kernel<MT, false, GATED><<<grid, SKINNY_WAVES * 64, 0, stream>>>(
+            (const __bf16*)a, (const __bf16*)w, out, M, N, K);
     return (int)hipGetLastError();
 }
 
@@ -250,10 +271,23 @@ extern "C" int mlr_gemm(const void* a, const void* w, void* out, int M, int N, i
                         hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
     if (K <= 0) return -1;
-    if (M <= 16) return launch_skinny<1>(a, w, out, M, N, K, out_float, stream);
-    if (M <= 32) return launch_skinny<2>(a, w, out, M, N, K, out_float, stream);
-    if (M <= 64) return launch_skinny<4>(a, w, out, M, N, K, out_float, stream);
+    if (M <= 16) return launch_skinny<1, false>(a, w, out, M, N, K, out_float, stream);
+    if (M <= 32) return launch_skinny<2, false>(a, w, out, M, N, K, out_float, stream);
+    if (M <= 64) return launch_skinny<4, false>(a, w, out, M, N, K, out_float, stream);
     if (M <= 128) return launch<2, 2, 2, 2>(a, w, out, M, N, K, out_float, stream);  // 64 x 64
     return launch<2, 2, 4, 4>(a, w, out, M, N, K, out_float, stream);                // 128 x 128
+}
+
+// out[M, N] = silu(a . w[0:N]^T) * (a . w[N:2N]^T) for M <= 64 (w is [2N, K]: gate rows, then up rows).
+// Returns 1 when M is too large for this kernel: the caller then runs the projection and the
+// activation separately.
+extern "C" int mlr_gemm_gated_silu(const void* a, const void* w, void* out, int M, int N, int K,
+                                   hipStream_t stream) {
+    if (M <= 0 || N <= 0) return 0;
+    if (K <= 0) return -1;
+    if (M <= 16) return launch_skinny<1, true>(a, w, out, M, N, K, 0, stream);
+    if (M <= 32) return launch_skinny<2, true>(a, w, out, M, N, K, 0, stream);
+    if (M <= 64) return launch_skinny<4, true>(a, w, out, M, N, K, 0, stream);
+    return 1;
 }
 #endif

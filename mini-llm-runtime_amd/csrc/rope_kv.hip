@@ -18,7 +18,8 @@ __global__ void qk_norm_rope_kv_kernel(
     const float* __restrict__ rope, int q_heads, int kv_heads, int head_dim, int page_size,
     int write_cache) {
     const int m = blockIdx.x;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
+    const int lane = threadIdx.x & 63, waves = gridDim.y * (blockDim.x >> 6);
+    const int wave = blockIdx.y * (blockDim.x >> 6) + (threadIdx.x >> 6);       // heads are dealt out to these
     const int half = head_dim >> 1;
     const int pos = positions[m];
     const int slot = slots[m];
@@ -102,7 +103,12 @@ extern "C" int mlr_qk_norm_rope_kv(
     int head_dim, int page_size, int write_cache, hipStream_t stream) {
     if (rows <= 0) return 0;
     if (head_dim % 2 != 0 || head_dim / 2 > 64 * MAX_PAIRS) return -1;
-    qk_norm_rope_kv_kernel<<<rows, 256, 0, stream>>>(
+    // few rows: spread a row's heads over several workgroups (a wavefront per head)
+    const int total_heads = q_heads + 2 * kv_heads;
+    int chunks = 1;
+    if (rows < 512) chunks = (total_heads + 3) / 4;
+    if (chunks > 64) chunks = 64;
+    qk_norm_rope_kv_kernel<<<dim3(rows, chunks), 256, 0, stream>>>(
         (const elem_t*)qkv, ld, (elem_t*)q_out, (elem_t*)k_pages, (elem_t*)v_pages, block_table,
         max_blocks, slots, positions, q_norm_w, k_norm_w, eps, rope, q_heads, kv_heads, head_dim,
         page_size, write_cache);

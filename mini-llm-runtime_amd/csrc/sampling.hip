@@ -1,31 +1,44 @@
-// Token choice from float logits, one workgroup per row:
+// Token choice from float logits:
 //   temperature <= 0: the largest logit, ties -> lowest id;
 //   temperature  > 0: inverse-CDF draw from softmax(logits / T) with the uniform number u[r]
 //                     that the host derived from the request's own generator state.
 // A row that holds a NaN or an infinity gives token -1 and sets status[0] |= 1,
-// status[1] = min(status[1], row).  Max, exponentials and sums are 32-bit; every thread owns
-// a contiguous range of the vocabulary and all sums run in ascending order, so a row's
-// token depends on that row only.
+// status[1] = min(status[1], row).  Max, exponentials and sums are 32-bit.
+//
+// A row is cut into CHUNKS equal ranges of the vocabulary, one workgroup each, so that a few rows
+// still fill the GPU; inside a workgroup every thread owns a contiguous sub-range.  All sums run in
+// ascending order of the vocabulary and the cut depends on the vocabulary size only, so a row's token
+// depends on that row only.
+//   pass 1 (rows x CHUNKS): max, first argmax and a non-finite flag per chunk;
+//   pass 2 (rows): row max and argmax; greedy rows are done here;
+//   pass 3 (rows x CHUNKS, only if some row samples): sum of exp((x - max) / T) per chunk;
+//   pass 4 (rows): scan of the chunk sums, the chunk that holds u * total, then the token inside it.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
-#define THREADS 1024
+#define CHUNKS 64
+#define THREADS 256
 
-__global__ __launch_bounds__(THREADS) void sample_kernel(const float* __restrict__ logits, int vocab,
-                                                         const float* __restrict__ temperature,
-                                                         const float* __restrict__ uniform,
-                                                         int32_t* __restrict__ tokens,
-                                                         int32_t* __restrict__ status) {
+__device__ __forceinline__ void chunk_range(int vocab, int chunk, int* begin, int* end) {
+    const int per = (vocab + CHUNKS - 1) / CHUNKS;
+    *begin = min(vocab, chunk * per);
+    *end = min(vocab, *begin + per);
+}
+
+__global__ __launch_bounds__(THREADS) void chunk_max_kernel(const float* __restrict__ logits, int vocab,
+                                                            float* __restrict__ cmax, int32_t* __restrict__ cidx,
+                                                            int32_t* __restrict__ cbad) {
     __shared__ float vals[THREADS];
     __shared__ int idxs[THREADS];
-    __shared__ int bad, chosen;
-    const int r = blockIdx.x, t = threadIdx.x;
+    __shared__ int bad;
+    const int r = blockIdx.x, chunk = blockIdx.y, t = threadIdx.x;
     const float* row = logits + (size_t)r * vocab;
-    const int chunk = (vocab + THREADS - 1) / THREADS;
-    const int begin = min(vocab, t * chunk), end = min(vocab, begin + chunk);
-    if (t == 0) { bad = 0; chosen = -1; }
+    int cb, ce;
+    chunk_range(vocab, chunk, &cb, &ce);
+    const int per = (ce - cb + THREADS - 1) / THREADS;
+    const int begin = min(ce, cb + t * per), end = min(ce, begin + per);
+    if (t == 0) bad = 0;
     __syncthreads();
-
     float best = -INFINITY;
     int best_i = 0x7fffffff;
     bool nonfinite = false;
@@ -46,34 +59,107 @@ __global__ __launch_bounds__(THREADS) void sample_kernel(const float* __restrict
         }
         __syncthreads();
     }
-    const float row_max = vals[0];
-    const int arg = idxs[0];
+    if (t == 0) {
+        cmax[r * CHUNKS + chunk] = vals[0];
+        cidx[r * CHUNKS + chunk] = idxs[0];
+        cbad[r * CHUNKS + chunk] = bad;
+    }
+}
+
+// One wavefront per row: CHUNKS == 64 lanes.
+__global__ __launch_bounds__(64) void row_max_kernel(const float* __restrict__ cmax, const int32_t* __restrict__ cidx,
+                                                     const int32_t* __restrict__ cbad,
+                                                     const float* __restrict__ temperature,
+                                                     float* __restrict__ rmax, int32_t* __restrict__ tokens,
+                                                     int32_t* __restrict__ status) {
+    const int r = blockIdx.x, lane = threadIdx.x;
+    float v = cmax[r * CHUNKS + lane];
+    int i = cidx[r * CHUNKS + lane];
+    int bad = cbad[r * CHUNKS + lane];
+    for (int off = 32; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(v, off, 64);
+        const int oi = __shfl_xor(i, off, 64);
+        bad |= __shfl_xor(bad, off, 64);
+        if (ov > v || (ov == v && oi < i)) { v = ov; i = oi; }
+    }
+    if (lane != 0) return;
+    rmax[r] = v;
     if (bad) {
-        if (t == 0) {
-            tokens[r] = -1;
-            atomicOr(&status[0], 1);
-            atomicMin(&status[1], r);
-        }
-        return;
+        tokens[r] = -1;
+        atomicOr(&status[0], 1);
+        atomicMin(&status[1], r);
+    } else {
+        tokens[r] = i;                              // sampling rows overwrite this in pass 4
     }
-    const float temp = temperature ? temperature[r] : 0.f;
-    if (!(temp > 0.f)) {
-        if (t == 0) tokens[r] = arg;
-        return;
-    }
-    __syncthreads();
-    const float inv_t = 1.0f / temp;
+}
+
+__global__ __launch_bounds__(THREADS) void chunk_sum_kernel(const float* __restrict__ logits, int vocab,
+                                                            const float* __restrict__ temperature,
+                                                            const float* __restrict__ rmax,
+                                                            float* __restrict__ csum) {
+    __shared__ float vals[THREADS];
+    const int r = blockIdx.x, chunk = blockIdx.y, t = threadIdx.x;
+    const float temp = temperature[r];
+    if (!(temp > 0.f)) return;
+    const float* row = logits + (size_t)r * vocab;
+    int cb, ce;
+    chunk_range(vocab, chunk, &cb, &ce);
+    const int per = (ce - cb + THREADS - 1) / THREADS;
+    const int begin = min(ce, cb + t * per), end = min(ce, begin + per);
+    const float inv_t = 1.0f / temp, row_max = rmax[r];
     float sum = 0.f;
     for (int i = begin; i < end; ++i) sum += expf((row[i] - row_max) * inv_t);
     vals[t] = sum;
     __syncthreads();
-    if (t == 0) {                                   // inclusive scan in ascending order
+    if (t == 0) {                                   // ascending order
         float c = 0.f;
+        for (int i = 0; i < THREADS; ++i) c += vals[i];
+        csum[r * CHUNKS + chunk] = c;
+    }
+}
+
+__global__ __launch_bounds__(THREADS) void pick_kernel(const float* __restrict__ logits, int vocab,
+                                                       const float* __restrict__ temperature,
+                                                       const float* __restrict__ uniform,
+                                                       const float* __restrict__ rmax, const float* __restrict__ csum,
+                                                       int32_t* __restrict__ tokens) {
+    __shared__ float scan[CHUNKS];
+    __shared__ float vals[THREADS];
+    __shared__ int chosen_chunk, chosen;
+    __shared__ float chunk_lo;
+    const int r = blockIdx.x, t = threadIdx.x;
+    const float temp = temperature[r];
+    if (!(temp > 0.f) || tokens[r] < 0) return;     // greedy, or a row that is not finite
+    if (t == 0) {
+        float c = 0.f;
+        for (int i = 0; i < CHUNKS; ++i) { c += csum[r * CHUNKS + i]; scan[i] = c; }
+        const float target = uniform[r] * c;
+        int pick = -1;
+        for (int i = 0; i < CHUNKS; ++i)
+            if (target < scan[i] && csum[r * CHUNKS + i] > 0.f) { pick = i; break; }
+        chosen_chunk = pick;
+        chunk_lo = pick > 0 ? scan[pick - 1] : 0.f;
+        chosen = -1;
+    }
+    __syncthreads();
+    if (chosen_chunk < 0) return;                   // rounding pushed the target past the end: keep the argmax
+    const float target = uniform[r] * scan[CHUNKS - 1];
+    const float* row = logits + (size_t)r * vocab;
+    int cb, ce;
+    chunk_range(vocab, chosen_chunk, &cb, &ce);
+    const int per = (ce - cb + THREADS - 1) / THREADS;
+    const int begin = min(ce, cb + t * per), end = min(ce, begin + per);
+    const float inv_t = 1.0f / temp, row_max = rmax[r];
+    float sum = 0.f;
+    for (int i = begin; i < end; ++i) sum += expf((row[i] - row_max) * inv_t);
+    vals[t] = sum;
+    __syncthreads();
+    if (t == 0) {
+        float c = chunk_lo;
         for (int i = 0; i < THREADS; ++i) { c += vals[i]; vals[i] = c; }
     }
     __syncthreads();
-    const float target = uniform[r] * vals[THREADS - 1];
-    const float lo = t ? vals[t - 1] : 0.f, hi = vals[t];
+    const float lo = t ? vals[t - 1] : chunk_lo, hi = vals[t];
     if (target >= lo && target < hi && end > begin) {
         float c = lo;
         int pick = end - 1;
@@ -84,7 +170,7 @@ __global__ __launch_bounds__(THREADS) void sample_kernel(const float* __restrict
         chosen = pick;
     }
     __syncthreads();
-    if (t == 0) tokens[r] = chosen >= 0 ? chosen : arg;
+    if (t == 0 && chosen >= 0) tokens[r] = chosen;
 }
 
 __global__ void reset_status_kernel(int32_t* status) {
@@ -92,11 +178,27 @@ __global__ void reset_status_kernel(int32_t* status) {
     status[1] = 0x7fffffff;
 }
 
+extern "C" int mlr_sample_scratch_floats(int rows) { return rows * (2 * CHUNKS + 1); }
+extern "C" int mlr_sample_scratch_ints(int rows) { return rows * 2 * CHUNKS; }
+
+// scratch_f: rows * (2 CHUNKS + 1) floats; scratch_i: rows * 2 CHUNKS ints.  `any_sampling` = 0 skips
+// passes 3 and 4 (every temperature <= 0).
 extern "C" int mlr_sample(const float* logits, int rows, int vocab, const float* temperature,
-                          const float* uniform, int32_t* tokens, int32_t* status, hipStream_t stream) {
+                          const float* uniform, int32_t* tokens, int32_t* status, float* scratch_f,
+                          int32_t* scratch_i, int any_sampling, hipStream_t stream) {
     if (rows <= 0) return 0;
     if (vocab <= 0) return -1;
+    float* cmax = scratch_f;
+    float* csum = scratch_f + (size_t)rows * CHUNKS;
+    float* rmax = scratch_f + (size_t)rows * 2 * CHUNKS;
+    int32_t* cidx = scratch_i;
+    int32_t* cbad = scratch_i + (size_t)rows * CHUNKS;
     reset_status_kernel<<<1, 1, 0, stream>>>(status);
-    sample_kernel<<<rows, THREADS, 0, stream>>>(logits, vocab, temperature, uniform, tokens, status);
+    chunk_max_kernel<<<dim3(rows, CHUNKS), THREADS, 0, stream>>>(logits, vocab, cmax, cidx, cbad);
+    row_max_kernel<<<rows, 64, 0, stream>>>(cmax, cidx, cbad, temperature, rmax, tokens, status);
+    if (any_sampling) {
+        chunk_sum_kernel<<<dim3(rows, CHUNKS), THREADS, 0, stream>>>(logits, vocab, temperature, rmax, csum);
+        pick_kernel<<<rows, THREADS, 0, stream>>>(logits, vocab, temperature, uniform, rmax, csum, tokens);
+    }
     return (int)hipGetLastError();
 }

@@ -149,6 +149,22 @@ class Kernels:
         _ok(fn(_p(a), _p(w), _p(out), _c_int(m), _c_int(n), _c_int(k),
                _c_int(1 if out.dtype == torch.float32 else 0), _stream()), "gemm")
 
+    def gated_silu_fused(self, rows):
+        """Whether `gemm_gated_silu` serves this many rows (the bfloat16 engine, up to 64)."""
+        return self.dtype == torch.bfloat16 and rows <= 64
+
+    def gemm_gated_silu(self, a, w, out):
+        """out[M, N] = silu(a . w[:N]^T) * (a . w[N:]^T), w = [gate; up] stacked, for few rows."""
+        _need(self.gated_silu_fused(a.shape[0]), "gemm_gated_silu: bfloat16 and at most 64 rows")
+        _tensor(a, "a", self.dtype, ndim=2)
+        _tensor(w, "w", self.dtype, ndim=2)
+        m, k = a.shape
+        two_n, k2 = w.shape
+        _need(k == k2 and two_n % 2 == 0, "gemm_gated_silu: sizes do not fit")
+        _tensor(out, "out", self.dtype, (m, two_n // 2))
+        fn = self._lib("gemm").mlr_gemm_gated_silu
+        _ok(fn(_p(a), _p(w), _p(out), _c_int(m), _c_int(two_n // 2), _c_int(k), _stream()), "gemm_gated_silu")
+
     # -- attention ---------------------------------------------------------------------------
     def _check_cache(self, k_pages, v_pages, kv_heads, head_dim, page_size):
         _tensor(k_pages, "k_pages", self.dtype, ndim=4)
@@ -258,7 +274,12 @@ class Kernels:
                _c_float(scale), _c_int(split_keys), _c_int(max_splits), _stream()), "attention_mfma")
 
     # -- sampling ----------------------------------------------------------------------------
-    def sample(self, logits, temperature, uniform, tokens, status):
+    def sample_scratch(self, rows):
+        """(floats, ints) of scratch memory that `sample` needs for this many rows."""
+        lib = self._lib("sampling")
+        return lib.mlr_sample_scratch_floats(_c_int(rows)), lib.mlr_sample_scratch_ints(_c_int(rows))
+
+    def sample(self, logits, temperature, uniform, tokens, status, scratch_f, scratch_i, any_sampling=True):
         """tokens[r] = argmax (temperature <= 0) or the inverse-CDF draw at uniform[r]."""
         _tensor(logits, "logits", torch.float32, ndim=2)
         rows, vocab = logits.shape
@@ -266,6 +287,11 @@ class Kernels:
         _tensor(uniform, "uniform", torch.float32, (rows,))
         _tensor(tokens, "tokens", torch.int32, (rows,))
         _tensor(status, "status", torch.int32, (2,))
+        need_f, need_i = self.sample_scratch(rows)
+        _tensor(scratch_f, "scratch_f", torch.float32, ndim=1)
+        _tensor(scratch_i, "scratch_i", torch.int32, ndim=1)
+        _need(scratch_f.numel() >= need_f and scratch_i.numel() >= need_i, "sample: scratch buffers too small")
+        _need(rows <= 65535, "sample: too many rows for the grid")
         fn = self._lib("sampling").mlr_sample
         _ok(fn(_p(logits), _c_int(rows), _c_int(vocab), _p(temperature), _p(uniform), _p(tokens),
-               _p(status), _stream()), "sample")
+               _p(status), _p(scratch_f), _p(scratch_i), _c_int(1 if any_sampling else 0), _stream()), "sample")

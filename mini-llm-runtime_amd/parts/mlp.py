@@ -34,10 +34,13 @@ class SwiGluMlp:
     def forward(self, ctx, x):
         s = self.spec
         m = x.shape[0]
-        gate_up = ctx.workspace.get("gate_up", (m, 2 * s.intermediate), x.dtype)
-        ctx.kernels.gemm(x, self.gate_up, gate_up)
         act = ctx.workspace.get("act", (m, s.intermediate), x.dtype)
-        ctx.kernels.silu_mul(gate_up, act)
+        if ctx.kernels.gated_silu_fused(m):           # few rows: the activation rides on the projection
+            ctx.kernels.gemm_gated_silu(x, self.gate_up, act)
+        else:
+            gate_up = ctx.workspace.get("gate_up", (m, 2 * s.intermediate), x.dtype)
+            ctx.kernels.gemm(x, self.gate_up, gate_up)
+            ctx.kernels.silu_mul(gate_up, act)
         out = ctx.workspace.get("ffn_out", (m, s.hidden), x.dtype)
         ctx.kernels.gemm(act, self.down, out)
         return out

@@ -53,6 +53,9 @@ class Sampler:
         self._host = torch.empty((2, rows), dtype=torch.float32).pin_memory()
         self._tokens = torch.empty(rows, dtype=torch.int32, device=self.device)
         self._status = torch.zeros(2, dtype=torch.int32, device=self.device)
+        need_f, need_i = self.kernels.sample_scratch(rows)
+        self._scratch_f = torch.empty(need_f, dtype=torch.float32, device=self.device)
+        self._scratch_i = torch.empty(need_i, dtype=torch.int32, device=self.device)
 
     def sample(self, logits, temperatures, uniforms):
         """logits: float [R, V] on the device; per row a temperature (<= 0: greedy) and a uniform
@@ -68,7 +71,8 @@ class Sampler:
         temp = self._params[0, :rows]
         uni = self._params[1, :rows]
         tokens = self._tokens[:rows]
-        self.kernels.sample(logits, temp, uni, tokens, self._status)
+        self.kernels.sample(logits, temp, uni, tokens, self._status, self._scratch_f, self._scratch_i,
+                            any_sampling=any(t > 0 for t in temperatures))
         out = torch.cat([tokens, self._status]).cpu().tolist()     # one copy back, one sync
         if out[rows] != 0:
             raise NonFiniteLogits(f"row {out[rows + 1]} of the logits holds a value that is not finite")

@@ -21,6 +21,12 @@ def kernels(dtype):
     return Kernels(dtype)
 
 
+def sample(k, logits, temp, u, tokens, status):
+    need_f, need_i = k.sample_scratch(logits.shape[0])
+    k.sample(logits, temp, u, tokens, status, torch.empty(need_f, device="cuda"),
+             torch.empty(need_i, dtype=torch.int32, device="cuda"))
+
+
 def rnd(shape, dtype, seed, scale=1.0):
     g = torch.Generator().manual_seed(seed)
     return (scale * torch.randn(shape, generator=g)).to(dtype).cuda()
@@ -371,7 +377,7 @@ def test_sample_greedy(vocab):
     u = torch.zeros(4).cuda()
     tokens = torch.full((4,), -7, dtype=torch.int32).cuda()
     status = torch.zeros(2, dtype=torch.int32).cuda()
-    k.sample(logits.cuda(), temp, u, tokens, status)
+    sample(k, logits.cuda(), temp, u, tokens, status)
     got = tokens.cpu().tolist()
     for r in range(4):
         row = logits[r]
@@ -400,7 +406,7 @@ def test_sample_temperature(vocab):
     u[0], u[1] = 0.0, 0.9999999
     tokens = torch.empty(rows, dtype=torch.int32).cuda()
     status = torch.zeros(2, dtype=torch.int32).cuda()
-    k.sample(logits.cuda(), temp.cuda(), u.cuda(), tokens, status)
+    sample(k, logits.cuda(), temp.cuda(), u.cuda(), tokens, status)
     got = tokens.cpu().tolist()
     for r in range(rows):
         cdf = temperature_cdf(logits[r].numpy(), float(temp[r]))
@@ -418,8 +424,8 @@ def test_sample_frequencies():
     g = torch.Generator().manual_seed(5)
     u = torch.rand(rows, generator=g).cuda()
     tokens = torch.empty(rows, dtype=torch.int32).cuda()
-    k.sample(logits[None, :].repeat(rows, 1).cuda().contiguous(), torch.full((rows,), temp_value).cuda(), u, tokens,
-             torch.zeros(2, dtype=torch.int32).cuda())
+    sample(k, logits[None, :].repeat(rows, 1).cuda().contiguous(), torch.full((rows,), temp_value).cuda(), u, tokens,
+           torch.zeros(2, dtype=torch.int32).cuda())
     freq = torch.bincount(tokens.cpu().long(), minlength=7).double() / rows
     want = torch.softmax(logits.double() / temp_value, 0)
     assert (freq - want).abs().max() < 0.015
@@ -464,3 +470,20 @@ def test_attention_window_edge(dtype, window):
                              1, 1, 1, d, page, 1.0, window=window)
             torch.testing.assert_close(out.double().cpu(), want, **tol(dtype))
             assert bool((out.float().cpu()[0] - vv[hot].to(dtype).float()).abs().max() < 0.05) == inside
+
+
+@pytest.mark.parametrize("mnk", [(1, 48, 64), (8, 3072, 1024), (17, 100, 76), (40, 208, 80), (64, 136, 264)])
+def test_gemm_gated_silu(mnk):
+    """The feed-forward's activation fused into its first projection (few rows, bfloat16):
+    silu(a Wgate^T) * (a Wup^T) with the sums kept in 32-bit until the product."""
+    m, n, kk = mnk
+    k = kernels(torch.bfloat16)
+    assert k.gated_silu_fused(m) and not k.gated_silu_fused(65)
+    a = rnd((m, kk), torch.bfloat16, 50)
+    w = rnd((2 * n, kk), torch.bfloat16, 51, 0.3)
+    out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    k.gemm_gated_silu(a, w, out)
+    g = a.double() @ w.double()[:n].T
+    u = a.double() @ w.double()[n:].T
+    want = g / (1 + torch.exp(-g)) * u
+    torch.testing.assert_close(out.double(), want, atol=2e-2 * float(want.abs().max()), rtol=2e-2)

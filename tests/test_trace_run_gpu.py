@@ -67,7 +67,8 @@ def test_replay_matches_the_plain_implementation(model_folders, plain_models, tm
         got = replay(model_folders[name], dtype, part, max(peak, 128), out_dir, vocab)
         compare(got, want, dtype)
         got_all[label] = got
-    limit = 2e-5 if dtype == "float32" else 0.05
+    scale = max(float(np.abs(v).max()) for v in want.values())
+    limit = 2e-5 if dtype == "float32" else 0.03 * scale        # bfloat16: rounding between kernels for few and many rows
     for label in ("last32", "portions", "mixed"):
         assert max(np.abs(got_all["whole"][k] - got_all[label][k]).max() for k in want) <= limit
 
