@@ -21,6 +21,7 @@ _ptr = ctypes.c_void_p
 
 MAX_HEAD_DIM = 256          # the attention and rotation kernels keep head_dim / 64 values per lane
 ATTENTION_TILE_KEYS = 64
+LIBRARY_GEMM_MIN_ROWS = 64    # above this many rows the bfloat16 engine's projections go to the library
 MAX_KEY_SPLITS = 1024         # the merge of key splits keeps one weight per split in LDS
 
 
@@ -59,11 +60,12 @@ def _ok(code, what):
 
 
 class Kernels:
-    def __init__(self, dtype):
+    def __init__(self, dtype, library_gemm=True):
         _need(dtype in (torch.float32, torch.bfloat16), f"no kernels for element type {dtype}")
         if not torch.cuda.is_available():
             raise KernelError("no GPU is visible: the engine's kernels are HIP only")
         self.dtype = dtype
+        self.library_gemm = library_gemm
         self._libs = {}
 
     # -- libraries ---------------------------------------------------------------------------
@@ -145,6 +147,11 @@ class Kernels:
         _need(k == k2, f"gemm: inner sizes differ ({k} and {k2})")
         _need(out.dtype in (self.dtype, torch.float32), f"gemm: output type {out.dtype} not supported")
         _tensor(out, "out", out.dtype, (m, n))
+        if self.library_gemm and self.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and m > LIBRARY_GEMM_MIN_ROWS:
+            # many rows: a plain matrix product, handed to the vendor library (hipBLASLt through torch),
+            # as the reference hands its projections to cuBLAS (src/minillm/cuda/matrix.cpp:11-37)
+            torch.matmul(a, w.t(), out=out)
+            return
         fn = self._lib("gemm").mlr_gemm
         _ok(fn(_p(a), _p(w), _p(out), _c_int(m), _c_int(n), _c_int(k),
                _c_int(1 if out.dtype == torch.float32 else 0), _stream()), "gemm")

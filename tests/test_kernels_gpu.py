@@ -120,17 +120,19 @@ def test_silu_mul_and_residual(dtype):
                                  (33, 48, 520), (48, 1000, 264), (8, 6144, 1024), (129, 100, 40)])
 def test_gemm(dtype, mnk):
     """Odd shapes as in the reference's GEMM test (tests/cuda_unit_tests.cu:207-209)."""
+    from mini_llm_runtime_amd.kernels import Kernels
     m, n, kk = mnk
-    k = kernels(dtype)
     a = rnd((m, kk), dtype, 7)
     w = rnd((n, kk), dtype, 8)
     want = a.double() @ w.double().T
-    for out_dtype in {dtype, torch.float32}:
-        out = torch.full((m, n), float("nan"), dtype=out_dtype, device="cuda")
-        k.gemm(a, w, out)
-        t = dict(atol=1e-4 * math.sqrt(kk), rtol=1e-5) if out_dtype == torch.float32 else \
-            dict(atol=2e-2 * math.sqrt(kk) / 4, rtol=2e-2)
-        torch.testing.assert_close(out.double(), want, **t)
+    # the engine's choice (many rows of the bfloat16 engine go to the library) and the hand-written kernels alone
+    for k in (kernels(dtype), Kernels(dtype, library_gemm=False)):
+        for out_dtype in {dtype, torch.float32}:
+            out = torch.full((m, n), float("nan"), dtype=out_dtype, device="cuda")
+            k.gemm(a, w, out)
+            t = dict(atol=1e-4 * math.sqrt(kk), rtol=1e-5) if out_dtype == torch.float32 else \
+                dict(atol=2e-2 * math.sqrt(kk) / 4, rtol=2e-2)
+            torch.testing.assert_close(out.double(), want, **t)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -139,7 +141,8 @@ def test_gemm_rows_do_not_depend_on_the_batch(dtype):
     additions for every M; the bfloat16 engine has two kernels (up to 64 rows the weight is streamed with k
     split over four wavefronts, above that it is tiled), each with a fixed order, so bits agree within a
     kernel and differ by rounding across the two."""
-    k = kernels(dtype)
+    from mini_llm_runtime_amd.kernels import Kernels
+    k = Kernels(dtype, library_gemm=False)
     a = rnd((200, 264), dtype, 9)
     w = rnd((150, 264), dtype, 10)
 
