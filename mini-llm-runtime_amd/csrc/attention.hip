@@ -543,15 +543,257 @@ __global__ __launch_bounds__(256, (NCH <= 4 ? 2 : 1)) void attention_mfma_kernel
     }
 }
 
+// ------------------------------------------------------------------------------------------------
+// Prompt portions: a workgroup serves up to 4 * (16 / g) consecutive tokens of one request (each
+// wavefront 16 columns: 16 / g tokens times g heads).  All four wavefronts walk the same key tiles,
+// which are staged once per workgroup through LDS (double-buffered: the next tile's global loads are in
+// flight while the current one is multiplied), so keys and values are read from memory once per
+// workgroup instead of once per wavefront.  The arithmetic per column is that of
+// `attention_mfma_kernel` without key splits, tile by tile in ascending order.
+template <int NCH>
+__global__ __launch_bounds__(256) void attention_prefill_kernel(AttnArgs a, const int32_t* __restrict__ group_row0,
+                                                                const int32_t* __restrict__ group_ntok) {
+    constexpr int DMAX = 32 * NCH;
+    constexpr int KPITCH = DMAX + 8;                  // elements per key row in LDS
+    constexpr int VPITCH = 32 + 4;                    // elements per channel row in LDS
+    constexpr int STAGE = (NCH + 1) / 2;              // 16-byte chunks a thread stages per tile, for K and for V
+    __shared__ __attribute__((aligned(16))) __bf16 k_lds[2][32 * KPITCH];
+    __shared__ __attribute__((aligned(16))) __bf16 v_lds[2][DMAX * VPITCH];
+    const int D = a.head_dim, P = a.page_size;
+    const int g = a.q_heads / a.kv_heads, tq = 16 / g;
+    const int grp = blockIdx.x, kvh = blockIdx.y;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int col = lane & 15, b = lane >> 4;
+    const int row0 = group_row0[grp], ntok = group_ntok[grp];
+    const int slot = a.slots[row0], pos0 = a.positions[row0];
+    const int tok = wave * tq + col / g, hh = col % g;          // this lane's column: token within the group, head
+    const bool col_valid = col / g < tq && tok < ntok;
+    const int kend_c = col_valid ? pos0 + tok + 1 : 0;
+    const int kbegin_c = a.window > 0 ? max(0, kend_c - a.window) : 0;
+    const int lo = a.window > 0 ? max(0, pos0 + 1 - a.window) : 0;
+    const int ke = pos0 + ntok;
+    // this wavefront's own key range (its tokens wave * tq .. wave * tq + tq - 1)
+    const int wtok0 = wave * tq;
+    const bool wave_active = wtok0 < ntok;
+    const int wave_hi = wave_active ? pos0 + min(ntok, wtok0 + tq) : 0;
+    const int wave_lo = a.window > 0 ? max(0, pos0 + wtok0 + 1 - a.window) : 0;
+
+    const __bf16* q = reinterpret_cast<const __bf16*>(a.q);
+    const __bf16* kp_base = reinterpret_cast<const __bf16*>(a.k_pages);
+    const __bf16* vp_base = reinterpret_cast<const __bf16*>(a.v_pages);
+    const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+    const int32_t* table = a.block_table + (size_t)slot * a.max_blocks;
+
+    bf16x8 qf[NCH];
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) {
+        const int d0 = 32 * c + 8 * b;
+        qf[c] = zero8;
+        if (col_valid && d0 < D)
+            qf[c] = *reinterpret_cast<const bf16x8*>(q + ((size_t)(row0 + tok) * a.q_heads + kvh * g + hh) * D + d0);
+    }
+    float m_run = -INFINITY, l_run = 0.f;
+    floatx4 o[2 * NCH];
+#pragma unroll
+    for (int i = 0; i < 2 * NCH; ++i) o[i] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    const int kchunks = 4 * D;                         // 32 keys x D / 8
+    const int vchunks = 4 * D;                         // D channels x 32 keys / 8
+    bf16x8 kst[STAGE], vst[STAGE];
+    auto fetch = [&](int t) {                          // global -> registers
+        const int tb = t * MFMA_TILE_KEYS;
+        size_t kbase[2], vbase[2];
+        bool ok[2];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int key0 = tb + 16 * j;
+            const int page = key0 < ke ? table[key0 / P] : -1;
+            ok[j] = page >= 0;
+            const size_t pk = (size_t)(ok[j] ? page : 0) * a.kv_heads + kvh;
+            kbase[j] = (pk * P + key0 % P) * D;
+            vbase[j] = pk * D * P + key0 % P;
+        }
+#pragma unroll
+        for (int i = 0; i < STAGE; ++i) {
+            const int ci = threadIdx.x + 256 * i;
+            kst[i] = zero8;
+            vst[i] = zero8;
+            if (ci < kchunks) {
+                const int key = ci / (D / 8), c8 = ci % (D / 8);
+                const int j = key >> 4;
+                if (ok[j]) kst[i] = *reinterpret_cast<const bf16x8*>(kp_base + kbase[j] + (size_t)(key & 15) * D + 8 * c8);
+            }
+            if (ci < vchunks) {
+                const int d = ci >> 2, q4 = ci & 3, j = q4 >> 1, half = q4 & 1;
+                if (ok[j]) {
+                    bf16x8 v = *reinterpret_cast<const bf16x8*>(vp_base + vbase[j] + (size_t)d * P + 8 * half);
+                    const int key0 = tb + 16 * j + 8 * half;
+                    if (key0 + 8 > ke) {               // keys that are not written yet count as zero
+#pragma unroll
+                        for (int e = 0; e < 8; ++e)
+                            if (key0 + e >= ke) v[e] = (__bf16)0.f;
+                    }
+                    vst[i] = v;
+                }
+            }
+        }
+    };
+    auto stash = [&](int buf) {                        // registers -> LDS
+#pragma unroll
+        for (int i = 0; i < STAGE; ++i) {
+            const int ci = threadIdx.x + 256 * i;
+            if (ci < kchunks) {
+                const int key = ci / (D / 8), c8 = ci % (D / 8);
+                *reinterpret_cast<bf16x8*>(&k_lds[buf][key * KPITCH + 8 * c8]) = kst[i];
+            }
+            if (ci < vchunks) {
+                const int d = ci >> 2, q4 = ci & 3;
+                *reinterpret_cast<bf16x4*>(&v_lds[buf][d * VPITCH + 8 * q4]) = bf16x4{vst[i][0], vst[i][1], vst[i][2], vst[i][3]};
+                *reinterpret_cast<bf16x4*>(&v_lds[buf][d * VPITCH + 8 * q4 + 4]) = bf16x4{vst[i][4], vst[i][5], vst[i][6], vst[i][7]};
+            }
+        }
+    };
+
+    const int t_begin = lo / MFMA_TILE_KEYS, t_end = (ke + MFMA_TILE_KEYS - 1) / MFMA_TILE_KEYS;
+    fetch(t_begin);
+    int buf = 0;
+    for (int t = t_begin; t < t_end; ++t, buf ^= 1) {
+        stash(buf);
+        __syncthreads();
+        if (t + 1 < t_end) fetch(t + 1);
+        const int tb = t * MFMA_TILE_KEYS;
+        if (!wave_active || tb >= wave_hi || tb + MFMA_TILE_KEYS <= wave_lo) continue;   // nothing for this wavefront
+        floatx4 s[2];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            s[j] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int c = 0; c < NCH; ++c) {
+                // channels at and beyond head_dim were never staged: they must read as zero, not as whatever
+                // the LDS held (a NaN there would turn the whole score into NaN)
+                bf16x8 kf = zero8;
+                if (32 * c + 8 * b < D)
+                    kf = *reinterpret_cast<const bf16x8*>(&k_lds[buf][(16 * j + col) * KPITCH + 32 * c + 8 * b]);
+                s[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[c], s[j], 0, 0, 0);
+            }
+        }
+        float sv[2][4];
+        float tile_max = -INFINITY;
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int key = tb + 16 * j + 4 * b + r;
+                const bool ok = key >= kbegin_c && key < kend_c;
+                sv[j][r] = ok ? s[j][r] * a.scale : -INFINITY;
+                tile_max = fmaxf(tile_max, sv[j][r]);
+            }
+        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, MLR_WAVE));
+        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, MLR_WAVE));
+        const float m_new = fmaxf(m_run, tile_max);
+        float corr = 1.f;
+        bf16x8 pf = zero8;
+        if (m_new > -INFINITY) {
+            corr = __expf(m_run - m_new);
+            float psum = 0.f;
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const float p = sv[j][r] > -INFINITY ? __expf(sv[j][r] - m_new) : 0.f;
+                    psum += p;
+                    pf[4 * j + r] = (__bf16)p;
+                }
+            l_run = l_run * corr + psum;
+            m_run = m_new;
+        }
+#pragma unroll
+        for (int db = 0; db < 2 * NCH; ++db) {
+            if (16 * db >= D) break;
+            o[db] *= corr;
+            const __bf16* vrow = &v_lds[buf][(16 * db + col) * VPITCH];
+            const bf16x4 v0 = *reinterpret_cast<const bf16x4*>(vrow + 4 * b);
+            const bf16x4 v1 = *reinterpret_cast<const bf16x4*>(vrow + 16 + 4 * b);
+            const bf16x8 vf = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+            o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, o[db], 0, 0, 0);
+        }
+    }
+    l_run += __shfl_xor(l_run, 16, MLR_WAVE);
+    l_run += __shfl_xor(l_run, 32, MLR_WAVE);
+    if (!col_valid) return;
+    __bf16* dst = reinterpret_cast<__bf16*>(a.out) + ((size_t)(row0 + tok) * a.q_heads + kvh * g + hh) * D;
+#pragma unroll
+    for (int db = 0; db < 2 * NCH; ++db) {
+        if (16 * db >= D) break;
+        bf16x4 w4;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) w4[r] = (__bf16)(l_run > 0.f ? o[db][r] / l_run : 0.f);
+        *reinterpret_cast<bf16x4*>(dst + 16 * db + 4 * b) = w4;
+    }
+}
+
+// The merge of key splits for the groups of `attention_mfma_kernel` (one wavefront per (group, head),
+// walking the group's tokens).
+__global__ __launch_bounds__(64) void attention_combine_groups_kernel(AttnArgs a, const int32_t* __restrict__ group_row0,
+                                                                      const int32_t* __restrict__ group_ntok) {
+    __shared__ float w_lds[COMBINE_MAX_SPLITS];
+    __shared__ float l_lds[COMBINE_MAX_SPLITS];
+    const int grp = blockIdx.x, head = blockIdx.y;
+    const int D = a.head_dim;
+    for (int j = 0; j < group_ntok[grp]; ++j) {
+        const int m = group_row0[grp] + j;
+        const int pos = a.positions[m];
+        const int first = a.window > 0 ? max(0, pos + 1 - a.window) / a.split_keys : 0;
+        const int last = min(a.max_splits - 1, pos / a.split_keys);
+        const int n = last - first + 1;
+        const float* base = a.partial + (((size_t)m * a.q_heads + head) * a.max_splits + first) * (D + 2);
+        float gmax = -INFINITY;
+        __syncthreads();
+        for (int s = threadIdx.x; s < n; s += 64) {
+            const float smax = base[(size_t)s * (D + 2) + D];
+            w_lds[s] = smax;
+            l_lds[s] = base[(size_t)s * (D + 2) + D + 1];
+            gmax = fmaxf(gmax, smax);
+        }
+        gmax = wave_max(gmax);
+        __syncthreads();
+        for (int s = threadIdx.x; s < n; s += 64) {
+            const float smax = w_lds[s];
+            w_lds[s] = smax > -INFINITY ? __expf(smax - gmax) : 0.f;
+        }
+        __syncthreads();
+        float den = 0.f;
+        for (int s = 0; s < n; ++s) den += w_lds[s] * l_lds[s];
+        float num[MAX_DIM_REGS];
+#pragma unroll
+        for (int i = 0; i < MAX_DIM_REGS; ++i) num[i] = 0.f;
+        for (int s = 0; s < n; ++s) {
+            const float w = w_lds[s];
+            const float* p = base + (size_t)s * (D + 2);
+#pragma unroll
+            for (int i = 0; i < MAX_DIM_REGS; ++i) {
+                const int d = threadIdx.x + 64 * i;
+                if (d < D) num[i] += w * p[d];
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < MAX_DIM_REGS; ++i) {
+            const int d = threadIdx.x + 64 * i;
+            if (d < D) a.out[((size_t)m * a.q_heads + head) * D + d] = from_float<elem_t>(den > 0.f ? num[i] / den : 0.f);
+        }
+    }
+}
+
 // Groups: group_row0[i] = first batch row of group i, group_ntok[i] = its tokens (consecutive rows of one
-// request, ntok * (q_heads / kv_heads) <= 16); together the groups cover the batch rows 0 .. rows - 1.
+// request, ntok * (q_heads / kv_heads) <= 16).  Rows outside the groups are left alone.
 // Needs page_size % 16 == 0, head_dim % 16 == 0, q_heads / kv_heads <= 16.
 extern "C" int mlr_attention_mfma(
     const void* q, const void* k_pages, const void* v_pages, const int32_t* block_table, int max_blocks,
     const int32_t* slots, const int32_t* positions, void* out, float* partial,
     const int32_t* group_row0, const int32_t* group_ntok, int groups, int rows, int q_heads, int kv_heads,
     int head_dim, int page_size, int window, float scale, int split_keys, int max_splits, hipStream_t stream) {
-    if (groups <= 0 || rows <= 0) return 0;
+    (void)rows;
+    if (groups <= 0) return 0;
     if (head_dim % 16 != 0 || head_dim > 256 || page_size % 16 != 0 || q_heads % kv_heads != 0 ||
         q_heads / kv_heads > 16) return -1;
     if (max_splits > 1 && (partial == nullptr || split_keys <= 0 || split_keys % MFMA_TILE_KEYS != 0 ||
@@ -575,9 +817,36 @@ extern "C" int mlr_attention_mfma(
     int err = (int)hipGetLastError();
     if (err != 0) return err;
     if (a.max_splits > 1) {
-        attention_combine_kernel<<<dim3(rows, q_heads), 64, 0, stream>>>(a);   // the groups cover rows 0 .. rows - 1
+        attention_combine_groups_kernel<<<dim3(groups, q_heads), 64, 0, stream>>>(a, group_row0, group_ntok);
         err = (int)hipGetLastError();
     }
     return err;
+}
+
+// Prompt portions: groups of up to 4 * (16 / g) consecutive tokens of one request each, no key splits.
+extern "C" int mlr_attention_prefill(
+    const void* q, const void* k_pages, const void* v_pages, const int32_t* block_table, int max_blocks,
+    const int32_t* slots, const int32_t* positions, void* out, const int32_t* group_row0,
+    const int32_t* group_ntok, int groups, int q_heads, int kv_heads, int head_dim, int page_size, int window,
+    float scale, hipStream_t stream) {
+    if (groups <= 0) return 0;
+    if (head_dim % 16 != 0 || head_dim > 256 || page_size % 16 != 0 || q_heads % kv_heads != 0 ||
+        q_heads / kv_heads > 16) return -1;
+    AttnArgs a{(const elem_t*)q, (const elem_t*)k_pages, (const elem_t*)v_pages, block_table, slots,
+               positions, (elem_t*)out, nullptr, max_blocks, q_heads, kv_heads, head_dim, page_size,
+               window, 0, 1, scale};
+    dim3 grid(groups, kv_heads);
+    const int nch = (head_dim + 31) / 32;
+    switch (nch) {
+        case 1: attention_prefill_kernel<1><<<grid, 256, 0, stream>>>(a, group_row0, group_ntok); break;
+        case 2: attention_prefill_kernel<2><<<grid, 256, 0, stream>>>(a, group_row0, group_ntok); break;
+        case 3: attention_prefill_kernel<3><<<grid, 256, 0, stream>>>(a, group_row0, group_ntok); break;
+        case 4: attention_prefill_kernel<4><<<grid, 256, 0, stream>>>(a, group_row0, group_ntok); break;
+        case 5: attention_prefill_kernel<5><<<grid, 256, 0, stream>>>(a, group_row0, group_ntok); break;
+        case 6: attention_prefill_kernel<6><<<grid, 256, 0, stream>>>(a, group_row0, group_ntok); break;
+        case 7: attention_prefill_kernel<7><<<grid, 256, 0, stream>>>(a, group_row0, group_ntok); break;
+        default: attention_prefill_kernel<8><<<grid, 256, 0, stream>>>(a, group_row0, group_ntok); break;
+    }
+    return (int)hipGetLastError();
 }
 #endif

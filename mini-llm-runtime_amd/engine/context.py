@@ -89,35 +89,48 @@ class StepContext:
         self._groups = {}
         self.single_token_groups = None
 
-    def token_groups(self, tokens_per_group):
-        """The step's rows cut into groups of at most `tokens_per_group` consecutive tokens of one request:
-        (first row of each group, tokens in each group) as device int32 vectors, and their number."""
-        hit = self._groups.get(tokens_per_group)
+    def token_groups(self, tokens_per_group, big_factor=0):
+        """The step's rows cut into groups of consecutive tokens of one request, as device int32 vectors
+        (first row of each group, tokens in each group) with their number.  Returns (small, big, rows in
+        small groups): small groups hold at most `tokens_per_group` tokens; with big_factor > 0, a request
+        that brings more than `tokens_per_group` tokens is cut into big groups of at most big_factor *
+        tokens_per_group instead (prompt portions), else `big` is empty."""
+        key = (tokens_per_group, big_factor)
+        hit = self._groups.get(key)
         if hit is not None:
             return hit
         if self.single_token_groups is not None:      # a step of single tokens with fixed buffers
-            return self.single_token_groups
-        first, count = [], []
+            return self.single_token_groups, (None, None, 0), self.n_tokens
+        first, count, big_first, big_count = [], [], [], []
+        small_rows = 0
         for _, row, n, _ in self.segments:
-            for i in range(0, n, tokens_per_group):
-                first.append(row + i)
-                count.append(min(tokens_per_group, n - i))
-        g = len(first)
-        dev = self.workspace.get(f"token_groups_{tokens_per_group}", (2 * g,), torch.int32)
+            if big_factor > 0 and n > tokens_per_group:
+                size = big_factor * tokens_per_group
+                for i in range(0, n, size):
+                    big_first.append(row + i)
+                    big_count.append(min(size, n - i))
+            else:
+                small_rows += n
+                for i in range(0, n, tokens_per_group):
+                    first.append(row + i)
+                    count.append(min(tokens_per_group, n - i))
+        g, gb = len(first), len(big_first)
+        dev = self.workspace.get(f"token_groups_{tokens_per_group}_{big_factor}", (2 * (g + gb),), torch.int32)
         if self._group_upload is None:
             self._group_upload = Uploader(4096, dev.device)
-        self._group_upload.send(first + count, dev)
-        hit = (dev[:g], dev[g:2 * g], g)
-        self._groups[tokens_per_group] = hit
+        self._group_upload.send(first + count + big_first + big_count, dev)
+        hit = ((dev[:g], dev[g:2 * g], g), (dev[2 * g:2 * g + gb], dev[2 * g + gb:2 * g + 2 * gb], gb), small_rows)
+        self._groups[key] = hit
         return hit
 
-    def attention_split(self, rows, kv_heads, q_heads, head_dim):
+    def attention_split(self, rows, batch_rows, kv_heads, q_heads, head_dim):
         """(split_keys, max_splits, partial buffer).  A batch of many tokens fills the GPU with one
         workgroup per (token group, kv head); a small batch over long contexts does not, so there the
         keys of a token are split over several workgroups, in ranges [s * split_keys, (s + 1) *
         split_keys) of absolute key positions, and merged in ascending order.  split_keys is the
         largest of base, 2 base, 4 base, ... that still gives `target_workgroups`; what a token's
-        result is does not depend on the choice beyond rounding."""
+        result is does not depend on the choice beyond rounding.  `rows` tokens take part; the partial
+        results are indexed by batch row, of which there are `batch_rows`."""
         base = self.split_keys
         if base <= 0 or rows > self.split_max_tokens or self.max_context <= base:
             return 0, 1, None
@@ -133,5 +146,5 @@ class StepContext:
         while max_splits > 1024:                     # the merge kernel's limit
             keys *= 2
             max_splits = -(-self.max_context // keys)
-        numel = self.kernels.attention_partial_numel(rows, q_heads, head_dim, max_splits)
+        numel = self.kernels.attention_partial_numel(batch_rows, q_heads, head_dim, max_splits)
         return keys, max_splits, self.workspace.get("attn_partial", (numel,), torch.float32)

@@ -92,7 +92,7 @@ class Runner:
         ctx.token_ids, ctx.positions, ctx.slots = meta[0:n], meta[n:2 * n], meta[2 * n:3 * n]
         ctx.segments = [(e.slot, i, 1, p0) for i, (e, p0) in enumerate(zip(entries, first))]
         ctx.max_context = self.max_length                 # the graph must serve every later context
-        ctx.single_token_groups = (meta[4 * n:5 * n], meta[5 * n:6 * n], n)
+        ctx.single_token_groups = (meta[4 * n:5 * n], meta[5 * n:6 * n], n)        # groups of one token each
         want_rows = meta[3 * n:4 * n]
         state["runs"] += 1
         if state["runs"] == 1:                            # first time: eager, sizes the scratch buffers

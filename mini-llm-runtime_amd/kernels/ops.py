@@ -280,6 +280,33 @@ class Kernels:
                _c_int(q_heads), _c_int(kv_heads), _c_int(head_dim), _c_int(page_size), _c_int(window or 0),
                _c_float(scale), _c_int(split_keys), _c_int(max_splits), _stream()), "attention_mfma")
 
+    def prefill_attention_supported(self, q_heads, kv_heads, head_dim, page_size):
+        """The LDS-staged kernel for prompt portions: as the matrix-core kernel, head sizes up to 224."""
+        return self.mfma_attention_supported(q_heads, kv_heads, head_dim, page_size) and head_dim <= 224
+
+    def attention_prefill(self, q, k_pages, v_pages, block_table, slots, positions, out, group_row0, group_ntok,
+                          groups, q_heads, kv_heads, head_dim, page_size, scale, window=None):
+        """Attention for prompt portions: groups of up to 4 * (16 // (q_heads // kv_heads)) consecutive rows
+        of one request each; keys and values of a group are staged once through LDS."""
+        _need(self.prefill_attention_supported(q_heads, kv_heads, head_dim, page_size),
+              "attention_prefill: sizes not supported")
+        _tensor(q, "q", self.dtype, ndim=2)
+        m = q.shape[0]
+        _need(q.shape[1] == q_heads * head_dim, "q: wrong width")
+        _tensor(out, "out", self.dtype, (m, q_heads * head_dim))
+        self._check_cache(k_pages, v_pages, kv_heads, head_dim, page_size)
+        _tensor(block_table, "block_table", torch.int32, ndim=2)
+        _tensor(slots, "slots", torch.int32, (m,))
+        _tensor(positions, "positions", torch.int32, (m,))
+        _tensor(group_row0, "group_row0", torch.int32, (groups,))
+        _tensor(group_ntok, "group_ntok", torch.int32, (groups,))
+        _need(kv_heads <= 65535, "too many kv heads for the grid")
+        fn = self._lib("attention").mlr_attention_prefill
+        _ok(fn(_p(q), _p(k_pages), _p(v_pages), _p(block_table), _c_int(block_table.shape[1]), _p(slots),
+               _p(positions), _p(out), _p(group_row0), _p(group_ntok), _c_int(groups), _c_int(q_heads),
+               _c_int(kv_heads), _c_int(head_dim), _c_int(page_size), _c_int(window or 0), _c_float(scale),
+               _stream()), "attention_prefill")
+
     # -- sampling ----------------------------------------------------------------------------
     def sample_scratch(self, rows):
         """(floats, ints) of scratch memory that `sample` needs for this many rows."""

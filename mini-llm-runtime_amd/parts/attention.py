@@ -77,14 +77,23 @@ class GqaAttention:
             self.q_norm.eps if self.q_norm is not None else 0.0, rope,
             s.q_heads, s.kv_heads, s.head_dim, view.page_size, write_cache)
         attn = ctx.workspace.get("attn", (m, s.q_heads * s.head_dim), x.dtype)
-        split_keys, max_splits, partial = ctx.attention_split(m, s.kv_heads, s.q_heads, s.head_dim)
         if k.mfma_attention_supported(s.q_heads, s.kv_heads, s.head_dim, view.page_size):
-            first, count, groups = ctx.token_groups(max(1, 16 // (s.q_heads // s.kv_heads)))
-            k.attention_mfma(q, view.k_pages, view.v_pages, view.block_table, ctx.slots, ctx.positions, attn,
-                             first, count, groups, s.q_heads, s.kv_heads, s.head_dim, view.page_size,
-                             float(s.scale), window=s.window, split_keys=split_keys, max_splits=max_splits,
-                             partial=partial)
+            # prompt portions go to the LDS-staged kernel, single tokens and short portions to the one
+            # that can split a token's keys over workgroups
+            big_factor = 4 if k.prefill_attention_supported(s.q_heads, s.kv_heads, s.head_dim, view.page_size) else 0
+            small, big, small_rows = ctx.token_groups(max(1, 16 // (s.q_heads // s.kv_heads)), big_factor)
+            if big[2]:
+                k.attention_prefill(q, view.k_pages, view.v_pages, view.block_table, ctx.slots, ctx.positions, attn,
+                                    big[0], big[1], big[2], s.q_heads, s.kv_heads, s.head_dim, view.page_size,
+                                    float(s.scale), window=s.window)
+            if small[2]:
+                split_keys, max_splits, partial = ctx.attention_split(small_rows, m, s.kv_heads, s.q_heads, s.head_dim)
+                k.attention_mfma(q, view.k_pages, view.v_pages, view.block_table, ctx.slots, ctx.positions, attn,
+                                 small[0], small[1], small[2], s.q_heads, s.kv_heads, s.head_dim, view.page_size,
+                                 float(s.scale), window=s.window, split_keys=split_keys, max_splits=max_splits,
+                                 partial=partial)
         else:
+            split_keys, max_splits, partial = ctx.attention_split(m, m, s.kv_heads, s.q_heads, s.head_dim)
             k.paged_attention(q, view.k_pages, view.v_pages, view.block_table, ctx.slots, ctx.positions, attn,
                               s.q_heads, s.kv_heads, s.head_dim, view.page_size, float(s.scale),
                               window=s.window, split_keys=split_keys, max_splits=max_splits, partial=partial)

@@ -260,6 +260,9 @@ def plain_attention(q, keys, values, scale, window):
     (6, 3, 48, 32, [100, 70], None, 0),
     (32, 2, 64, 16, [130, 5], None, 64),
     (8, 8, 80, 16, [77], 40, 0),
+    (16, 8, 128, 16, [530, 3], None, 0),
+    (4, 1, 96, 32, [150], 50, 0),
+    (14, 2, 224, 16, [40], None, 0),
 ])
 def test_paged_attention(dtype, case):
     """Every length is one request whose LAST token is the query (a decoded token) plus, for the
@@ -322,6 +325,20 @@ def test_paged_attention(dtype, case):
     got = out2.double().cpu().view(m, hq, d)
     for i in range(m):
         torch.testing.assert_close(got[i], wants[i], **tol(dtype))
+    if not k.prefill_attention_supported(hq, hkv, d, page):
+        return
+    # the kernel for prompt portions: the first request's rows in groups of up to 4 tq tokens; other rows untouched
+    big = 4 * tq
+    first = list(range(0, lengths[0], big))
+    count = [min(big, lengths[0] - r) for r in first]
+    out3 = torch.full((m, hq * d), float("nan"), dtype=dtype, device="cuda")
+    k.attention_prefill(q.view(m, hq * d).cuda(), k_pages.cuda(), v_pages.cuda(), table.cuda(), slots, pos, out3,
+                        torch.tensor(first, dtype=torch.int32).cuda(), torch.tensor(count, dtype=torch.int32).cuda(),
+                        len(first), hq, hkv, d, page, scale, window=window)
+    got = out3.double().cpu().view(m, hq, d)
+    for i in range(lengths[0]):
+        torch.testing.assert_close(got[i], wants[i], **tol(dtype))
+    assert torch.isnan(out3[lengths[0]:].float()).all()
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
