@@ -550,6 +550,7 @@ __global__ __launch_bounds__(256, (NCH <= 4 ? 2 : 1)) void attention_mfma_kernel
 // flight while the current one is multiplied), so keys and values are read from memory once per
 // workgroup instead of once per wavefront.  The arithmetic per column is that of
 // `attention_mfma_kernel` without key splits, tile by tile in ascending order.
+#define PAGE_CACHE 2048
 template <int NCH>
 __global__ __launch_bounds__(256) void attention_prefill_kernel(AttnArgs a, const int32_t* __restrict__ group_row0,
                                                                 const int32_t* __restrict__ group_ntok) {
@@ -559,6 +560,7 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(AttnArgs a, cons
     constexpr int STAGE = (NCH + 1) / 2;              // 16-byte chunks a thread stages per tile, for K and for V
     __shared__ __attribute__((aligned(16))) __bf16 k_lds[2][32 * KPITCH];
     __shared__ __attribute__((aligned(16))) __bf16 v_lds[2][DMAX * VPITCH];
+    __shared__ int32_t page_lds[PAGE_CACHE];          // the request's page ids for this group's key range
     const int D = a.head_dim, P = a.page_size;
     const int g = a.q_heads / a.kv_heads, tq = 16 / g;
     const int grp = blockIdx.x, kvh = blockIdx.y;
@@ -597,72 +599,72 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(AttnArgs a, cons
 #pragma unroll
     for (int i = 0; i < 2 * NCH; ++i) o[i] = floatx4{0.f, 0.f, 0.f, 0.f};
 
+    // page ids first: looked up in LDS, a tile's loads do not have to wait for a load of the block table
+    // (the first tile starts at the multiple of 32 at or below lo, so the cache starts at that key's page)
+    const int first_page = (lo / MFMA_TILE_KEYS) * MFMA_TILE_KEYS / P;
+    {
+        const int n_pages = min(PAGE_CACHE, (ke + P - 1) / P - first_page);
+        for (int i = threadIdx.x; i < n_pages; i += 256) page_lds[i] = table[first_page + i];
+        __syncthreads();
+    }
     const int kchunks = 4 * D;                         // 32 keys x D / 8
     const int vchunks = 4 * D;                         // D channels x 32 keys / 8
-    bf16x8 kst[STAGE], vst[STAGE];
-    auto fetch = [&](int t) {                          // global -> registers
+    struct Staged {
+        bf16x8 k[STAGE], v[STAGE];
+        int tb;
+        int ok;                                        // bit j: the page of keys tb + 16 j .. is mapped
+    };                                                 // (no array indexed at run time: that would live in scratch)
+    // global -> registers.  No branch around a load: a load behind a branch makes the compiler wait for
+    // every load in flight.  Addresses are clamped to valid memory (page 0 for a missing page, the last
+    // chunk for a thread without one); what must read as zero is zeroed when the registers go to LDS.
+    auto fetch = [&](int t, Staged& st) {
         const int tb = t * MFMA_TILE_KEYS;
-        size_t kbase[2], vbase[2];
-        bool ok[2];
+        st.tb = tb;
+        st.ok = 0;
+        size_t kbase0 = 0, kbase1 = 0, vbase0 = 0, vbase1 = 0;
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             const int key0 = tb + 16 * j;
-            const int page = key0 < ke ? table[key0 / P] : -1;
-            ok[j] = page >= 0;
-            const size_t pk = (size_t)(ok[j] ? page : 0) * a.kv_heads + kvh;
-            kbase[j] = (pk * P + key0 % P) * D;
-            vbase[j] = pk * D * P + key0 % P;
+            const int idx = min(max(key0 / P - first_page, 0), PAGE_CACHE - 1);
+            const int page = key0 < ke ? page_lds[idx] : -1;       // the host keeps the group's pages within the cache
+            const bool ok = page >= 0;
+            st.ok |= (ok ? 1 : 0) << j;
+            const size_t pk = (size_t)(ok ? page : 0) * a.kv_heads + kvh;
+            const size_t kb = (pk * P + key0 % P) * D, vb = pk * D * P + key0 % P;
+            if (j == 0) { kbase0 = kb; vbase0 = vb; } else { kbase1 = kb; vbase1 = vb; }
         }
 #pragma unroll
         for (int i = 0; i < STAGE; ++i) {
-            const int ci = threadIdx.x + 256 * i;
-            kst[i] = zero8;
-            vst[i] = zero8;
-            if (ci < kchunks) {
-                const int key = ci / (D / 8), c8 = ci % (D / 8);
-                const int j = key >> 4;
-                if (ok[j]) kst[i] = *reinterpret_cast<const bf16x8*>(kp_base + kbase[j] + (size_t)(key & 15) * D + 8 * c8);
-            }
-            if (ci < vchunks) {
-                const int d = ci >> 2, q4 = ci & 3, j = q4 >> 1, half = q4 & 1;
-                if (ok[j]) {
-                    bf16x8 v = *reinterpret_cast<const bf16x8*>(vp_base + vbase[j] + (size_t)d * P + 8 * half);
-                    const int key0 = tb + 16 * j + 8 * half;
-                    if (key0 + 8 > ke) {               // keys that are not written yet count as zero
-#pragma unroll
-                        for (int e = 0; e < 8; ++e)
-                            if (key0 + e >= ke) v[e] = (__bf16)0.f;
-                    }
-                    vst[i] = v;
-                }
-            }
+            const int ci = min((int)threadIdx.x + 256 * i, kchunks - 1);
+            const int key = ci / (D / 8), c8 = ci % (D / 8);
+            st.k[i] = *reinterpret_cast<const bf16x8*>(kp_base + ((key >> 4) ? kbase1 : kbase0) + (size_t)(key & 15) * D + 8 * c8);
+            const int d = ci >> 2, q4 = ci & 3;
+            st.v[i] = *reinterpret_cast<const bf16x8*>(vp_base + ((q4 >> 1) ? vbase1 : vbase0) + (size_t)d * P + 8 * (q4 & 1));
         }
     };
-    auto stash = [&](int buf) {                        // registers -> LDS
+    auto stash = [&](int buf, const Staged& st) {      // registers -> LDS
 #pragma unroll
         for (int i = 0; i < STAGE; ++i) {
             const int ci = threadIdx.x + 256 * i;
-            if (ci < kchunks) {
-                const int key = ci / (D / 8), c8 = ci % (D / 8);
-                *reinterpret_cast<bf16x8*>(&k_lds[buf][key * KPITCH + 8 * c8]) = kst[i];
+            if (ci >= kchunks) continue;
+            const int key = ci / (D / 8), c8 = ci % (D / 8);
+            *reinterpret_cast<bf16x8*>(&k_lds[buf][key * KPITCH + 8 * c8]) = ((st.ok >> (key >> 4)) & 1) ? st.k[i] : zero8;
+            const int d = ci >> 2, q4 = ci & 3, j = q4 >> 1;
+            bf16x8 v = ((st.ok >> j) & 1) ? st.v[i] : zero8;
+            const int key0 = st.tb + 16 * j + 8 * (q4 & 1);
+            if (key0 + 8 > ke) {                       // keys that are not written yet count as zero
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    if (key0 + e >= ke) v[e] = (__bf16)0.f;
             }
-            if (ci < vchunks) {
-                const int d = ci >> 2, q4 = ci & 3;
-                *reinterpret_cast<bf16x4*>(&v_lds[buf][d * VPITCH + 8 * q4]) = bf16x4{vst[i][0], vst[i][1], vst[i][2], vst[i][3]};
-                *reinterpret_cast<bf16x4*>(&v_lds[buf][d * VPITCH + 8 * q4 + 4]) = bf16x4{vst[i][4], vst[i][5], vst[i][6], vst[i][7]};
-            }
+            *reinterpret_cast<bf16x4*>(&v_lds[buf][d * VPITCH + 8 * q4]) = bf16x4{v[0], v[1], v[2], v[3]};
+            *reinterpret_cast<bf16x4*>(&v_lds[buf][d * VPITCH + 8 * q4 + 4]) = bf16x4{v[4], v[5], v[6], v[7]};
         }
     };
 
-    const int t_begin = lo / MFMA_TILE_KEYS, t_end = (ke + MFMA_TILE_KEYS - 1) / MFMA_TILE_KEYS;
-    fetch(t_begin);
-    int buf = 0;
-    for (int t = t_begin; t < t_end; ++t, buf ^= 1) {
-        stash(buf);
-        __syncthreads();
-        if (t + 1 < t_end) fetch(t + 1);
+    auto compute = [&](int t, int buf) {
         const int tb = t * MFMA_TILE_KEYS;
-        if (!wave_active || tb >= wave_hi || tb + MFMA_TILE_KEYS <= wave_lo) continue;   // nothing for this wavefront
+        if (!wave_active || tb >= wave_hi || tb + MFMA_TILE_KEYS <= wave_lo) return;     // nothing for this wavefront
         floatx4 s[2];
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
@@ -717,6 +719,37 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(AttnArgs a, cons
             const bf16x8 vf = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
             o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, o[db], 0, 0, 0);
         }
+    };
+
+    // Three tiles are under way at any time: one being multiplied out of LDS, two in flight from memory
+    // into registers.  One barrier per tile suffices with two LDS buffers: a wavefront can only reach the
+    // second write of a buffer after the barrier that follows every wavefront's read of it.
+    const int t_begin = lo / MFMA_TILE_KEYS, t_end = (ke + MFMA_TILE_KEYS - 1) / MFMA_TILE_KEYS;
+    // (fetches are unconditional, clamped to the last tile: a fetch behind a branch would again make
+    // the compiler drain every load in flight)
+    Staged sa, sb, sc;
+    const int t_last = t_end - 1;
+    fetch(t_begin, sa);
+    fetch(min(t_begin + 1, t_last), sb);
+    int buf = 0;
+    for (int t = t_begin; t < t_end; t += 3) {
+        fetch(min(t + 2, t_last), sc);
+        stash(buf, sa);
+        __syncthreads();
+        compute(t, buf);
+        buf ^= 1;
+        if (t + 1 >= t_end) break;
+        fetch(min(t + 3, t_last), sa);
+        stash(buf, sb);
+        __syncthreads();
+        compute(t + 1, buf);
+        buf ^= 1;
+        if (t + 2 >= t_end) break;
+        fetch(min(t + 4, t_last), sb);
+        stash(buf, sc);
+        __syncthreads();
+        compute(t + 2, buf);
+        buf ^= 1;
     }
     l_run += __shfl_xor(l_run, 16, MLR_WAVE);
     l_run += __shfl_xor(l_run, 32, MLR_WAVE);
@@ -824,14 +857,16 @@ extern "C" int mlr_attention_mfma(
 }
 
 // Prompt portions: groups of up to 4 * (16 / g) consecutive tokens of one request each, no key splits.
+// A group's keys must span at most PAGE_CACHE (2048) pages: the caller sends longer contexts to
+// `mlr_attention_mfma`.
 extern "C" int mlr_attention_prefill(
     const void* q, const void* k_pages, const void* v_pages, const int32_t* block_table, int max_blocks,
     const int32_t* slots, const int32_t* positions, void* out, const int32_t* group_row0,
     const int32_t* group_ntok, int groups, int q_heads, int kv_heads, int head_dim, int page_size, int window,
     float scale, hipStream_t stream) {
     if (groups <= 0) return 0;
-    if (head_dim % 16 != 0 || head_dim > 256 || page_size % 16 != 0 || q_heads % kv_heads != 0 ||
-        q_heads / kv_heads > 16) return -1;
+    if (head_dim % 16 != 0 || head_dim > 192 || page_size % 16 != 0 || q_heads % kv_heads != 0 ||
+        q_heads / kv_heads > 16) return -1;            // 192: the two LDS tile buffers and the page ids fit 64 KB
     AttnArgs a{(const elem_t*)q, (const elem_t*)k_pages, (const elem_t*)v_pages, block_table, slots,
                positions, (elem_t*)out, nullptr, max_blocks, q_heads, kv_heads, head_dim, page_size,
                window, 0, 1, scale};
@@ -843,9 +878,7 @@ extern "C" int mlr_attention_prefill(
         case 3: attention_prefill_kernel<3><<<grid, 256, 0, stream>>>(a, group_row0, group_ntok); break;
         case 4: attention_prefill_kernel<4><<<grid, 256, 0, stream>>>(a, group_row0, group_ntok); break;
         case 5: attention_prefill_kernel<5><<<grid, 256, 0, stream>>>(a, group_row0, group_ntok); break;
-        case 6: attention_prefill_kernel<6><<<grid, 256, 0, stream>>>(a, group_row0, group_ntok); break;
-        case 7: attention_prefill_kernel<7><<<grid, 256, 0, stream>>>(a, group_row0, group_ntok); break;
-        default: attention_prefill_kernel<8><<<grid, 256, 0, stream>>>(a, group_row0, group_ntok); break;
+        default: attention_prefill_kernel<6><<<grid, 256, 0, stream>>>(a, group_row0, group_ntok); break;
     }
     return (int)hipGetLastError();
 }

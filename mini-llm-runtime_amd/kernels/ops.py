@@ -22,6 +22,7 @@ _ptr = ctypes.c_void_p
 MAX_HEAD_DIM = 256          # the attention and rotation kernels keep head_dim / 64 values per lane
 ATTENTION_TILE_KEYS = 64
 LIBRARY_GEMM_MIN_ROWS = 64    # above this many rows the bfloat16 engine's projections go to the library
+PREFILL_MAX_PAGES = 2048      # page ids of one group that the prompt-portion attention kernel keeps in LDS
 MAX_KEY_SPLITS = 1024         # the merge of key splits keeps one weight per split in LDS
 
 
@@ -280,16 +281,21 @@ class Kernels:
                _c_int(q_heads), _c_int(kv_heads), _c_int(head_dim), _c_int(page_size), _c_int(window or 0),
                _c_float(scale), _c_int(split_keys), _c_int(max_splits), _stream()), "attention_mfma")
 
-    def prefill_attention_supported(self, q_heads, kv_heads, head_dim, page_size):
-        """The LDS-staged kernel for prompt portions: as the matrix-core kernel, head sizes up to 224."""
-        return self.mfma_attention_supported(q_heads, kv_heads, head_dim, page_size) and head_dim <= 224
+    def prefill_attention_supported(self, q_heads, kv_heads, head_dim, page_size, max_context=0):
+        """The LDS-staged kernel for prompt portions: as the matrix-core kernel, head sizes up to 192 and
+        contexts of at most 2048 pages (it keeps a group's page ids in LDS)."""
+        return (self.mfma_attention_supported(q_heads, kv_heads, head_dim, page_size) and head_dim <= 192
+                and max_context <= PREFILL_MAX_PAGES * page_size)
 
     def attention_prefill(self, q, k_pages, v_pages, block_table, slots, positions, out, group_row0, group_ntok,
-                          groups, q_heads, kv_heads, head_dim, page_size, scale, window=None):
+                          groups, q_heads, kv_heads, head_dim, page_size, scale, window=None, max_context=None):
         """Attention for prompt portions: groups of up to 4 * (16 // (q_heads // kv_heads)) consecutive rows
         of one request each; keys and values of a group are staged once through LDS."""
         _need(self.prefill_attention_supported(q_heads, kv_heads, head_dim, page_size),
               "attention_prefill: sizes not supported")
+        _need(block_table.shape[1] <= PREFILL_MAX_PAGES or max_context is not None,
+              "attention_prefill: give max_context when the block table is wider than the kernel's page cache")
+        _need((max_context or 0) <= PREFILL_MAX_PAGES * page_size, "attention_prefill: context too long")
         _tensor(q, "q", self.dtype, ndim=2)
         m = q.shape[0]
         _need(q.shape[1] == q_heads * head_dim, "q: wrong width")

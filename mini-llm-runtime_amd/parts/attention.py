@@ -80,12 +80,13 @@ class GqaAttention:
         if k.mfma_attention_supported(s.q_heads, s.kv_heads, s.head_dim, view.page_size):
             # prompt portions go to the LDS-staged kernel, single tokens and short portions to the one
             # that can split a token's keys over workgroups
-            big_factor = 4 if k.prefill_attention_supported(s.q_heads, s.kv_heads, s.head_dim, view.page_size) else 0
+            big_factor = 4 if k.prefill_attention_supported(s.q_heads, s.kv_heads, s.head_dim, view.page_size,
+                                                            ctx.max_context) else 0
             small, big, small_rows = ctx.token_groups(max(1, 16 // (s.q_heads // s.kv_heads)), big_factor)
             if big[2]:
                 k.attention_prefill(q, view.k_pages, view.v_pages, view.block_table, ctx.slots, ctx.positions, attn,
                                     big[0], big[1], big[2], s.q_heads, s.kv_heads, s.head_dim, view.page_size,
-                                    float(s.scale), window=s.window)
+                                    float(s.scale), window=s.window, max_context=ctx.max_context)
             if small[2]:
                 split_keys, max_splits, partial = ctx.attention_split(small_rows, m, s.kv_heads, s.q_heads, s.head_dim)
                 k.attention_mfma(q, view.k_pages, view.v_pages, view.block_table, ctx.slots, ctx.positions, attn,

@@ -262,7 +262,9 @@ def plain_attention(q, keys, values, scale, window):
     (8, 8, 80, 16, [77], 40, 0),
     (16, 8, 128, 16, [530, 3], None, 0),
     (4, 1, 96, 32, [150], 50, 0),
-    (14, 2, 224, 16, [40], None, 0),
+    (14, 2, 192, 16, [40], None, 0),
+    (2, 1, 224, 16, [40], None, 0),
+    (4, 2, 32, 16, [300], 70, 0),
 ])
 def test_paged_attention(dtype, case):
     """Every length is one request whose LAST token is the query (a decoded token) plus, for the
