@@ -49,11 +49,87 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ h, const elem_t* __restri
     }
 }
 
+// The same for widths that are a multiple of 8 (bfloat16) or 4 (float), 16 bytes per lane and access:
+// one wavefront per row, four rows per workgroup, the row kept in registers between the two passes
+// when it fits (width <= 64 * MLR_VEC * ROW_REGS), else re-read.
+#define ROW_REGS 4
+__global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict__ h, const elem_t* __restrict__ delta,
+                                                              const float* __restrict__ weight,
+                                                              elem_t* __restrict__ out, const int32_t* __restrict__ rows,
+                                                              int n_out, int width, float eps, int write_h) {
+    const int lane = threadIdx.x & 63;
+    const int r = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (r >= n_out) return;
+    const size_t src = rows ? (size_t)rows[r] : (size_t)r;
+    float* hrow = h + src * width;
+    const elem_t* drow = delta ? delta + src * width : nullptr;
+    float x[ROW_REGS][MLR_VEC];
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < ROW_REGS; ++i) {
+        const int c = (lane + 64 * i) * MLR_VEC;
+        if (c < width) {
+#pragma unroll
+            for (int e = 0; e < MLR_VEC; e += 4) {
+                const float4 v = *reinterpret_cast<const float4*>(hrow + c + e);
+                x[i][e] = v.x; x[i][e + 1] = v.y; x[i][e + 2] = v.z; x[i][e + 3] = v.w;
+            }
+            if (drow) {
+                float dv[MLR_VEC];
+                load_vec(drow + c, dv);
+#pragma unroll
+                for (int e = 0; e < MLR_VEC; ++e) x[i][e] += dv[e];
+                if (write_h) {
+#pragma unroll
+                    for (int e = 0; e < MLR_VEC; e += 4)
+                        *reinterpret_cast<float4*>(hrow + c + e) = make_float4(x[i][e], x[i][e + 1], x[i][e + 2], x[i][e + 3]);
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < MLR_VEC; ++e) sum += x[i][e] * x[i][e];
+        }
+    }
+    sum = wave_sum(sum);
+    const float scale = 1.0f / sqrtf(sum / (float)width + eps);
+    elem_t* orow = out + (size_t)r * width;
+#pragma unroll
+    for (int i = 0; i < ROW_REGS; ++i) {
+        const int c = (lane + 64 * i) * MLR_VEC;
+        if (c < width) {
+            float y[MLR_VEC];
+#pragma unroll
+            for (int e = 0; e < MLR_VEC; e += 4) {
+                const float4 w = *reinterpret_cast<const float4*>(weight + c + e);
+                y[e] = (x[i][e] * scale) * w.x;
+                y[e + 1] = (x[i][e + 1] * scale) * w.y;
+                y[e + 2] = (x[i][e + 2] * scale) * w.z;
+                y[e + 3] = (x[i][e + 3] * scale) * w.w;
+            }
+            store_vec(orow + c, y);
+        }
+    }
+}
+
 // h[m, :] += delta[m, :] (the last residual sum when nothing is normed afterwards).
 __global__ void residual_add_kernel(float* __restrict__ h, const elem_t* __restrict__ delta, size_t count) {
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count;
          i += (size_t)gridDim.x * blockDim.x) {
         h[i] += to_float(delta[i]);
+    }
+}
+
+// The same, 16 bytes per lane and access, for inter % MLR_VEC == 0.
+__global__ void silu_mul_vec_kernel(const elem_t* __restrict__ gate_up, elem_t* __restrict__ act, int rows, int inter) {
+    const int per_row = inter / MLR_VEC;
+    const size_t total = (size_t)rows * per_row;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        const size_t m = i / per_row, f = (i % per_row) * MLR_VEC;
+        float g[MLR_VEC], u[MLR_VEC], y[MLR_VEC];
+        load_vec(gate_up + m * 2 * inter + f, g);
+        load_vec(gate_up + m * 2 * inter + inter + f, u);
+#pragma unroll
+        for (int e = 0; e < MLR_VEC; ++e) y[e] = (g[e] / (1.0f + expf(-g[e]))) * u[e];
+        store_vec(act + m * inter + f, y);
     }
 }
 
@@ -87,6 +163,12 @@ int mlr_embed_gather(const int32_t* ids, const void* table, float* h, int rows, 
 int mlr_add_rmsnorm(float* h, const void* delta, const float* weight, void* out, const int32_t* rows,
                     int n_out, int width, float eps, int write_h, hipStream_t stream) {
     if (n_out <= 0) return 0;
+    // (the float engine keeps its one order of additions for every batch size)
+    if (MLR_BF16 && width % MLR_VEC == 0 && width <= 64 * MLR_VEC * ROW_REGS && n_out >= 64) {
+        add_rmsnorm_vec_kernel<<<(n_out + 3) / 4, 256, 0, stream>>>(h, (const elem_t*)delta, weight, (elem_t*)out,
+                                                                     rows, n_out, width, eps, write_h);
+        return (int)hipGetLastError();
+    }
     add_rmsnorm_kernel<<<n_out, 256, 0, stream>>>(h, (const elem_t*)delta, weight, (elem_t*)out, rows,
                                                   width, eps, write_h);
     return (int)hipGetLastError();
@@ -100,6 +182,11 @@ int mlr_residual_add(float* h, const void* delta, size_t count, hipStream_t stre
 
 int mlr_silu_mul(const void* gate_up, void* act, int rows, int inter, hipStream_t stream) {
     if (rows <= 0) return 0;
+    if (inter % MLR_VEC == 0) {
+        silu_mul_vec_kernel<<<grid_for((size_t)rows * (inter / MLR_VEC), 256), 256, 0, stream>>>(
+            (const elem_t*)gate_up, (elem_t*)act, rows, inter);
+        return (int)hipGetLastError();
+    }
     silu_mul_kernel<<<grid_for((size_t)rows * inter, 256), 256, 0, stream>>>(
         (const elem_t*)gate_up, (elem_t*)act, rows, inter);
     return (int)hipGetLastError();

@@ -96,6 +96,97 @@ __global__ void qk_norm_rope_kv_kernel(
     }
 }
 
+#if MLR_BF16
+// The same for many rows of the bfloat16 engine and head sizes 16, 32, 64, 128, 256: head_dim / 16 lanes
+// serve a head, each with eight consecutive channels of the first half and their partners of the second
+// half (16-byte accesses); a wavefront serves 64 / (head_dim / 16) heads at once.
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+
+__global__ __launch_bounds__(256) void qk_norm_rope_kv_vec_kernel(
+    const __bf16* __restrict__ qkv, int ld, __bf16* __restrict__ q_out, __bf16* __restrict__ k_pages,
+    __bf16* __restrict__ v_pages, const int32_t* __restrict__ block_table, int max_blocks,
+    const int32_t* __restrict__ slots, const int32_t* __restrict__ positions, const float* __restrict__ q_norm_w,
+    const float* __restrict__ k_norm_w, float eps, const float* __restrict__ rope, int q_heads, int kv_heads,
+    int head_dim, int page_size, int write_cache) {
+    const int m = blockIdx.x;
+    const int lph = head_dim / 16;                         // lanes per head (a power of two)
+    const int half = head_dim >> 1;
+    const int total = q_heads + 2 * kv_heads;
+    const int head = (blockIdx.y * blockDim.x + threadIdx.x) / lph;
+    const int c = threadIdx.x % lph;                       // this lane: channels 8c .. 8c + 7 and half + 8c ..
+    const int pos = positions[m], slot = slots[m];
+    const bool active = head < total;
+    const __bf16* src = qkv + (size_t)m * ld + (size_t)(active ? head : 0) * head_dim;
+    const bf16x8 lo8 = *reinterpret_cast<const bf16x8*>(src + 8 * c);
+    const bf16x8 hi8 = *reinterpret_cast<const bf16x8*>(src + half + 8 * c);
+    float a[8], b[8];
+    float sum = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        a[e] = (float)lo8[e];
+        b[e] = (float)hi8[e];
+        sum += a[e] * a[e] + b[e] * b[e];
+    }
+    for (int off = 1; off < lph; off <<= 1) sum += __shfl_xor(sum, off, MLR_WAVE);
+    if (!active) return;
+    size_t cache_page = 0;
+    int in_page = 0;
+    bool cache_ok = false;
+    if (write_cache) {
+        const int page = block_table[(size_t)slot * max_blocks + pos / page_size];
+        cache_ok = page >= 0;
+        cache_page = (size_t)(page < 0 ? 0 : page) * kv_heads;
+        in_page = pos % page_size;
+    }
+    if (head >= q_heads + kv_heads) {                      // a value head: into its transposed page
+        if (!cache_ok) return;
+        __bf16* dst = v_pages + (cache_page + (head - q_heads - kv_heads)) * head_dim * page_size + in_page;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            dst[(size_t)(8 * c + e) * page_size] = lo8[e];
+            dst[(size_t)(half + 8 * c + e) * page_size] = hi8[e];
+        }
+        return;
+    }
+    const bool is_q = head < q_heads;
+    const float* w = is_q ? q_norm_w : k_norm_w;
+    if (w) {
+        const float scale = 1.0f / sqrtf(sum / (float)head_dim + eps);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            a[e] = (a[e] * scale) * w[8 * c + e];
+            b[e] = (b[e] * scale) * w[half + 8 * c + e];
+        }
+    }
+    if (rope) {
+        const float* cs = rope + (size_t)pos * head_dim;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float co = cs[8 * c + e], si = cs[half + 8 * c + e];
+            const float x = a[e] * co - b[e] * si;
+            const float y = a[e] * si + b[e] * co;
+            a[e] = x;
+            b[e] = y;
+        }
+    }
+    __bf16* dst;
+    if (is_q) {
+        dst = q_out + ((size_t)m * q_heads + head) * head_dim;
+    } else {
+        if (!cache_ok) return;
+        dst = k_pages + ((cache_page + (head - q_heads)) * page_size + in_page) * head_dim;
+    }
+    bf16x8 o_lo, o_hi;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        o_lo[e] = (__bf16)a[e];
+        o_hi[e] = (__bf16)b[e];
+    }
+    *reinterpret_cast<bf16x8*>(dst + 8 * c) = o_lo;
+    *reinterpret_cast<bf16x8*>(dst + half + 8 * c) = o_hi;
+}
+#endif
+
 extern "C" int mlr_qk_norm_rope_kv(
     const void* qkv, int ld, void* q_out, void* k_pages, void* v_pages, const int32_t* block_table,
     int max_blocks, const int32_t* slots, const int32_t* positions, const float* q_norm_w,
@@ -103,8 +194,18 @@ extern "C" int mlr_qk_norm_rope_kv(
     int head_dim, int page_size, int write_cache, hipStream_t stream) {
     if (rows <= 0) return 0;
     if (head_dim % 2 != 0 || head_dim / 2 > 64 * MAX_PAIRS) return -1;
-    // few rows: spread a row's heads over several workgroups (a wavefront per head)
     const int total_heads = q_heads + 2 * kv_heads;
+#if MLR_BF16
+    const int lph = head_dim / 16;
+    if (rows >= 64 && head_dim % 16 == 0 && (lph & (lph - 1)) == 0 && ld % 8 == 0) {
+        const int threads_needed = total_heads * lph;
+        qk_norm_rope_kv_vec_kernel<<<dim3(rows, (threads_needed + 255) / 256), 256, 0, stream>>>(
+            (const __bf16*)qkv, ld, (__bf16*)q_out, (__bf16*)k_pages, (__bf16*)v_pages, block_table, max_blocks,
+            slots, positions, q_norm_w, k_norm_w, eps, rope, q_heads, kv_heads, head_dim, page_size, write_cache);
+        return (int)hipGetLastError();
+    }
+#endif
+    // few rows: spread a row's heads over several workgroups (a wavefront per head)
     int chunks = 1;
     if (rows < 512) chunks = (total_heads + 3) / 4;
     if (chunks > 64) chunks = 64;

@@ -509,3 +509,85 @@ def test_gemm_gated_silu(mnk):
     u = a.double() @ w.double()[n:].T
     want = g / (1 + torch.exp(-g)) * u
     torch.testing.assert_close(out.double(), want, atol=2e-2 * float(want.abs().max()), rtol=2e-2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", [(4, 2, 128, 16), (6, 3, 48, 32), (16, 8, 64, 16), (3, 1, 16, 16), (2, 2, 256, 64)])
+def test_qk_norm_rope_kv_many_rows(dtype, shape):
+    """A whole prompt portion (the many-row variants of the kernel): 90 consecutive positions of one request
+    beside 10 of another."""
+    hq, hkv, d, page = shape
+    k = kernels(dtype)
+    counts = [90, 10]
+    starts = [37, 0]
+    m = sum(counts)
+    positions = torch.tensor([starts[s] + i for s in range(2) for i in range(counts[s])], dtype=torch.int32)
+    slots = torch.tensor([s for s in range(2) for _ in range(counts[s])], dtype=torch.int32)
+    max_blocks = 16
+    n_pages = 2 * max_blocks
+    perm = torch.randperm(n_pages, generator=torch.Generator().manual_seed(3)).to(torch.int32)
+    table = perm.view(2, max_blocks).contiguous()
+    qkv = rnd((m, (hq + 2 * hkv) * d), dtype, 60)
+    qw, kw = rnd((d,), torch.float32, 61) + 1, rnd((d,), torch.float32, 62) + 1
+    eps, base = 1e-6, 10000.0
+    rope = rope_table(256, d, base)
+    k_pages = torch.full((n_pages, hkv, page, d), float("nan"), dtype=dtype, device="cuda")
+    v_pages = torch.full((n_pages, hkv, d, page), float("nan"), dtype=dtype, device="cuda")
+    q_out = torch.empty((m, hq * d), dtype=dtype, device="cuda")
+    k.qk_norm_rope_kv(qkv, q_out, k_pages, v_pages, table.cuda(), slots.cuda(), positions.cuda(), qw, kw, eps, rope,
+                      hq, hkv, d, page)
+    x = qkv.double().cpu()
+    q = x[:, :hq * d].view(m, hq, d)
+    kk = x[:, hq * d:(hq + hkv) * d].view(m, hkv, d)
+
+    def norm(t, w):
+        return t * torch.rsqrt((t * t).mean(-1, keepdim=True) + eps) * w.double().cpu()
+    q_want = plain_rope(norm(q, qw), positions, base)
+    k_want = plain_rope(norm(kk, kw), positions, base)
+    torch.testing.assert_close(q_out.double().cpu().view(m, hq, d), q_want, **tol(dtype))
+    kp, vp = k_pages.cpu(), v_pages.cpu()
+    for i in range(m):
+        p, s = int(positions[i]), int(slots[i])
+        pg = int(table[s, p // page])
+        torch.testing.assert_close(kp[pg, :, p % page].double(), k_want[i], **tol(dtype))
+        assert torch.equal(vp[pg, :, :, p % page], qkv[i, (hq + hkv) * d:].view(hkv, d).cpu())
+    written = sum(counts) * hkv * d
+    assert int((~torch.isnan(kp.float())).sum()) == written and int((~torch.isnan(vp.float())).sum()) == written
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("width", [8, 72, 1024, 2048, 2056, 76])
+def test_add_rmsnorm_many_rows(dtype, width):
+    k = kernels(dtype)
+    rows = 130
+    h0 = rnd((rows, width), torch.float32, 70, 2.0)
+    delta = rnd((rows, width), dtype, 71)
+    w = rnd((width,), torch.float32, 72)
+    x = h0.double() + delta.double()
+    want = x * torch.rsqrt((x * x).mean(-1, keepdim=True) + 1e-6) * w.double()
+    h = h0.clone()
+    out = torch.empty((rows, width), dtype=dtype, device="cuda")
+    k.add_rmsnorm(h, delta, w, out, 1e-6)
+    torch.testing.assert_close(h.double(), x, atol=1e-6, rtol=1e-6)
+    torch.testing.assert_close(out.double(), want, **tol(dtype))
+    idx = torch.arange(rows - 1, -1, -1, dtype=torch.int32).cuda()[:100].contiguous()
+    h = h0.clone()
+    out = torch.empty((100, width), dtype=dtype, device="cuda")
+    k.add_rmsnorm(h, delta, w, out, 1e-6, rows=idx, write_h=False)
+    assert torch.equal(h, h0)
+    torch.testing.assert_close(out.double(), want[idx.long()], **tol(dtype))
+    out = torch.empty((rows, width), dtype=dtype, device="cuda")
+    k.add_rmsnorm(h, None, w, out, 1e-6)
+    x = h0.double()
+    torch.testing.assert_close(out.double(), x * torch.rsqrt((x * x).mean(-1, keepdim=True) + 1e-6) * w.double(), **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("inter", [8, 104, 3072])
+def test_silu_mul_wide(dtype, inter):
+    k = kernels(dtype)
+    gate_up = rnd((70, 2 * inter), dtype, 80, 3.0)
+    act = torch.empty((70, inter), dtype=dtype, device="cuda")
+    k.silu_mul(gate_up, act)
+    g, u = gate_up.double()[:, :inter], gate_up.double()[:, inter:]
+    torch.testing.assert_close(act.double(), g / (1 + torch.exp(-g)) * u, **tol(dtype))
