@@ -552,7 +552,7 @@ __global__ __launch_bounds__(256, (NCH <= 4 ? 2 : 1)) void attention_mfma_kernel
 // `attention_mfma_kernel` without key splits, tile by tile in ascending order.
 #define PAGE_CACHE 2048
 template <int NCH>
-__global__ __launch_bounds__(256) void attention_prefill_kernel(AttnArgs a, const int32_t* __restrict__ group_row0,
+__global__ __launch_bounds__(256, 2) void attention_prefill_kernel(AttnArgs a, const int32_t* __restrict__ group_row0,
                                                                 const int32_t* __restrict__ group_ntok) {
     constexpr int DMAX = 32 * NCH;
     constexpr int KPITCH = DMAX + 8;                  // elements per key row in LDS
@@ -607,61 +607,75 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(AttnArgs a, cons
         for (int i = threadIdx.x; i < n_pages; i += 256) page_lds[i] = table[first_page + i];
         __syncthreads();
     }
-    const int kchunks = 4 * D;                         // 32 keys x D / 8
-    const int vchunks = 4 * D;                         // D channels x 32 keys / 8
+    const int kchunks = 4 * D;                         // 32 keys x D / 8 chunks of 16 bytes; as many for V
     struct Staged {
         bf16x8 k[STAGE], v[STAGE];
         int tb;
         int ok;                                        // bit j: the page of keys tb + 16 j .. is mapped
     };                                                 // (no array indexed at run time: that would live in scratch)
+    // what a thread stages does not change from tile to tile: offsets computed once
+    int k_goff[STAGE], k_loff[STAGE], v_goff[STAGE], v_loff[STAGE], v_key[STAGE];
+    bool st_valid[STAGE], k_sel[STAGE], v_sel[STAGE];
+#pragma unroll
+    for (int i = 0; i < STAGE; ++i) {
+        st_valid[i] = (int)threadIdx.x + 256 * i < kchunks;
+        const int ci = min((int)threadIdx.x + 256 * i, kchunks - 1);
+        const int key = ci / (D / 8), c8 = ci % (D / 8);
+        k_sel[i] = (key >> 4) != 0;
+        k_goff[i] = (key & 15) * D + 8 * c8;
+        k_loff[i] = key * KPITCH + 8 * c8;
+        const int d = ci >> 2, q4 = ci & 3;
+        v_sel[i] = (q4 >> 1) != 0;
+        v_goff[i] = d * P + 8 * (q4 & 1);
+        v_loff[i] = d * VPITCH + 8 * q4;
+        v_key[i] = 8 * q4;                             // first key of the chunk within the tile
+    }
     // global -> registers.  No branch around a load: a load behind a branch makes the compiler wait for
     // every load in flight.  Addresses are clamped to valid memory (page 0 for a missing page, the last
     // chunk for a thread without one); what must read as zero is zeroed when the registers go to LDS.
     auto fetch = [&](int t, Staged& st) {
         const int tb = t * MFMA_TILE_KEYS;
         st.tb = tb;
-        st.ok = 0;
-        size_t kbase0 = 0, kbase1 = 0, vbase0 = 0, vbase1 = 0;
-#pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const int key0 = tb + 16 * j;
-            const int idx = min(max(key0 / P - first_page, 0), PAGE_CACHE - 1);
-            const int page = key0 < ke ? page_lds[idx] : -1;       // the host keeps the group's pages within the cache
-            const bool ok = page >= 0;
-            st.ok |= (ok ? 1 : 0) << j;
-            const size_t pk = (size_t)(ok ? page : 0) * a.kv_heads + kvh;
-            const size_t kb = (pk * P + key0 % P) * D, vb = pk * D * P + key0 % P;
-            if (j == 0) { kbase0 = kb; vbase0 = vb; } else { kbase1 = kb; vbase1 = vb; }
-        }
+        const int idx0 = min(max(tb / P - first_page, 0), PAGE_CACHE - 1);
+        const int idx1 = min(max((tb + 16) / P - first_page, 0), PAGE_CACHE - 1);
+        const int page0 = tb < ke ? page_lds[idx0] : -1;           // the host keeps the group's pages within the cache
+        const int page1 = tb + 16 < ke ? page_lds[idx1] : -1;
+        st.ok = (page0 >= 0 ? 1 : 0) | (page1 >= 0 ? 2 : 0);
+        const size_t pk0 = (size_t)max(page0, 0) * a.kv_heads + kvh, pk1 = (size_t)max(page1, 0) * a.kv_heads + kvh;
+        const __bf16* k0 = kp_base + (pk0 * P + tb % P) * D;
+        const __bf16* k1 = kp_base + (pk1 * P + (tb + 16) % P) * D;
+        const __bf16* v0 = vp_base + pk0 * D * P + tb % P;
+        const __bf16* v1 = vp_base + pk1 * D * P + (tb + 16) % P;
 #pragma unroll
         for (int i = 0; i < STAGE; ++i) {
-            const int ci = min((int)threadIdx.x + 256 * i, kchunks - 1);
-            const int key = ci / (D / 8), c8 = ci % (D / 8);
-            st.k[i] = *reinterpret_cast<const bf16x8*>(kp_base + ((key >> 4) ? kbase1 : kbase0) + (size_t)(key & 15) * D + 8 * c8);
-            const int d = ci >> 2, q4 = ci & 3;
-            st.v[i] = *reinterpret_cast<const bf16x8*>(vp_base + ((q4 >> 1) ? vbase1 : vbase0) + (size_t)d * P + 8 * (q4 & 1));
+            st.k[i] = *reinterpret_cast<const bf16x8*>((k_sel[i] ? k1 : k0) + k_goff[i]);
+            st.v[i] = *reinterpret_cast<const bf16x8*>((v_sel[i] ? v1 : v0) + v_goff[i]);
         }
     };
     auto stash = [&](int buf, const Staged& st) {      // registers -> LDS
+        const bool whole = st.ok == 3 && st.tb + MFMA_TILE_KEYS <= ke;    // the usual tile: nothing to zero
 #pragma unroll
         for (int i = 0; i < STAGE; ++i) {
-            const int ci = threadIdx.x + 256 * i;
-            if (ci >= kchunks) continue;
-            const int key = ci / (D / 8), c8 = ci % (D / 8);
-            *reinterpret_cast<bf16x8*>(&k_lds[buf][key * KPITCH + 8 * c8]) = ((st.ok >> (key >> 4)) & 1) ? st.k[i] : zero8;
-            const int d = ci >> 2, q4 = ci & 3, j = q4 >> 1;
-            bf16x8 v = ((st.ok >> j) & 1) ? st.v[i] : zero8;
-            const int key0 = st.tb + 16 * j + 8 * (q4 & 1);
-            if (key0 + 8 > ke) {                       // keys that are not written yet count as zero
+            if (!st_valid[i]) continue;
+            bf16x8 kv = st.k[i], v = st.v[i];
+            if (!whole) {
+                if (!((st.ok >> (k_sel[i] ? 1 : 0)) & 1)) kv = zero8;
+                if (!((st.ok >> (v_sel[i] ? 1 : 0)) & 1)) v = zero8;
+                const int key0 = st.tb + v_key[i];
 #pragma unroll
-                for (int e = 0; e < 8; ++e)
+                for (int e = 0; e < 8; ++e)            // keys that are not written yet count as zero
                     if (key0 + e >= ke) v[e] = (__bf16)0.f;
             }
-            *reinterpret_cast<bf16x4*>(&v_lds[buf][d * VPITCH + 8 * q4]) = bf16x4{v[0], v[1], v[2], v[3]};
-            *reinterpret_cast<bf16x4*>(&v_lds[buf][d * VPITCH + 8 * q4 + 4]) = bf16x4{v[4], v[5], v[6], v[7]};
+            *reinterpret_cast<bf16x8*>(&k_lds[buf][k_loff[i]]) = kv;
+            *reinterpret_cast<bf16x4*>(&v_lds[buf][v_loff[i]]) = bf16x4{v[0], v[1], v[2], v[3]};
+            *reinterpret_cast<bf16x4*>(&v_lds[buf][v_loff[i] + 4]) = bf16x4{v[4], v[5], v[6], v[7]};
         }
     };
 
+    // Scores are kept in the base-2 domain: s * (scale * log2 e), so that a probability is one v_exp_f32.
+    const float c2 = a.scale * 1.44269504088896340736f;
+    const int wave_first_kend = pos0 + wtok0 + 1;                     // key range end of the wavefront's first token
+    const int wave_last_kbegin = a.window > 0 ? max(0, wave_hi - a.window) : 0;
     auto compute = [&](int t, int buf) {
         const int tb = t * MFMA_TILE_KEYS;
         if (!wave_active || tb >= wave_hi || tb + MFMA_TILE_KEYS <= wave_lo) return;     // nothing for this wavefront
@@ -680,39 +694,50 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(AttnArgs a, cons
             }
         }
         float sv[2][4];
-        float tile_max = -INFINITY;
+        // a tile that every token of this wavefront sees whole needs no mask (all but the last one or two)
+        const bool interior = tb + MFMA_TILE_KEYS <= wave_first_kend && tb >= wave_last_kbegin;
+        if (interior) {
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+            for (int j = 0; j < 2; ++j)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int key = tb + 16 * j + 4 * b + r;
-                const bool ok = key >= kbegin_c && key < kend_c;
-                sv[j][r] = ok ? s[j][r] * a.scale : -INFINITY;
-                tile_max = fmaxf(tile_max, sv[j][r]);
-            }
-        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, MLR_WAVE));
-        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, MLR_WAVE));
-        const float m_new = fmaxf(m_run, tile_max);
-        float corr = 1.f;
-        bf16x8 pf = zero8;
-        if (m_new > -INFINITY) {
-            corr = __expf(m_run - m_new);
-            float psum = 0.f;
+                for (int r = 0; r < 4; ++r) sv[j][r] = s[j][r] * c2;
+        } else {
 #pragma unroll
             for (int j = 0; j < 2; ++j)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    const float p = sv[j][r] > -INFINITY ? __expf(sv[j][r] - m_new) : 0.f;
-                    psum += p;
-                    pf[4 * j + r] = (__bf16)p;
+                    const int key = tb + 16 * j + 4 * b + r;
+                    sv[j][r] = (key >= kbegin_c && key < kend_c) ? s[j][r] * c2 : -INFINITY;
                 }
-            l_run = l_run * corr + psum;
+        }
+        float tile_max = fmaxf(fmaxf(fmaxf(sv[0][0], sv[0][1]), fmaxf(sv[0][2], sv[0][3])),
+                               fmaxf(fmaxf(sv[1][0], sv[1][1]), fmaxf(sv[1][2], sv[1][3])));
+        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, MLR_WAVE));
+        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, MLR_WAVE));
+        // the running maximum rarely moves after the first tiles: rescale only when it does, for any column
+        if (__builtin_amdgcn_ballot_w64(tile_max > m_run) != 0) {
+            const float m_new = fmaxf(m_run, tile_max);
+            const float corr = m_new > -INFINITY ? __builtin_amdgcn_exp2f(m_run - m_new) : 1.f;   // -inf - finite: 0
+            l_run *= corr;
+#pragma unroll
+            for (int db = 0; db < 2 * NCH; ++db) o[db] *= corr;
             m_run = m_new;
         }
+        const float m_use = fmaxf(m_run, -1e30f);      // a column with no key yet: exp2(-inf - finite) = 0, not NaN
+        bf16x8 pf;
+        float psum = 0.f;
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float p = __builtin_amdgcn_exp2f(sv[j][r] - m_use);
+                psum += p;
+                pf[4 * j + r] = (__bf16)p;
+            }
+        l_run += psum;
 #pragma unroll
         for (int db = 0; db < 2 * NCH; ++db) {
             if (16 * db >= D) break;
-            o[db] *= corr;
             const __bf16* vrow = &v_lds[buf][(16 * db + col) * VPITCH];
             const bf16x4 v0 = *reinterpret_cast<const bf16x4*>(vrow + 4 * b);
             const bf16x4 v1 = *reinterpret_cast<const bf16x4*>(vrow + 16 + 4 * b);
