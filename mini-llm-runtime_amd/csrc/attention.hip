@@ -297,18 +297,17 @@ template <int NCH>
 struct KvTile {
     bf16x8 k[2][NCH];
     bf16x4 v[2 * NCH][2];
-    bool ok[2];
+    int ok;                  // bit j: the page of keys tb + 16 j .. is mapped
     int tb;
 };
 
-struct TilePages {
-    int page[2];
-};
+#define DECODE_PAGE_CACHE 4096
 
 template <int NCH>   // ceil(head_dim / 32)
 __global__ __launch_bounds__(256, (NCH <= 4 ? 2 : 1)) void attention_mfma_kernel(AttnArgs a, const int32_t* __restrict__ group_row0,
                                                              const int32_t* __restrict__ group_ntok) {
     extern __shared__ float lds[];
+    __shared__ int32_t page_lds[DECODE_PAGE_CACHE];    // the request's page ids for this workgroup's key range
     const int D = a.head_dim, P = a.page_size;
     const int g = a.q_heads / a.kv_heads;
     const int grp = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z;
@@ -337,8 +336,15 @@ __global__ __launch_bounds__(256, (NCH <= 4 ? 2 : 1)) void attention_mfma_kernel
     const __bf16* kp_base = reinterpret_cast<const __bf16*>(a.k_pages);
     const __bf16* vp_base = reinterpret_cast<const __bf16*>(a.v_pages);
     const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
-    const bf16x4 zero4 = {0, 0, 0, 0};
     const int32_t* table = a.block_table + (size_t)slot * a.max_blocks;
+
+    // page ids first, into LDS: a tile's loads then never wait on a load of the block table
+    const int t_begin = lo / MFMA_TILE_KEYS, t_end = (hi + MFMA_TILE_KEYS - 1) / MFMA_TILE_KEYS;
+    const int first_page = t_begin * MFMA_TILE_KEYS / P;
+    {
+        const int n_pages = min(DECODE_PAGE_CACHE, (hi + P - 1) / P - first_page);
+        for (int i = threadIdx.x; i < n_pages; i += 256) page_lds[i] = table[first_page + i];
+    }
 
     bf16x8 qf[NCH];
 #pragma unroll
@@ -348,40 +354,39 @@ __global__ __launch_bounds__(256, (NCH <= 4 ? 2 : 1)) void attention_mfma_kernel
         if (col_valid && d0 < D)
             qf[c] = *reinterpret_cast<const bf16x8*>(q + ((size_t)(row0 + tok) * a.q_heads + kvh * g + hh) * D + d0);
     }
+    __syncthreads();
 
+    // Scores are kept in the base-2 domain: s * (scale * log2 e), so that a probability is one v_exp_f32.
+    const float c2 = a.scale * 1.44269504088896340736f;
     float m_run = -INFINITY, l_run = 0.f;
     floatx4 o[2 * NCH];
 #pragma unroll
     for (int i = 0; i < 2 * NCH; ++i) o[i] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-    auto lookup = [&](int t) {
-        TilePages tp;
-#pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const int key0 = t * MFMA_TILE_KEYS + 16 * j;
-            tp.page[j] = (key0 < hi) ? table[key0 / P] : -1;
-        }
-        return tp;
-    };
-    auto load = [&](int t, const TilePages& tp, KvTile<NCH>& T) {
+    // this lane's fixed offsets into a key page (row col, channels 8b ..) and a value page (row col, keys 4b ..)
+    const int k_lane = col * D + 8 * b, v_lane = col * P + 4 * b;
+    const bool d_whole = (D & 31) == 0;
+    // No branch around a load: a load behind a branch makes the compiler wait for every load in flight.
+    // A missing page reads page 0 instead, channels beyond head_dim read channel block 0; both are
+    // discarded when the tile is used.
+    auto load = [&](int t, KvTile<NCH>& T) {
         T.tb = t * MFMA_TILE_KEYS;
+        T.ok = 0;
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             const int key0 = T.tb + 16 * j;
-            T.ok[j] = tp.page[j] >= 0;
-            const size_t pk = (size_t)(T.ok[j] ? tp.page[j] : 0) * a.kv_heads + kvh;
-            const __bf16* kptr = kp_base + (pk * P + key0 % P + col) * D + 8 * b;
-            const __bf16* vptr = vp_base + pk * D * P + key0 % P + (size_t)col * P + 4 * b;
+            const int idx = min(max(key0 / P - first_page, 0), DECODE_PAGE_CACHE - 1);
+            const int page = key0 < hi ? page_lds[idx] : -1;
+            T.ok |= (page >= 0 ? 1 : 0) << j;
+            const size_t pk = (size_t)max(page, 0) * a.kv_heads + kvh;
+            const __bf16* kptr = kp_base + (pk * P + key0 % P) * D + k_lane;
+            const __bf16* vptr = vp_base + pk * D * P + key0 % P + v_lane;
 #pragma unroll
-            for (int c = 0; c < NCH; ++c) {
-                T.k[j][c] = zero8;
-                if (T.ok[j] && 32 * c + 8 * b < D) T.k[j][c] = *reinterpret_cast<const bf16x8*>(kptr + 32 * c);
-            }
+            for (int c = 0; c < NCH; ++c)
+                T.k[j][c] = *reinterpret_cast<const bf16x8*>(kptr + (32 * c + 8 * b < D ? 32 * c : 0));
 #pragma unroll
-            for (int db = 0; db < 2 * NCH; ++db) {
-                T.v[db][j] = zero4;
-                if (T.ok[j] && 16 * db < D) T.v[db][j] = *reinterpret_cast<const bf16x4*>(vptr + (size_t)16 * db * P);
-            }
+            for (int db = 0; db < 2 * NCH; ++db)
+                T.v[db][j] = *reinterpret_cast<const bf16x4*>(vptr + (size_t)(16 * db < D ? 16 * db : 0) * P);
         }
     };
     auto compute = [&](KvTile<NCH>& T) {
@@ -389,83 +394,87 @@ __global__ __launch_bounds__(256, (NCH <= 4 ? 2 : 1)) void attention_mfma_kernel
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             s[j] = floatx4{0.f, 0.f, 0.f, 0.f};
-            if (T.ok[j]) {
+            if (d_whole) {
 #pragma unroll
                 for (int c = 0; c < NCH; ++c)
                     s[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(T.k[j][c], qf[c], s[j], 0, 0, 0);
+            } else {
+#pragma unroll
+                for (int c = 0; c < NCH; ++c) {
+                    const bf16x8 kf = (32 * c + 8 * b < D) ? T.k[j][c] : zero8;
+                    s[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[c], s[j], 0, 0, 0);
+                }
             }
         }
         // this lane: keys tb + 16 j + 4 b + r of column `col`
         float sv[2][4];
-        float tile_max = -INFINITY;
 #pragma unroll
         for (int j = 0; j < 2; ++j)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int key = T.tb + 16 * j + 4 * b + r;
-                const bool ok = T.ok[j] && key >= kbegin_c && key < kstop_c;
-                sv[j][r] = ok ? s[j][r] * a.scale : -INFINITY;
-                tile_max = fmaxf(tile_max, sv[j][r]);
+                const bool ok = ((T.ok >> j) & 1) && key >= kbegin_c && key < kstop_c;
+                sv[j][r] = ok ? s[j][r] * c2 : -INFINITY;
             }
+        float tile_max = fmaxf(fmaxf(fmaxf(sv[0][0], sv[0][1]), fmaxf(sv[0][2], sv[0][3])),
+                               fmaxf(fmaxf(sv[1][0], sv[1][1]), fmaxf(sv[1][2], sv[1][3])));
         tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, MLR_WAVE));
         tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, MLR_WAVE));
-        const float m_new = fmaxf(m_run, tile_max);
-        float corr = 1.f;
-        bf16x8 pf = zero8;
-        if (m_new > -INFINITY) {
-            corr = __expf(m_run - m_new);              // m_run = -inf gives 0
-            float psum = 0.f;
+        // the running maximum rarely moves after the first tiles: rescale only when it does, for any column
+        if (__builtin_amdgcn_ballot_w64(tile_max > m_run) != 0) {
+            const float m_new = fmaxf(m_run, tile_max);
+            const float corr = m_new > -INFINITY ? __builtin_amdgcn_exp2f(m_run - m_new) : 1.f;   // -inf - finite: 0
+            l_run *= corr;
 #pragma unroll
-            for (int j = 0; j < 2; ++j)
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const float p = sv[j][r] > -INFINITY ? __expf(sv[j][r] - m_new) : 0.f;
-                    psum += p;
-                    pf[4 * j + r] = (__bf16)p;
-                }
-            l_run = l_run * corr + psum;
+            for (int db = 0; db < 2 * NCH; ++db) o[db] *= corr;
             m_run = m_new;
         }
-        const bool tail = T.tb + MFMA_TILE_KEYS > ke;  // some keys of the tile are not written yet
+        const float m_use = fmaxf(m_run, -1e30f);      // a column with no key yet: exp2(-inf - finite) = 0, not NaN
+        bf16x8 pf;
+        float psum = 0.f;
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float p = __builtin_amdgcn_exp2f(sv[j][r] - m_use);
+                psum += p;
+                pf[4 * j + r] = (__bf16)p;
+            }
+        l_run += psum;
+        // values of keys that are not written yet (or of a page that is not there) must count as zero: a
+        // probability of zero does not cancel a NaN.  Only a workgroup's last tile can hold such keys.
+        const bool ragged = T.ok != 3 || T.tb + MFMA_TILE_KEYS > ke;
 #pragma unroll
         for (int db = 0; db < 2 * NCH; ++db) {
             if (16 * db >= D) break;
-            o[db] *= corr;
-            bf16x8 vf;
+            bf16x4 v0 = T.v[db][0], v1 = T.v[db][1];
+            if (ragged) {
 #pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                bf16x4 v4 = T.v[db][j];
-                if (tail) {
-#pragma unroll
-                    for (int r = 0; r < 4; ++r)
-                        if (T.tb + 16 * j + 4 * b + r >= ke) v4[r] = (__bf16)0.f;
+                for (int r = 0; r < 4; ++r) {
+                    if (!(T.ok & 1) || T.tb + 4 * b + r >= ke) v0[r] = (__bf16)0.f;
+                    if (!(T.ok & 2) || T.tb + 16 + 4 * b + r >= ke) v1[r] = (__bf16)0.f;
                 }
-#pragma unroll
-                for (int r = 0; r < 4; ++r) vf[4 * j + r] = v4[r];
             }
+            const bf16x8 vf = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
             o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, o[db], 0, 0, 0);
         }
     };
 
     {
+        // two tiles under way per wavefront: one being multiplied, one in flight; fetches are unconditional
+        // (clamped to the wavefront's last tile) for the reason given above
         KvTile<NCH> ta, tb2;
-        int t = lo / MFMA_TILE_KEYS + wave;
-        const int t_end = (hi + MFMA_TILE_KEYS - 1) / MFMA_TILE_KEYS;
+        int t = t_begin + wave;
         if (t < t_end) {
-            TilePages pa = lookup(t);
-            TilePages pb = lookup(t + 4);
-            load(t, pa, ta);
+            const int t_last = t + ((t_end - 1 - t) / 4) * 4;
+            load(t, ta);
             for (;;) {
-                const bool more_b = t + 4 < t_end;
-                pa = lookup(t + 8);
-                if (more_b) load(t + 4, pb, tb2);
+                load(min(t + 4, t_last), tb2);
                 compute(ta);
-                if (!more_b) break;
-                const bool more_a = t + 8 < t_end;
-                pb = lookup(t + 12);
-                if (more_a) load(t + 8, pa, ta);
+                if (t + 4 >= t_end) break;
+                load(min(t + 8, t_last), ta);
                 compute(tb2);
-                if (!more_a) break;
+                if (t + 8 >= t_end) break;
                 t += 8;
             }
         }
@@ -497,7 +506,7 @@ __global__ __launch_bounds__(256, (NCH <= 4 ? 2 : 1)) void attention_mfma_kernel
         float l_tot = 0.f;
         float own = 0.f;
         if (m_tot > -INFINITY) {
-            own = m_run > -INFINITY ? __expf(m_run - m_tot) : 0.f;
+            own = m_run > -INFINITY ? __builtin_amdgcn_exp2f(m_run - m_tot) : 0.f;
             l_tot = l_run * own;
         }
 #pragma unroll
@@ -506,7 +515,7 @@ __global__ __launch_bounds__(256, (NCH <= 4 ? 2 : 1)) void attention_mfma_kernel
             const float* src = lds + (size_t)w * stride;
             const float mw = src[16 * D + col];
             if (!(mw > -INFINITY)) continue;
-            const float f = __expf(mw - m_tot);
+            const float f = __builtin_amdgcn_exp2f(mw - m_tot);
             l_tot += src[16 * D + 16 + col] * f;
 #pragma unroll
             for (int db = 0; db < 2 * NCH; ++db) {
@@ -817,7 +826,7 @@ __global__ __launch_bounds__(64) void attention_combine_groups_kernel(AttnArgs a
         __syncthreads();
         for (int s = threadIdx.x; s < n; s += 64) {
             const float smax = w_lds[s];
-            w_lds[s] = smax > -INFINITY ? __expf(smax - gmax) : 0.f;
+            w_lds[s] = smax > -INFINITY ? __builtin_amdgcn_exp2f(smax - gmax) : 0.f;   // maxima are base-2 exponents
         }
         __syncthreads();
         float den = 0.f;
@@ -856,6 +865,8 @@ extern "C" int mlr_attention_mfma(
         q_heads / kv_heads > 16) return -1;
     if (max_splits > 1 && (partial == nullptr || split_keys <= 0 || split_keys % MFMA_TILE_KEYS != 0 ||
                            max_splits > COMBINE_MAX_SPLITS)) return -2;
+    // a workgroup keeps the page ids of its key range in LDS
+    if ((max_splits > 1 ? split_keys / page_size + 2 : max_blocks) > DECODE_PAGE_CACHE) return -3;
     AttnArgs a{(const elem_t*)q, (const elem_t*)k_pages, (const elem_t*)v_pages, block_table, slots,
                positions, (elem_t*)out, partial, max_blocks, q_heads, kv_heads, head_dim, page_size,
                window, split_keys, max_splits < 1 ? 1 : max_splits, scale};

@@ -275,6 +275,8 @@ class Kernels:
             _tensor(partial, "partial", torch.float32, ndim=1)
             _need(partial.numel() >= self.attention_partial_numel(m, q_heads, head_dim, max_splits),
                   "partial buffer too small")
+        _need((split_keys // page_size + 2 if max_splits > 1 else block_table.shape[1]) <= 4096,
+              "attention_mfma: a workgroup's key range spans more than 4096 pages; split the keys")
         fn = self._lib("attention").mlr_attention_mfma
         _ok(fn(_p(q), _p(k_pages), _p(v_pages), _p(block_table), _c_int(block_table.shape[1]), _p(slots),
                _p(positions), _p(out), _p(partial), _p(group_row0), _p(group_ntok), _c_int(groups), _c_int(m),
