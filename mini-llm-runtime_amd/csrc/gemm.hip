@@ -239,6 +239,113 @@ __global__ __launch_bounds__(SKINNY_WAVES * 64) void gemm_skinny_kernel(const __
     }
 }
 
+// Up to 16 rows: the residual add and the RMSNorm that precede a projection, done inside it.
+//   x = h_in + delta (delta may be null);  h_out = x (written by workgroup 0; h_out != h_in);
+//   out = (bf16((x * rsqrt(mean(x^2) + eps)) * norm_w)) . w^T      [GATED: silu(. gate) * (. up)]
+// Every workgroup recomputes the norm of the few rows (they come from the L2 cache); each wavefront
+// holds the slice of x that belongs to its part of k, the sums of squares meet in LDS and are added in
+// the order of the wavefronts.  K <= 2048 (a lane keeps its slice in registers).
+#define NORM_MAX_STEPS 8                              // 32-wide k steps per wavefront: K <= 8 * 8 * 32
+template <bool GATED, int PW>                         // PW: k steps a wavefront takes (1, 2, 4 or 8)
+__global__ __launch_bounds__(SKINNY_WAVES * 64) void gemm_skinny_norm_kernel(
+    const float* __restrict__ h_in, const __bf16* __restrict__ delta, const float* __restrict__ norm_w, float eps,
+    float* __restrict__ h_out, const __bf16* __restrict__ w, __bf16* __restrict__ out, int M, int N, int K) {
+    constexpr int NW = GATED ? 2 : 1;
+    __shared__ float part[SKINNY_WAVES - 1][NW][64][4];
+    __shared__ float sumsq[SKINNY_WAVES][16];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r16 = lane & 15, b = lane >> 4;
+    const int n0 = blockIdx.x * 16;
+    const int steps = K / 32;                         // K % 32 == 0
+    const int s_begin = wave * PW, s_end = min(steps, s_begin + PW);
+    const bool row_ok = r16 < M;
+
+    // the weight first: its loads fly while the norm is computed (no branch around a load; a wavefront
+    // beyond the end of k re-reads the last step and ignores it)
+    bf16x8 wf[NW][PW];
+#pragma unroll
+    for (int i = 0; i < PW; ++i) {
+        const int k = min(s_begin + i, steps - 1) * 32 + b * 8;
+#pragma unroll
+        for (int g = 0; g < NW; ++g)
+            wf[g][i] = *reinterpret_cast<const bf16x8*>(w + ((size_t)g * N + min(n0 + r16, N - 1)) * K + k);
+    }
+    float x[PW][8];
+    float sq = 0.f;
+#pragma unroll
+    for (int i = 0; i < PW; ++i) {
+        const int s = s_begin + i;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[i][e] = 0.f;
+        if (s < s_end && row_ok) {
+            const size_t at = (size_t)r16 * K + s * 32 + b * 8;
+            const float4 a0 = *reinterpret_cast<const float4*>(h_in + at);
+            const float4 a1 = *reinterpret_cast<const float4*>(h_in + at + 4);
+            x[i][0] = a0.x; x[i][1] = a0.y; x[i][2] = a0.z; x[i][3] = a0.w;
+            x[i][4] = a1.x; x[i][5] = a1.y; x[i][6] = a1.z; x[i][7] = a1.w;
+            if (delta) {
+                const bf16x8 d8 = *reinterpret_cast<const bf16x8*>(delta + at);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) x[i][e] += (float)d8[e];
+            }
+            if (h_out && blockIdx.x == 0) {
+                *reinterpret_cast<float4*>(h_out + at) = make_float4(x[i][0], x[i][1], x[i][2], x[i][3]);
+                *reinterpret_cast<float4*>(h_out + at + 4) = make_float4(x[i][4], x[i][5], x[i][6], x[i][7]);
+            }
+#pragma unroll
+            for (int e = 0; e < 8; ++e) sq += x[i][e] * x[i][e];
+        }
+    }
+    sq += __shfl_xor(sq, 16, MLR_WAVE);
+    sq += __shfl_xor(sq, 32, MLR_WAVE);
+    if (b == 0) sumsq[wave][r16] = sq;
+    __syncthreads();
+    float total = 0.f;
+#pragma unroll
+    for (int i = 0; i < SKINNY_WAVES; ++i) total += sumsq[i][r16];
+    const float scale = 1.0f / sqrtf(total / (float)K + eps);
+
+    floatx4 acc[NW];
+#pragma unroll
+    for (int g = 0; g < NW; ++g) acc[g] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < PW; ++i) {
+        const int s = s_begin + i;
+        if (s >= s_end) break;
+        const int k = s * 32 + b * 8;
+        const float4 w0 = *reinterpret_cast<const float4*>(norm_w + k);
+        const float4 w1 = *reinterpret_cast<const float4*>(norm_w + k + 4);
+        const float nw[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+        bf16x8 xf;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) xf[e] = (__bf16)((x[i][e] * scale) * nw[e]);
+#pragma unroll
+        for (int g = 0; g < NW; ++g)
+            acc[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[g][i], xf, acc[g], 0, 0, 0);
+    }
+    if (wave > 0) {
+#pragma unroll
+        for (int g = 0; g < NW; ++g)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) part[wave - 1][g][lane][r] = acc[g][r];
+    }
+    __syncthreads();
+    if (wave != 0) return;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        float v[NW];
+#pragma unroll
+        for (int g = 0; g < NW; ++g) {
+            v[g] = acc[g][r];
+            for (int p = 0; p < SKINNY_WAVES - 1; ++p) v[g] += part[p][g][lane][r];
+        }
+        float y = v[0];
+        if (GATED) y = (v[0] / (1.0f + expf(-v[0]))) * v[NW - 1];
+        const int n = n0 + 4 * b + r;
+        if (row_ok && n < N) out[(size_t)r16 * N + n] = (__bf16)y;
+    }
+}
+
 template <int MT, bool GATED>
 static int launch_skinny(const void* a, const void* w, void* out, int M, int N, int K, int out_float,
                          hipStream_t stream) {
@@ -289,5 +396,32 @@ extern "C" int mlr_gemm_gated_silu(const void* a, const void* w, void* out, int 
     if (M <= 32) return launch_skinny<2, true>(a, w, out, M, N, K, 0, stream);
     if (M <= 64) return launch_skinny<4, true>(a, w, out, M, N, K, 0, stream);
     return 1;
+}
+
+// Residual add + RMSNorm + projection in one launch, for M <= 16, K % 32 == 0, K <= 2048 (see the kernel).
+// gated != 0: w is [2N, K] = [gate; up] and out = silu(gate) * up.
+extern "C" int mlr_norm_gemm(const float* h_in, const void* delta, const float* norm_w, float eps, float* h_out,
+                             const void* w, void* out, int M, int N, int K, int gated, hipStream_t stream) {
+    if (M <= 0 || N <= 0) return 0;
+    if (M > 16 || K <= 0 || K % 32 != 0 || K > 32 * SKINNY_WAVES * NORM_MAX_STEPS) return -1;
+    if (h_out == h_in) return -2;
+    dim3 grid((N + 15) / 16);
+    const int per_wave = (K / 32 + SKINNY_WAVES - 1) / SKINNY_WAVES;
+#define MLR_NORM_LAUNCH(G, PWV)                                                                      \
+    gemm_skinny_norm_kernel<G, PWV><<<grid, SKINNY_WAVES * 64, 0, stream>>>(                          \
+        h_in, (const __bf16*)delta, norm_w, eps, h_out, (const __bf16*)w, (__bf16*)out, M, N, K)
+    if (gated) {
+        if (per_wave <= 1) MLR_NORM_LAUNCH(true, 1);
+        else if (per_wave <= 2) MLR_NORM_LAUNCH(true, 2);
+        else if (per_wave <= 4) MLR_NORM_LAUNCH(true, 4);
+        else MLR_NORM_LAUNCH(true, 8);
+    } else {
+        if (per_wave <= 1) MLR_NORM_LAUNCH(false, 1);
+        else if (per_wave <= 2) MLR_NORM_LAUNCH(false, 2);
+        else if (per_wave <= 4) MLR_NORM_LAUNCH(false, 4);
+        else MLR_NORM_LAUNCH(false, 8);
+    }
+#undef MLR_NORM_LAUNCH
+    return (int)hipGetLastError();
 }
 #endif

@@ -173,6 +173,30 @@ class Kernels:
         fn = self._lib("gemm").mlr_gemm_gated_silu
         _ok(fn(_p(a), _p(w), _p(out), _c_int(m), _c_int(two_n // 2), _c_int(k), _stream()), "gemm_gated_silu")
 
+    def norm_gemm_supported(self, rows, width):
+        """Whether `norm_gemm` (residual add + RMSNorm inside the projection) serves these sizes."""
+        return self.dtype == torch.bfloat16 and rows <= 16 and width % 32 == 0 and width <= 2048
+
+    def norm_gemm(self, h_in, delta, norm_w, eps, h_out, w, out, gated=False):
+        """x = h_in + delta (delta may be None); h_out = x; out = rmsnorm(x, norm_w) . w^T, or with
+        gated=True (w = [gate; up] stacked) silu(. gate^T) * (. up^T).  For few rows: one launch instead
+        of two."""
+        _tensor(h_in, "h_in", torch.float32, ndim=2)
+        m, k = h_in.shape
+        _need(self.norm_gemm_supported(m, k), "norm_gemm: bfloat16, at most 16 rows, width % 32 == 0 and <= 2048")
+        if delta is not None:
+            _tensor(delta, "delta", self.dtype, (m, k))
+        _tensor(norm_w, "norm_w", torch.float32, (k,))
+        _tensor(h_out, "h_out", torch.float32, (m, k))
+        _need(h_out.data_ptr() != h_in.data_ptr(), "norm_gemm: h_out must not be h_in")
+        _tensor(w, "w", self.dtype, ndim=2)
+        n = w.shape[0] // 2 if gated else w.shape[0]
+        _need(w.shape[1] == k and (not gated or w.shape[0] % 2 == 0), "norm_gemm: weight does not fit")
+        _tensor(out, "out", self.dtype, (m, n))
+        fn = self._lib("gemm").mlr_norm_gemm
+        _ok(fn(_p(h_in), _p(delta), _p(norm_w), _c_float(eps), _p(h_out), _p(w), _p(out), _c_int(m), _c_int(n),
+               _c_int(k), _c_int(1 if gated else 0), _stream()), "norm_gemm")
+
     # -- attention ---------------------------------------------------------------------------
     def _check_cache(self, k_pages, v_pages, kv_heads, head_dim, page_size):
         _tensor(k_pages, "k_pages", self.dtype, ndim=4)

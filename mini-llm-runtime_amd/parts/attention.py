@@ -61,13 +61,28 @@ class GqaAttention:
     def libraries(self):
         return ["gemm", "rope_kv", "attention"]
 
+    def forward_prenorm(self, ctx, h, delta, norm, h_out, cache_id, write_cache=True):
+        """As `forward` on norm(h + delta), the residual add and the norm done inside the first
+        projection (few rows); h_out receives h + delta."""
+        s = self.spec
+        m = h.shape[0]
+        qkv = ctx.workspace.get("qkv", (m, (s.q_heads + 2 * s.kv_heads) * s.head_dim), ctx.dtype)
+        ctx.kernels.norm_gemm(h, delta, norm.weight, norm.eps, h_out, self.qkv, qkv)
+        return self._attend(ctx, qkv, cache_id, write_cache)
+
     def forward(self, ctx, x, cache_id, write_cache=True):
         s = self.spec
-        k = ctx.kernels
         m = x.shape[0]
-        view = ctx.cache.kv_view(cache_id)
         qkv = ctx.workspace.get("qkv", (m, (s.q_heads + 2 * s.kv_heads) * s.head_dim), x.dtype)
-        k.gemm(x, self.qkv, qkv)
+        ctx.kernels.gemm(x, self.qkv, qkv)
+        return self._attend(ctx, qkv, cache_id, write_cache)
+
+    def _attend(self, ctx, qkv, cache_id, write_cache):
+        s = self.spec
+        k = ctx.kernels
+        x = qkv
+        m = qkv.shape[0]
+        view = ctx.cache.kv_view(cache_id)
         q = ctx.workspace.get("q", (m, s.q_heads * s.head_dim), x.dtype)
         rope = self.position.rotation_table(ctx.max_positions, x.device) if self.position is not None else None
         k.qk_norm_rope_kv(

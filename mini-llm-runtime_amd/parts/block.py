@@ -20,6 +20,14 @@ class PreNormBlock:
         return {"norm1": self.norm1, "mixer": self.mixer, "norm2": self.norm2, "ffn": self.ffn}
 
     def forward(self, ctx, h, pending, cache_id, write_cache=True):
+        if (ctx.kernels.norm_gemm_supported(h.shape[0], h.shape[1])
+                and getattr(self.norm1, "fusable_rmsnorm", False) and getattr(self.norm2, "fusable_rmsnorm", False)
+                and hasattr(self.mixer, "forward_prenorm") and hasattr(self.ffn, "forward_prenorm")):
+            # few rows: each norm rides in the projection that follows it; the residual stream goes to a
+            # second buffer and back, so that no workgroup reads a row that another one is updating
+            h_alt = ctx.workspace.get("hidden_alt", tuple(h.shape), h.dtype)
+            mixed = self.mixer.forward_prenorm(ctx, h, pending, self.norm1, h_alt, cache_id, write_cache)
+            return self.ffn.forward_prenorm(ctx, h_alt, mixed, self.norm2, h)
         normed = ctx.workspace.get("normed", tuple(h.shape), ctx.dtype)
         self.norm1.forward(ctx, h, pending, normed)
         mixed = self.mixer.forward(ctx, normed, cache_id, write_cache)

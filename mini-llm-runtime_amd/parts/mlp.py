@@ -31,6 +31,16 @@ class SwiGluMlp:
     def libraries(self):
         return ["gemm", "elementwise"]
 
+    def forward_prenorm(self, ctx, h, delta, norm, h_out):
+        """As `forward` on norm(h + delta), add and norm done inside the first projection (few rows)."""
+        s = self.spec
+        m = h.shape[0]
+        act = ctx.workspace.get("act", (m, s.intermediate), ctx.dtype)
+        ctx.kernels.norm_gemm(h, delta, norm.weight, norm.eps, h_out, self.gate_up, act, gated=True)
+        out = ctx.workspace.get("ffn_out", (m, s.hidden), ctx.dtype)
+        ctx.kernels.gemm(act, self.down, out)
+        return out
+
     def forward(self, ctx, x):
         s = self.spec
         m = x.shape[0]

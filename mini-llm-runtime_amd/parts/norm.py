@@ -10,6 +10,7 @@ from .registry import register_part
 @register_part("norm", "rmsnorm")
 class RmsNorm:
     graph_safe = True        # forward launches kernels over the step's device vectors only
+    fusable_rmsnorm = True   # a following projection may do this norm itself (weight, eps as here)
     def __init__(self, spec):
         self.size, self.eps = spec.size, float(spec.eps)
         self.weight = None

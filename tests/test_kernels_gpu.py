@@ -591,3 +591,31 @@ def test_silu_mul_wide(dtype, inter):
     k.silu_mul(gate_up, act)
     g, u = gate_up.double()[:, :inter], gate_up.double()[:, inter:]
     torch.testing.assert_close(act.double(), g / (1 + torch.exp(-g)) * u, **tol(dtype))
+
+
+@pytest.mark.parametrize("gated", [False, True])
+@pytest.mark.parametrize("mnk", [(1, 48, 64), (8, 4096, 1024), (16, 100, 1024), (5, 208, 96), (3, 40, 2048), (7, 24, 32)])
+def test_norm_gemm(mnk, gated):
+    """Residual add + RMSNorm inside the projection (few rows, bfloat16): h_out = h + delta and
+    out = rmsnorm(h + delta) W^T (or the gated activation of two such products)."""
+    m, n, kk = mnk
+    k = kernels(torch.bfloat16)
+    assert k.norm_gemm_supported(m, kk) and not k.norm_gemm_supported(17, kk) and not k.norm_gemm_supported(m, 40)
+    h = rnd((m, kk), torch.float32, 90, 2.0)
+    delta = rnd((m, kk), torch.bfloat16, 91)
+    nw = rnd((kk,), torch.float32, 92) + 1
+    w = rnd(((2 if gated else 1) * n, kk), torch.bfloat16, 93, 0.2)
+    eps = 1e-5
+    for d in (delta, None):
+        h_out = torch.full((m, kk), float("nan"), device="cuda")
+        out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+        k.norm_gemm(h, d, nw, eps, h_out, w, out, gated=gated)
+        x = h.double() + (d.double() if d is not None else 0)
+        torch.testing.assert_close(h_out.double(), x, atol=1e-6, rtol=1e-6)
+        xn = (x * torch.rsqrt((x * x).mean(-1, keepdim=True) + eps) * nw.double()).to(torch.bfloat16).double()
+        if gated:
+            g, u = xn @ w.double()[:n].T, xn @ w.double()[n:].T
+            want = g / (1 + torch.exp(-g)) * u
+        else:
+            want = xn @ w.double().T
+        torch.testing.assert_close(out.double(), want, atol=2e-2 * float(want.abs().max()), rtol=2e-2)
