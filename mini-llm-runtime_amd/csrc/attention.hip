@@ -834,13 +834,14 @@ __global__ __launch_bounds__(64) void attention_combine_groups_kernel(AttnArgs a
         float num[MAX_DIM_REGS];
 #pragma unroll
         for (int i = 0; i < MAX_DIM_REGS; ++i) num[i] = 0.f;
+#pragma unroll 8
         for (int s = 0; s < n; ++s) {
             const float w = w_lds[s];
             const float* p = base + (size_t)s * (D + 2);
 #pragma unroll
             for (int i = 0; i < MAX_DIM_REGS; ++i) {
-                const int d = threadIdx.x + 64 * i;
-                if (d < D) num[i] += w * p[d];
+                const int d = min((int)threadIdx.x + 64 * i, D - 1);      // clamped: no branch around the load
+                num[i] += w * p[d];
             }
         }
 #pragma unroll

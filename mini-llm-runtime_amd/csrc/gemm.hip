@@ -193,18 +193,50 @@ __global__ __launch_bounds__(SKINNY_WAVES * 64) void gemm_skinny_kernel(const __
     for (int g = 0; g < NW; ++g)
 #pragma unroll
         for (int i = 0; i < MT; ++i) acc[g][i] = floatx4{0.f, 0.f, 0.f, 0.f};
+    if ((K & 31) == 0) {
+        // The usual case, K a multiple of 32: no branch anywhere near a load (a load behind a branch makes
+        // the compiler wait for every load in flight).  Rows beyond N or M read the last valid row; what
+        // they produce is never stored.  Eight steps' worth of weight loads are issued before they are used.
+        const __bf16* wrow = w + (size_t)min(n0 + r16, N - 1) * K + b * 8;
+        const __bf16* xrow[MT];
+#pragma unroll
+        for (int i = 0; i < MT; ++i) xrow[i] = a + (size_t)min(16 * i + r16, M - 1) * K + b * 8;
+        constexpr int U = 8;
+        for (int s0 = s_begin; s0 < s_end; s0 += U) {
+            bf16x8 wf[NW][U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int k = min(s0 + u, s_end - 1) * 32;
+#pragma unroll
+                for (int g = 0; g < NW; ++g) wf[g][u] = *reinterpret_cast<const bf16x8*>(wrow + (size_t)g * N * K + k);
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                if (s0 + u >= s_end) break;
+                const int k = (s0 + u) * 32;
+#pragma unroll
+                for (int i = 0; i < MT; ++i) {
+                    const bf16x8 xf = *reinterpret_cast<const bf16x8*>(xrow[i] + k);
+#pragma unroll
+                    for (int g = 0; g < NW; ++g)
+                        acc[g][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[g][u], xf, acc[g][i], 0, 0, 0);
+                }
+            }
+        }
+    } else {
 #pragma unroll 4
-    for (int s = s_begin; s < s_end; ++s) {
-        const int k = s * 32 + b * 8;
-        bf16x8 wf[NW];
+        for (int s = s_begin; s < s_end; ++s) {
+            const int k = s * 32 + b * 8;
+            bf16x8 wf[NW];
 #pragma unroll
-        for (int g = 0; g < NW; ++g) wf[g] = load_k8(w + (size_t)g * N * K, n0 + r16, N, k, K, vector_ok);
+            for (int g = 0; g < NW; ++g) wf[g] = load_k8(w + (size_t)g * N * K, n0 + r16, N, k, K, vector_ok);
 #pragma unroll
-        for (int i = 0; i < MT; ++i) {
-            const bf16x8 xf = load_k8(a, 16 * i + r16, M, k, K, vector_ok);
+            for (int i = 0; i < MT; ++i) {
+                const bf16x8 xf = load_k8(a, 16 * i + r16, M, k, K, vector_ok);
 #pragma unroll
-            for (int g = 0; g < NW; ++g)
-                acc[g][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[g], xf, acc[g][i], 0, 0, 0);
+                for (int g = 0; g < NW; ++g)
+                    acc[g][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[g], xf, acc[g][i], 0, 0, 0);
+            }
         }
     }
     if (wave > 0) {
