@@ -1,0 +1,74 @@
+"""The engine at the widths of the benchmark model (hidden 1024, 16 q / 8 kv heads of 128, feed-forward
+3072, vocabulary 151936, tied), with two layers so that the plain implementation stays quick: a 256-token
+prompt whole, in portions and with its last tokens decoded one by one, in 32-bit and in bfloat16, against
+the plain logits.  Tiny models cannot show a fault that needs a head of 128 channels, sixteen query heads
+or a vocabulary that fills many workgroups."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import compare, make_requests
+
+pytestmark = pytest.mark.gpu
+
+CFG = dict(architectures=["Qwen3ForCausalLM"], hidden_size=1024, num_hidden_layers=2, num_attention_heads=16,
+           num_key_value_heads=8, head_dim=128, intermediate_size=3072, vocab_size=151936,
+           max_position_embeddings=4096, rms_norm_eps=1e-6, rope_theta=1000000.0, tie_word_embeddings=True)
+WANT = [0, 1, 15, 16, 17, 32, 127, 128, 255]          # the reference's probe positions (tests/data/qwen3_validation_cases.json)
+
+
+@pytest.fixture(scope="module")
+def folder(tmp_path_factory):
+    from mini_llm_runtime_amd.config import config_from_dict
+    from mini_llm_runtime_amd.weights import write_random_model
+    path = str(tmp_path_factory.mktemp("real-sizes"))
+    # N(0, 0.02) as in the benchmark; norm weights 1 + N(0, 0.1)
+    write_random_model(path, config_from_dict(CFG), seed=7)
+    return path
+
+
+@pytest.fixture(scope="module")
+def expected(folder):
+    from plain.qwen3_plain import PlainQwen3
+    toks = make_requests(CFG["vocab_size"], [256], seed=17)["r0"]
+    plain = PlainQwen3(folder)
+    rows = plain.logits(toks, WANT)
+    return toks, {("r0", p): rows[i] for i, p in enumerate(WANT)}
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_prompt_of_256_tokens_every_way(folder, expected, dtype_name):
+    from helpers import run_steps
+    from mini_llm_runtime_amd.engine import Runner
+    from mini_llm_runtime_amd.parts import DecoderModel
+    toks, want = expected
+    model = DecoderModel.load(folder, torch.float32 if dtype_name == "float32" else torch.bfloat16)
+    r = Runner(model, max_tokens=512, max_slots=2, page_size=16)
+
+    def wanted(lo, hi):
+        return [p - lo for p in WANT if lo <= p < hi]
+    whole = [dict(step=0, entries=[dict(id="r0", tokens=toks, want=WANT)], end=["r0"])]
+    cuts = [0, 7, 16, 18, 100, 128, 224]
+    portions = [dict(step=i, entries=[dict(id="r0", tokens=toks[lo:hi], want=wanted(lo, hi))], end=[])
+                for i, (lo, hi) in enumerate(zip(cuts, cuts[1:]))]
+    portions += [dict(step=100 + p, entries=[dict(id="r0", tokens=[toks[p]], want=wanted(p, p + 1))], end=[])
+                 for p in range(224, 256)]
+    portions[-1]["end"] = ["r0"]
+    results = []
+    for steps in (whole, portions):
+        got = run_steps(r, steps)
+        compare(got, want, dtype_name)
+        results.append(got)
+    scale = max(float(np.abs(v).max()) for v in want.values())
+    limit = 2e-5 if dtype_name == "float32" else 0.03 * scale
+    assert max(float(np.abs(results[0][k] - results[1][k]).max()) for k in want) <= limit
+    # greedy continuation through the sampler: the plain argmax of the last position
+    from mini_llm_runtime_amd.sampling import Sampler
+    from mini_llm_runtime_amd.engine import Entry
+    s = r.open_request()
+    logits = r.step([Entry(s, toks, [255])])
+    token = Sampler(r.kernels, r.device, 1).sample(logits, [0.0], [0.0])[0]
+    row = want[("r0", 255)]
+    top = np.sort(row)[-2:]
+    if dtype_name == "float32" or top[1] - top[0] > 0.05 * np.abs(row).max():
+        assert token == int(np.argmax(row))
