@@ -12,7 +12,6 @@ import argparse
 import json
 import os
 import sys
-import tempfile
 import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
@@ -20,10 +19,18 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK = 8.0e12              # bytes/s, MI355X
 MFMA_PEAK = {"bf16": 2.5e15, "fp32": 157.3e12}
-SIZES = dict(hidden_size=1024, num_attention_heads=16, num_key_value_heads=8, head_dim=128,
-             intermediate_size=3072, vocab_size=151936, max_position_embeddings=40960, rms_norm_eps=1e-6,
-             rope_theta=1000000.0, tie_word_embeddings=True)
-FULL_LAYERS = 28
+# layer sizes of the Qwen3 dense family; the default is the 0.6B one
+SIZES = {
+    "0.6b": (28, dict(hidden_size=1024, num_attention_heads=16, num_key_value_heads=8, head_dim=128,
+                      intermediate_size=3072, vocab_size=151936, max_position_embeddings=40960,
+                      rms_norm_eps=1e-6, rope_theta=1000000.0, tie_word_embeddings=True)),
+    "8b": (36, dict(hidden_size=4096, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
+                    intermediate_size=12288, vocab_size=151936, max_position_embeddings=40960,
+                    rms_norm_eps=1e-6, rope_theta=1000000.0, tie_word_embeddings=False)),
+    "32b": (64, dict(hidden_size=5120, num_attention_heads=64, num_key_value_heads=8, head_dim=128,
+                     intermediate_size=25600, vocab_size=151936, max_position_embeddings=40960,
+                     rms_norm_eps=1e-6, rope_theta=1000000.0, tie_word_embeddings=False)),
+}
 PREFILL_TOKENS = 2048
 
 
@@ -32,7 +39,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=8)
-    ap.add_argument("--layers", type=int, default=FULL_LAYERS)
+    ap.add_argument("--size", default="0.6b", choices=sorted(SIZES), help="layer sizes of which Qwen3 dense model")
+    ap.add_argument("--layers", type=int, default=0, help="fewer layers than the model has (0: all of them)")
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--context", type=int, default=4096)
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
@@ -51,21 +59,33 @@ def main():
     from mini_llm_runtime_amd.api import parse_dtype
     from mini_llm_runtime_amd.config import config_from_dict
     from mini_llm_runtime_amd.engine import Entry, Runner
-    from mini_llm_runtime_amd.parts import DecoderModel
+    from mini_llm_runtime_amd.parts import DecoderModel, expected_tensors
     from mini_llm_runtime_amd.sampling import Sampler
-    from mini_llm_runtime_amd.weights import write_random_model
 
     dtype = parse_dtype(args.dtype)
     tag = "bf16" if dtype == torch.bfloat16 else "fp32"
-    cfg = config_from_dict(dict(SIZES, architectures=["Qwen3ForCausalLM"], num_hidden_layers=args.layers))
-    with tempfile.TemporaryDirectory(prefix="mlr-bench-") as folder:
-        write_random_model(folder, cfg, seed=0)
-        model = DecoderModel.load(folder, dtype)
+    FULL_LAYERS, sizes = SIZES[args.size]
+    if args.layers <= 0:
+        args.layers = FULL_LAYERS
+    cfg = config_from_dict(dict(sizes, architectures=["Qwen3ForCausalLM"], num_hidden_layers=args.layers))
+    # Random weights N(0, 0.02) (norm weights 1 + N(0, 0.1)) drawn on the GPU: the same tensors that the
+    # random-weights mode would write to a model folder, without the trip through a file of many gigabytes.
+    torch.manual_seed(0)
+    weights = {}
+    for name, spec in expected_tensors(cfg).items():
+        if spec.optional:
+            continue
+        if spec.keep_float32:
+            weights[name] = 1.0 + 0.1 * torch.randn(spec.shape, device="cuda", dtype=torch.float32)
+        else:
+            weights[name] = (0.02 * torch.randn(spec.shape, device="cuda", dtype=torch.float32)).to(dtype)
+    model = DecoderModel(cfg, weights, dtype, "cuda:0")
+    del weights
     c = cfg
     layer_params = c.hidden_size * (c.num_attention_heads + 2 * c.num_key_value_heads) * c.head_dim \
         + c.num_attention_heads * c.head_dim * c.hidden_size + 3 * c.hidden_size * c.intermediate_size
     elem = 2 if dtype == torch.bfloat16 else 4
-    weight_bytes = (args.layers * layer_params + c.vocab_size * c.hidden_size) * elem
+    weight_bytes = (args.layers * layer_params + c.vocab_size * c.hidden_size) * elem     # layers + output projection
     kv_bytes_per_token = args.layers * 2 * c.num_key_value_heads * c.head_dim * elem
     g = torch.Generator().manual_seed(0)
 
@@ -137,15 +157,16 @@ def main():
     step_bytes = weight_bytes + args.batch * mean_context * kv_bytes_per_token
     achieved = step_bytes / (seconds / args.steps) / 1e9
     line = {
-        "metric": "decode tok/s, Qwen3-0.6B sizes, batch 8, context 4096", "value": round(value, 1),
+        "metric": f"decode tok/s, Qwen3-{args.size.upper()} sizes, batch {args.batch}, context {args.context}",
+        "value": round(value, 1),
         "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": tag, "data": "synthetic token ids, random weights N(0, 0.02)",
-        "config": {"model": "Qwen3-0.6B sizes", "layers": args.layers, "layers_full": FULL_LAYERS,
+        "config": {"model": f"Qwen3-{args.size.upper()} sizes", "layers": args.layers, "layers_full": FULL_LAYERS,
                    "hidden_size": c.hidden_size, "q_heads": c.num_attention_heads,
                    "kv_heads": c.num_key_value_heads, "head_dim": c.head_dim,
                    "intermediate_size": c.intermediate_size, "vocab_size": c.vocab_size,
-                   "tied_embeddings": True, "rope_theta": c.rope_theta, "rms_norm_eps": c.rms_norm_eps,
+                   "tied_embeddings": c.tie_word_embeddings, "rope_theta": c.rope_theta, "rms_norm_eps": c.rms_norm_eps,
                    "global_batch": args.batch, "seq_len": args.context, "page_size": 16,
                    "sampling": "greedy", "parallelism": "single GPU"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
