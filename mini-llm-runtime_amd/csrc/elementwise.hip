@@ -49,6 +49,67 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ h, const elem_t* __restri
     }
 }
 
+// One workgroup per row as above, 16 bytes per thread and access (width a multiple of MLR_VEC): for few
+// rows of the bfloat16 engine, where the scalar kernel's latency would show.
+__global__ __launch_bounds__(256) void add_rmsnorm_row_vec_kernel(float* __restrict__ h, const elem_t* __restrict__ delta,
+                                                                  const float* __restrict__ weight,
+                                                                  elem_t* __restrict__ out, const int32_t* __restrict__ rows,
+                                                                  int width, float eps, int write_h) {
+    __shared__ float scratch[16];
+    const int r = blockIdx.x;
+    const size_t src = rows ? (size_t)rows[r] : (size_t)r;
+    float* hrow = h + src * width;
+    const elem_t* drow = delta ? delta + src * width : nullptr;
+    float sum = 0.f;
+    for (int c = threadIdx.x * MLR_VEC; c < width; c += 256 * MLR_VEC) {
+        float x[MLR_VEC];
+#pragma unroll
+        for (int e = 0; e < MLR_VEC; e += 4) {
+            const float4 v = *reinterpret_cast<const float4*>(hrow + c + e);
+            x[e] = v.x; x[e + 1] = v.y; x[e + 2] = v.z; x[e + 3] = v.w;
+        }
+        if (drow) {
+            float dv[MLR_VEC];
+            load_vec(drow + c, dv);
+#pragma unroll
+            for (int e = 0; e < MLR_VEC; ++e) x[e] += dv[e];
+            if (write_h) {
+#pragma unroll
+                for (int e = 0; e < MLR_VEC; e += 4)
+                    *reinterpret_cast<float4*>(hrow + c + e) = make_float4(x[e], x[e + 1], x[e + 2], x[e + 3]);
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < MLR_VEC; ++e) sum += x[e] * x[e];
+    }
+    sum = block_sum(sum, scratch);
+    const float scale = 1.0f / sqrtf(sum / (float)width + eps);
+    elem_t* orow = out + (size_t)r * width;
+    for (int c = threadIdx.x * MLR_VEC; c < width; c += 256 * MLR_VEC) {
+        float x[MLR_VEC], y[MLR_VEC];
+#pragma unroll
+        for (int e = 0; e < MLR_VEC; e += 4) {
+            const float4 v = *reinterpret_cast<const float4*>(hrow + c + e);
+            x[e] = v.x; x[e + 1] = v.y; x[e + 2] = v.z; x[e + 3] = v.w;
+        }
+        if (drow && !write_h) {
+            float dv[MLR_VEC];
+            load_vec(drow + c, dv);
+#pragma unroll
+            for (int e = 0; e < MLR_VEC; ++e) x[e] += dv[e];
+        }
+#pragma unroll
+        for (int e = 0; e < MLR_VEC; e += 4) {
+            const float4 w = *reinterpret_cast<const float4*>(weight + c + e);
+            y[e] = (x[e] * scale) * w.x;
+            y[e + 1] = (x[e + 1] * scale) * w.y;
+            y[e + 2] = (x[e + 2] * scale) * w.z;
+            y[e + 3] = (x[e + 3] * scale) * w.w;
+        }
+        store_vec(orow + c, y);
+    }
+}
+
 // The same for widths that are a multiple of 8 (bfloat16) or 4 (float), 16 bytes per lane and access:
 // one wavefront per row, four rows per workgroup, the row kept in registers between the two passes
 // when it fits (width <= 64 * MLR_VEC * ROW_REGS), else re-read.
@@ -167,6 +228,11 @@ int mlr_add_rmsnorm(float* h, const void* delta, const float* weight, void* out,
     if (MLR_BF16 && width % MLR_VEC == 0 && width <= 64 * MLR_VEC * ROW_REGS && n_out >= 64) {
         add_rmsnorm_vec_kernel<<<(n_out + 3) / 4, 256, 0, stream>>>(h, (const elem_t*)delta, weight, (elem_t*)out,
                                                                      rows, n_out, width, eps, write_h);
+        return (int)hipGetLastError();
+    }
+    if (MLR_BF16 && width % MLR_VEC == 0) {
+        add_rmsnorm_row_vec_kernel<<<n_out, 256, 0, stream>>>(h, (const elem_t*)delta, weight, (elem_t*)out, rows,
+                                                              width, eps, write_h);
         return (int)hipGetLastError();
     }
     add_rmsnorm_kernel<<<n_out, 256, 0, stream>>>(h, (const elem_t*)delta, weight, (elem_t*)out, rows,

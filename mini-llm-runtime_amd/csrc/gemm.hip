@@ -201,7 +201,7 @@ __global__ __launch_bounds__(SKINNY_WAVES * 64) void gemm_skinny_kernel(const __
         const __bf16* xrow[MT];
 #pragma unroll
         for (int i = 0; i < MT; ++i) xrow[i] = a + (size_t)min(16 * i + r16, M - 1) * K + b * 8;
-        constexpr int U = 8;
+        constexpr int U = (MT * NW <= 2) ? 16 : 8;      // weight loads in flight per lane
         for (int s0 = s_begin; s0 < s_end; s0 += U) {
             bf16x8 wf[NW][U];
 #pragma unroll
