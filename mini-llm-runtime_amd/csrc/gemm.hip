@@ -411,6 +411,8 @@ extern "C" int mlr_gemm(const void* a, const void* w, void* out, int M, int N, i
     if (M <= 0 || N <= 0) return 0;
     if (K <= 0) return -1;
     if (M <= 16) return launch_skinny<1, false>(a, w, out, M, N, K, out_float, stream);
+    // 17..64 rows against many columns (the output projection): tiles through LDS re-read the rows less often
+    if (M <= 64 && N >= 16384) return launch<2, 2, 2, 2>(a, w, out, M, N, K, out_float, stream);
     if (M <= 32) return launch_skinny<2, false>(a, w, out, M, N, K, out_float, stream);
     if (M <= 64) return launch_skinny<4, false>(a, w, out, M, N, K, out_float, stream);
     if (M <= 128) return launch<2, 2, 2, 2>(a, w, out, M, N, K, out_float, stream);  // 64 x 64

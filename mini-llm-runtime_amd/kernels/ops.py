@@ -21,7 +21,7 @@ _ptr = ctypes.c_void_p
 
 MAX_HEAD_DIM = 256          # the attention and rotation kernels keep head_dim / 64 values per lane
 ATTENTION_TILE_KEYS = 64
-LIBRARY_GEMM_MIN_ROWS = 64    # above this many rows the bfloat16 engine's projections go to the library
+LIBRARY_GEMM_MIN_ROWS = 16    # above this many rows the bfloat16 engine's projections go to the library
 PREFILL_MAX_PAGES = 2048      # page ids of one group that the prompt-portion attention kernel keeps in LDS
 MAX_KEY_SPLITS = 1024         # the merge of key splits keeps one weight per split in LDS
 
@@ -158,12 +158,14 @@ class Kernels:
                _c_int(1 if out.dtype == torch.float32 else 0), _stream()), "gemm")
 
     def gated_silu_fused(self, rows):
-        """Whether `gemm_gated_silu` serves this many rows (the bfloat16 engine, up to 64)."""
-        return self.dtype == torch.bfloat16 and rows <= 64
+        """Whether `gemm_gated_silu` is the path for this many rows: the bfloat16 engine, up to 16 rows with
+        the library in use (above that the library's product and a separate activation are faster), up to
+        64 without."""
+        return self.dtype == torch.bfloat16 and rows <= (LIBRARY_GEMM_MIN_ROWS if self.library_gemm else 64)
 
     def gemm_gated_silu(self, a, w, out):
         """out[M, N] = silu(a . w[:N]^T) * (a . w[N:]^T), w = [gate; up] stacked, for few rows."""
-        _need(self.gated_silu_fused(a.shape[0]), "gemm_gated_silu: bfloat16 and at most 64 rows")
+        _need(self.dtype == torch.bfloat16 and a.shape[0] <= 64, "gemm_gated_silu: bfloat16 and at most 64 rows")
         _tensor(a, "a", self.dtype, ndim=2)
         _tensor(w, "w", self.dtype, ndim=2)
         m, k = a.shape

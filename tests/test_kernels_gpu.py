@@ -498,9 +498,11 @@ def test_attention_window_edge(dtype, window):
 def test_gemm_gated_silu(mnk):
     """The feed-forward's activation fused into its first projection (few rows, bfloat16):
     silu(a Wgate^T) * (a Wup^T) with the sums kept in 32-bit until the product."""
+    from mini_llm_runtime_amd.kernels import Kernels
     m, n, kk = mnk
-    k = kernels(torch.bfloat16)
+    k = Kernels(torch.bfloat16, library_gemm=False)
     assert k.gated_silu_fused(m) and not k.gated_silu_fused(65)
+    assert kernels(torch.bfloat16).gated_silu_fused(16) and not kernels(torch.bfloat16).gated_silu_fused(17)
     a = rnd((m, kk), torch.bfloat16, 50)
     w = rnd((2 * n, kk), torch.bfloat16, 51, 0.3)
     out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
