@@ -44,6 +44,7 @@ def main():
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--context", type=int, default=4096)
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--page-size", type=int, default=16, help="tokens in a page of the cache")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points and the prefill")
     ap.add_argument("--only", default="all", choices=["all", "decode", "prefill"],
                     help="profiling aid: run just the decode steps or just the prefill")
@@ -92,7 +93,7 @@ def main():
     def decode_run(batch, steps, warmup):
         """Fill `batch` requests so that warmup + steps decode steps end at the context length; time `steps`."""
         runner = Runner(model, max_tokens=batch * (-(-args.context // 64) * 64), max_slots=batch,
-                        max_length=args.context, max_batch_tokens=max(PREFILL_TOKENS, batch), page_size=16)
+                        max_length=args.context, max_batch_tokens=max(PREFILL_TOKENS, batch), page_size=args.page_size)
         sampler = Sampler(runner.kernels, runner.device, max_rows=batch)
         fill = args.context - steps - warmup
         assert fill >= 1
@@ -129,7 +130,7 @@ def main():
 
     def prefill_run():
         runner = Runner(model, max_tokens=PREFILL_TOKENS, max_slots=1, max_length=PREFILL_TOKENS,
-                        max_batch_tokens=PREFILL_TOKENS, page_size=16)
+                        max_batch_tokens=PREFILL_TOKENS, page_size=args.page_size)
         ids = torch.randint(0, c.vocab_size, (PREFILL_TOKENS,), generator=g).tolist()
         times = []
         for i in range(4):
@@ -167,7 +168,7 @@ def main():
                    "kv_heads": c.num_key_value_heads, "head_dim": c.head_dim,
                    "intermediate_size": c.intermediate_size, "vocab_size": c.vocab_size,
                    "tied_embeddings": c.tie_word_embeddings, "rope_theta": c.rope_theta, "rms_norm_eps": c.rms_norm_eps,
-                   "global_batch": args.batch, "seq_len": args.context, "page_size": 16,
+                   "global_batch": args.batch, "seq_len": args.context, "page_size": args.page_size,
                    "sampling": "greedy", "parallelism": "single GPU"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                      "frac": round(achieved * 1e9 / HBM_PEAK, 5)},
