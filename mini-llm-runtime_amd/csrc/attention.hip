@@ -561,18 +561,16 @@ __global__ __launch_bounds__(256, (NCH <= 4 ? 2 : 1)) void attention_mfma_kernel
 // `attention_mfma_kernel` without key splits, tile by tile in ascending order.
 #define PAGE_CACHE 2048
 template <int NCH>
-__global__ __launch_bounds__(256, 2) void attention_prefill_kernel(AttnArgs a, const int32_t* __restrict__ group_row0,
-                                                                const int32_t* __restrict__ group_ntok) {
+__device__ __forceinline__ void prefill_group(const AttnArgs& a, const int32_t* __restrict__ group_row0,
+                                              const int32_t* __restrict__ group_ntok, int grp, int kvh,
+                                              __bf16 (*k_lds)[32 * (32 * NCH + 8)], __bf16 (*v_lds)[32 * NCH * 36],
+                                              int32_t* page_lds) {
     constexpr int DMAX = 32 * NCH;
     constexpr int KPITCH = DMAX + 8;                  // elements per key row in LDS
     constexpr int VPITCH = 32 + 4;                    // elements per channel row in LDS
     constexpr int STAGE = (NCH + 1) / 2;              // 16-byte chunks a thread stages per tile, for K and for V
-    __shared__ __attribute__((aligned(16))) __bf16 k_lds[2][32 * KPITCH];
-    __shared__ __attribute__((aligned(16))) __bf16 v_lds[2][DMAX * VPITCH];
-    __shared__ int32_t page_lds[PAGE_CACHE];          // the request's page ids for this group's key range
     const int D = a.head_dim, P = a.page_size;
     const int g = a.q_heads / a.kv_heads, tq = 16 / g;
-    const int grp = blockIdx.x, kvh = blockIdx.y;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int col = lane & 15, b = lane >> 4;
     const int row0 = group_row0[grp], ntok = group_ntok[grp];
@@ -799,6 +797,22 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(AttnArgs a, c
     }
 }
 
+// A workgroup takes two groups, one after the other: group i and group (groups - 1 - i).  Within a long
+// prompt the groups' key ranges grow with their position, so every workgroup gets about the same work.
+template <int NCH>
+__global__ __launch_bounds__(256, 2) void attention_prefill_kernel(AttnArgs a, const int32_t* __restrict__ group_row0,
+                                                                const int32_t* __restrict__ group_ntok, int groups) {
+    __shared__ __attribute__((aligned(16))) __bf16 k_lds[2][32 * (32 * NCH + 8)];
+    __shared__ __attribute__((aligned(16))) __bf16 v_lds[2][32 * NCH * 36];
+    __shared__ int32_t page_lds[PAGE_CACHE];          // the request's page ids for the group's key range
+    const int first = blockIdx.x, second = groups - 1 - first;
+    if (second > first) {
+        prefill_group<NCH>(a, group_row0, group_ntok, second, blockIdx.y, k_lds, v_lds, page_lds);
+        __syncthreads();
+    }
+    prefill_group<NCH>(a, group_row0, group_ntok, first, blockIdx.y, k_lds, v_lds, page_lds);
+}
+
 // The merge of key splits for the groups of `attention_mfma_kernel` (one wavefront per (group, head),
 // walking the group's tokens).
 __global__ __launch_bounds__(64) void attention_combine_groups_kernel(AttnArgs a, const int32_t* __restrict__ group_row0,
@@ -907,15 +921,15 @@ extern "C" int mlr_attention_prefill(
     AttnArgs a{(const elem_t*)q, (const elem_t*)k_pages, (const elem_t*)v_pages, block_table, slots,
                positions, (elem_t*)out, nullptr, max_blocks, q_heads, kv_heads, head_dim, page_size,
                window, 0, 1, scale};
-    dim3 grid(groups, kv_heads);
+    dim3 grid((groups + 1) / 2, kv_heads);
     const int nch = (head_dim + 31) / 32;
     switch (nch) {
-        case 1: attention_prefill_kernel<1><<<grid, 256, 0, stream>>>(a, group_row0, group_ntok); break;
-        case 2: attention_prefill_kernel<2><<<grid, 256, 0, stream>>>(a, group_row0, group_ntok); break;
-        case 3: attention_prefill_kernel<3><<<grid, 256, 0, stream>>>(a, group_row0, group_ntok); break;
-        case 4: attention_prefill_kernel<4><<<grid, 256, 0, stream>>>(a, group_row0, group_ntok); break;
-        case 5: attention_prefill_kernel<5><<<grid, 256, 0, stream>>>(a, group_row0, group_ntok); break;
-        default: attention_prefill_kernel<6><<<grid, 256, 0, stream>>>(a, group_row0, group_ntok); break;
+        case 1: attention_prefill_kernel<1><<<grid, 256, 0, stream>>>(a, group_row0, group_ntok, groups); break;
+        case 2: attention_prefill_kernel<2><<<grid, 256, 0, stream>>>(a, group_row0, group_ntok, groups); break;
+        case 3: attention_prefill_kernel<3><<<grid, 256, 0, stream>>>(a, group_row0, group_ntok, groups); break;
+        case 4: attention_prefill_kernel<4><<<grid, 256, 0, stream>>>(a, group_row0, group_ntok, groups); break;
+        case 5: attention_prefill_kernel<5><<<grid, 256, 0, stream>>>(a, group_row0, group_ntok, groups); break;
+        default: attention_prefill_kernel<6><<<grid, 256, 0, stream>>>(a, group_row0, group_ntok, groups); break;
     }
     return (int)hipGetLastError();
 }
