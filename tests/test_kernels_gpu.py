@@ -515,20 +515,21 @@ def test_gemm_gated_silu(mnk):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("shape", [(4, 2, 128, 16), (6, 3, 48, 32), (16, 8, 64, 16), (3, 1, 16, 16), (2, 2, 256, 64)])
-def test_qk_norm_rope_kv_many_rows(dtype, shape):
-    """A whole prompt portion (the many-row variants of the kernel): 90 consecutive positions of one request
-    beside 10 of another."""
+@pytest.mark.parametrize("layout", [([90, 10], [37, 0]), ([96, 16], [32, 8]), ([64, 3, 40], [0, 5, 16])])
+def test_qk_norm_rope_kv_many_rows(dtype, shape, layout):
+    """Whole prompt portions (the many-row variants of the kernels): consecutive positions of a few requests,
+    starting inside a page, at a page's edge and at multiples of eight."""
     hq, hkv, d, page = shape
     k = kernels(dtype)
-    counts = [90, 10]
-    starts = [37, 0]
+    counts, starts = layout
     m = sum(counts)
-    positions = torch.tensor([starts[s] + i for s in range(2) for i in range(counts[s])], dtype=torch.int32)
-    slots = torch.tensor([s for s in range(2) for _ in range(counts[s])], dtype=torch.int32)
+    n_req = len(counts)
+    positions = torch.tensor([starts[s] + i for s in range(n_req) for i in range(counts[s])], dtype=torch.int32)
+    slots = torch.tensor([s for s in range(n_req) for _ in range(counts[s])], dtype=torch.int32)
     max_blocks = 16
-    n_pages = 2 * max_blocks
+    n_pages = n_req * max_blocks
     perm = torch.randperm(n_pages, generator=torch.Generator().manual_seed(3)).to(torch.int32)
-    table = perm.view(2, max_blocks).contiguous()
+    table = perm.view(n_req, max_blocks).contiguous()
     qkv = rnd((m, (hq + 2 * hkv) * d), dtype, 60)
     qw, kw = rnd((d,), torch.float32, 61) + 1, rnd((d,), torch.float32, 62) + 1
     eps, base = 1e-6, 10000.0
