@@ -80,6 +80,7 @@ def _host_lib():
         intp = ctypes.POINTER(ctypes.c_int)
         lib.mlr_cache_prepare.argtypes = [ctypes.c_void_p, i32p, i32p, ctypes.c_int, intp, intp]
         lib.mlr_cache_commit.argtypes = [ctypes.c_void_p, i32p, i32p, ctypes.c_int]
+        lib.mlr_cache_commit_first.argtypes = [ctypes.c_void_p, i32p, i32p, ctypes.c_int, i32p]
         lib.mlr_cache_retire.argtypes = [ctypes.c_void_p, i32p, ctypes.c_int]
         lib.mlr_cache_take_dirty.argtypes = [ctypes.c_void_p, ctypes.c_int, i32p]
         lib.mlr_cache_check.argtypes = [ctypes.c_void_p]
@@ -177,6 +178,18 @@ class PageBook:
         if rc != 0:
             self._raise(rc, -1, (0, 0))
 
+    def commit_first(self, slots, counts):
+        """`commit`, returning each entry's first position (the slot's length before the batch).  Raises
+        like `prepare`, with nothing changed."""
+        s, sp = _i32(slots)
+        c, cp = _i32(counts)
+        first = np.empty(len(s), dtype=np.int32)
+        rc = self._lib.mlr_cache_commit_first(self._h, sp, cp, len(s), first.ctypes.data_as(ctypes.POINTER(ctypes.c_int32)))
+        if rc != 0:
+            self.prepare(slots, counts)           # raises the precise error
+            self._raise(rc, -1, (0, 0))
+        return first.tolist()
+
     def retire(self, slots):
         s, sp = _i32(slots)
         rc = self._lib.mlr_cache_retire(self._h, sp, len(s))
@@ -267,6 +280,11 @@ class CacheManager:
     def commit(self, slots, counts):
         self.book.commit(slots, counts)
         self.sync_tables()
+
+    def commit_first(self, slots, counts):
+        first = self.book.commit_first(slots, counts)
+        self.sync_tables()
+        return first
 
     def retire(self, slots):
         """After a step: give back what windows have passed.  The device tables are brought up

@@ -193,33 +193,46 @@ __global__ __launch_bounds__(SKINNY_WAVES * 64) void gemm_skinny_kernel(const __
     for (int g = 0; g < NW; ++g)
 #pragma unroll
         for (int i = 0; i < MT; ++i) acc[g][i] = floatx4{0.f, 0.f, 0.f, 0.f};
-    if ((K & 31) == 0) {
-        // The usual case, K a multiple of 32: no branch anywhere near a load (a load behind a branch makes
+    if ((K & 63) == 0) {
+        // The usual case, K a multiple of 64: no branch anywhere near a load (a load behind a branch makes
         // the compiler wait for every load in flight).  Rows beyond N or M read the last valid row; what
-        // they produce is never stored.  Eight steps' worth of weight loads are issued before they are used.
-        const __bf16* wrow = w + (size_t)min(n0 + r16, N - 1) * K + b * 8;
+        // they produce is never stored.  Two k steps are taken together: a lane reads 32 consecutive bytes
+        // of its weight row (four lanes a whole 128-byte line), each 16 of them feed one product; the
+        // activation is read the same way, so the k slots of both operands agree.  (Measured: 64 bytes a
+        // lane is slower again.)
+        constexpr int W = 2;                              // 16-byte chunks per lane and group
+        const int groups = steps / W;
+        const int per_wave_g = (groups + SKINNY_WAVES - 1) / SKINNY_WAVES;
+        const int g_begin = wave * per_wave_g, g_end = min(groups, g_begin + per_wave_g);
+        const __bf16* wrow = w + (size_t)min(n0 + r16, N - 1) * K + b * (8 * W);
         const __bf16* xrow[MT];
 #pragma unroll
-        for (int i = 0; i < MT; ++i) xrow[i] = a + (size_t)min(16 * i + r16, M - 1) * K + b * 8;
-        constexpr int U = (MT * NW <= 2) ? 16 : 8;      // weight loads in flight per lane
-        for (int s0 = s_begin; s0 < s_end; s0 += U) {
-            bf16x8 wf[NW][U];
+        for (int i = 0; i < MT; ++i) xrow[i] = a + (size_t)min(16 * i + r16, M - 1) * K + b * (8 * W);
+        constexpr int U = (MT * NW <= 2) ? 8 : 4;         // groups whose weight loads are in flight per lane
+        for (int g0 = g_begin; g0 < g_end; g0 += U) {
+            bf16x8 wf[NW][U][W];
 #pragma unroll
             for (int u = 0; u < U; ++u) {
-                const int k = min(s0 + u, s_end - 1) * 32;
+                const int k = min(g0 + u, g_end - 1) * (32 * W);
 #pragma unroll
-                for (int g = 0; g < NW; ++g) wf[g][u] = *reinterpret_cast<const bf16x8*>(wrow + (size_t)g * N * K + k);
+                for (int g = 0; g < NW; ++g)
+#pragma unroll
+                    for (int c = 0; c < W; ++c)
+                        wf[g][u][c] = *reinterpret_cast<const bf16x8*>(wrow + (size_t)g * N * K + k + 8 * c);
             }
 #pragma unroll
             for (int u = 0; u < U; ++u) {
-                if (s0 + u >= s_end) break;
-                const int k = (s0 + u) * 32;
+                if (g0 + u >= g_end) break;
+                const int k = (g0 + u) * (32 * W);
 #pragma unroll
                 for (int i = 0; i < MT; ++i) {
-                    const bf16x8 xf = *reinterpret_cast<const bf16x8*>(xrow[i] + k);
 #pragma unroll
-                    for (int g = 0; g < NW; ++g)
-                        acc[g][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[g][u], xf, acc[g][i], 0, 0, 0);
+                    for (int c = 0; c < W; ++c) {
+                        const bf16x8 xf = *reinterpret_cast<const bf16x8*>(xrow[i] + k + 8 * c);
+#pragma unroll
+                        for (int g = 0; g < NW; ++g)
+                            acc[g][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[g][u][c], xf, acc[g][i], 0, 0, 0);
+                    }
                 }
             }
         }

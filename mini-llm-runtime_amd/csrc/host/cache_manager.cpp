@@ -180,6 +180,16 @@ int mlr_cache_commit(void* h, const int32_t* slots, const int32_t* counts, int n
     return 0;
 }
 
+// `commit` that also reports where each entry's tokens start (the slot's length before the batch).
+int mlr_cache_commit_first(void* h, const int32_t* slots, const int32_t* counts, int n, int32_t* first) {
+    auto* c = static_cast<Cache*>(h);
+    for (int i = 0; i < n; ++i) {
+        const int s = slots[i];
+        first[i] = (s >= 0 && s < c->max_slots && c->live[s]) ? c->length[s] : -1;
+    }
+    return mlr_cache_commit(h, slots, counts, n);
+}
+
 // After the step ran: in groups with a window, pages whose keys no later query can see go
 // back to the pool.  A query at position >= length sees keys > position - window.
 int mlr_cache_retire(void* h, const int32_t* slots, int n) {

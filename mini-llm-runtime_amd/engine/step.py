@@ -133,9 +133,7 @@ class Runner:
         total = self._validate(entries)
         slots = [e.slot for e in entries]
         counts = [len(e.tokens) for e in entries]
-        self.cache.prepare(slots, counts)                 # raises, nothing changed
-        first = [self.cache.length(s) for s in slots]
-        self.cache.commit(slots, counts)
+        first = self.cache.commit_first(slots, counts)    # raises with nothing changed, else takes the pages
         try:
             if (self.use_graphs and total == len(entries) <= self.graph_max_batch
                     and all(list(e.want) == [0] for e in entries)):

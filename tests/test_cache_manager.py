@@ -198,3 +198,17 @@ def test_random_orders_of_requests(seed, window):
                 else:
                     assert p == -1
         assert len(seen) + b.free_pages() == pages
+
+
+def test_commit_reports_first_positions():
+    b = book(pages=8, page=16, slots=3)
+    s0, s1 = b.acquire_slot(), b.acquire_slot()
+    assert b.commit_first([s0, s1], [5, 20]) == [0, 0]
+    assert b.commit_first([s1, s0], [1, 3]) == [20, 5]
+    before = (b.table().copy(), b.free_pages(), b.length(s0), b.length(s1))
+    with pytest.raises(CacheFull):
+        b.commit_first([s0, s1], [60, 60])
+    with pytest.raises(CacheError):
+        b.commit_first([s0, 2], [1, 1])
+    assert (b.table() == before[0]).all() and (b.free_pages(), b.length(s0), b.length(s1)) == before[1:]
+    b.check()
