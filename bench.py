@@ -45,6 +45,8 @@ def main():
     ap.add_argument("--context", type=int, default=4096)
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--page-size", type=int, default=16, help="tokens in a page of the cache")
+    ap.add_argument("--attn-workgroups", type=int, default=512,
+                    help="tuning aid: workgroups that the split of a token's keys aims for")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points and the prefill")
     ap.add_argument("--only", default="all", choices=["all", "decode", "prefill"],
                     help="profiling aid: run just the decode steps or just the prefill")
@@ -93,7 +95,8 @@ def main():
     def decode_run(batch, steps, warmup):
         """Fill `batch` requests so that warmup + steps decode steps end at the context length; time `steps`."""
         runner = Runner(model, max_tokens=batch * (-(-args.context // 64) * 64), max_slots=batch,
-                        max_length=args.context, max_batch_tokens=max(PREFILL_TOKENS, batch), page_size=args.page_size)
+                        max_length=args.context, max_batch_tokens=max(PREFILL_TOKENS, batch), page_size=args.page_size,
+                        target_workgroups=args.attn_workgroups)
         sampler = Sampler(runner.kernels, runner.device, max_rows=batch)
         fill = args.context - steps - warmup
         assert fill >= 1

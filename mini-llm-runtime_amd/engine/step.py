@@ -30,7 +30,8 @@ class Entry:
 
 class Runner:
     def __init__(self, model, max_tokens, max_slots=4, max_length=None, max_batch_tokens=None,
-                 page_size=16, split_keys=256, split_max_tokens=256, use_graphs=True, graph_max_batch=256):
+                 page_size=16, split_keys=256, split_max_tokens=256, use_graphs=True, graph_max_batch=256,
+                 target_workgroups=512):
         self.model = model
         self.dtype, self.device = model.dtype, model.device
         spec = model.spec
@@ -43,6 +44,7 @@ class Runner:
         self.workspace = Workspace(self.device)
         self.ctx = StepContext(self.kernels, self.cache, self.workspace, self.dtype, self.max_length,
                                split_keys, split_max_tokens)
+        self.ctx.target_workgroups = target_workgroups
         self._upload = Uploader(4 * self.max_batch_tokens, self.device)
         self._meta = torch.empty(4 * self.max_batch_tokens, dtype=torch.int32, device=self.device)
         self.poisoned = False
