@@ -77,6 +77,8 @@ class StepContext:
         self.max_positions = max_positions
         self.split_keys, self.split_max_tokens = split_keys, split_max_tokens
         self.target_workgroups = 512      # about two workgroups per compute unit
+        self.compute_units = (torch.cuda.get_device_properties(torch.cuda.current_device()).multi_processor_count
+                              if torch.cuda.is_available() else 1)
         self.n_tokens = 0
         self.token_ids = self.positions = self.slots = None
         self.segments = []            # (slot, first row, number of tokens, first position)

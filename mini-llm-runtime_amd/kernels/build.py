@@ -32,6 +32,7 @@ HIP_LIBRARIES = {
     "rope_kv": (["rope_kv.hip"], ["common.h"], True),
     "attention": (["attention.hip"], ["common.h"], True),
     "gemm": (["gemm.hip"], ["common.h"], True),
+    "attention_tiles": (["attention_tiles.hip"], [], False),      # bfloat16 only by nature
     "sampling": (["sampling.hip"], [], False),
 }
 HOST_LIBRARIES = {

@@ -23,6 +23,8 @@ MAX_HEAD_DIM = 256          # the attention and rotation kernels keep head_dim /
 ATTENTION_TILE_KEYS = 64
 LIBRARY_GEMM_MIN_ROWS = 16    # above this many rows the bfloat16 engine's projections go to the library
 PREFILL_MAX_PAGES = 2048      # page ids of one group that the prompt-portion attention kernel keeps in LDS
+TILES_MAX_HEAD_DIM = 128      # the 32x32-tile kernel for prompt portions keeps two sets of accumulators per lane
+TILES_COLUMNS = (128, 64)     # (token, head) columns of one of its workgroups: the usual and the small one
 MAX_KEY_SPLITS = 1024         # the merge of key splits keeps one weight per split in LDS
 
 
@@ -34,25 +36,36 @@ def _p(t):
     return _ptr(t.data_ptr()) if t is not None else _ptr(0)
 
 
+try:
+    _raw_stream = torch._C._cuda_getCurrentRawStream          # the current stream's handle without a Stream object
+except AttributeError:                                         # pragma: no cover
+    _raw_stream = None
+
+
 def _stream():
+    """Handle of torch's current stream on the current device."""
+    if _raw_stream is not None:
+        return _ptr(_raw_stream(torch.cuda.current_device()))
     return _ptr(torch.cuda.current_stream().cuda_stream)
 
 
 def _need(cond, message):
+    """`message` is a string or, where building it costs time, a function that returns one."""
     if not cond:
-        raise KernelError(message)
+        raise KernelError(message() if callable(message) else message)
 
 
 def _tensor(t, name, dtype, shape=None, ndim=None):
+    # one cheap test on the way that every launch takes; the message is only put together on failure
+    if (isinstance(t, torch.Tensor) and t.is_cuda and t.dtype == dtype and t.is_contiguous()
+            and (ndim is None or t.dim() == ndim) and (shape is None or t.shape == tuple(shape))):
+        return t
     _need(isinstance(t, torch.Tensor), f"{name}: expected a tensor")
     _need(t.is_cuda, f"{name}: must lie on the GPU (there is no CPU path)")
     _need(t.dtype == dtype, f"{name}: expected {dtype}, got {t.dtype}")
     _need(t.is_contiguous(), f"{name}: must be contiguous")
-    if ndim is not None:
-        _need(t.dim() == ndim, f"{name}: expected {ndim} dimensions, got {tuple(t.shape)}")
-    if shape is not None:
-        _need(tuple(t.shape) == tuple(shape), f"{name}: expected shape {tuple(shape)}, got {tuple(t.shape)}")
-    return t
+    _need(ndim is None or t.dim() == ndim, f"{name}: expected {ndim} dimensions, got {tuple(t.shape)}")
+    raise KernelError(f"{name}: expected shape {tuple(shape)}, got {tuple(t.shape)}")
 
 
 def _ok(code, what):
@@ -145,8 +158,8 @@ class Kernels:
         _tensor(w, "w", self.dtype, ndim=2)
         m, k = a.shape
         n, k2 = w.shape
-        _need(k == k2, f"gemm: inner sizes differ ({k} and {k2})")
-        _need(out.dtype in (self.dtype, torch.float32), f"gemm: output type {out.dtype} not supported")
+        _need(k == k2, lambda: f"gemm: inner sizes differ ({k} and {k2})")
+        _need(out.dtype in (self.dtype, torch.float32), lambda: f"gemm: output type {out.dtype} not supported")
         _tensor(out, "out", out.dtype, (m, n))
         if self.library_gemm and self.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and m > LIBRARY_GEMM_MIN_ROWS:
             # many rows: a plain matrix product, handed to the vendor library (hipBLASLt through torch),
@@ -202,8 +215,8 @@ class Kernels:
     # -- attention ---------------------------------------------------------------------------
     def _check_cache(self, k_pages, v_pages, kv_heads, head_dim, page_size):
         _tensor(k_pages, "k_pages", self.dtype, ndim=4)
-        _need(tuple(k_pages.shape[1:]) == (kv_heads, page_size, head_dim),
-              f"k_pages: expected [pages, {kv_heads}, {page_size}, {head_dim}], got {tuple(k_pages.shape)}")
+        _need(k_pages.shape[1:] == (kv_heads, page_size, head_dim),
+              lambda: f"k_pages: expected [pages, {kv_heads}, {page_size}, {head_dim}], got {tuple(k_pages.shape)}")
         _tensor(v_pages, "v_pages", self.dtype, (k_pages.shape[0], kv_heads, head_dim, page_size))
 
     def qk_norm_rope_kv(self, qkv, q_out, k_pages, v_pages, block_table, slots, positions, q_norm_w,
@@ -211,11 +224,11 @@ class Kernels:
         """Per head: RMSNorm of q and k (weights may be None), rotation by `rope`
         [max_positions, head_dim] (may be None), q into q_out, k and v into their pages."""
         _need(head_dim % 2 == 0 and 2 <= head_dim <= MAX_HEAD_DIM,
-              f"head_dim {head_dim}: the rotation kernel takes even sizes up to {MAX_HEAD_DIM}")
+              lambda: f"head_dim {head_dim}: the rotation kernel takes even sizes up to {MAX_HEAD_DIM}")
         width = (q_heads + 2 * kv_heads) * head_dim
         _tensor(qkv, "qkv", self.dtype, ndim=2)
         m = qkv.shape[0]
-        _need(qkv.shape[1] == width, f"qkv: expected width {width}, got {qkv.shape[1]}")
+        _need(qkv.shape[1] == width, lambda: f"qkv: expected width {width}, got {qkv.shape[1]}")
         _tensor(q_out, "q_out", self.dtype, (m, q_heads * head_dim))
         self._check_cache(k_pages, v_pages, kv_heads, head_dim, page_size)
         _tensor(block_table, "block_table", torch.int32, ndim=2)
@@ -241,7 +254,8 @@ class Kernels:
                         partial=None):
         """out[m, h] = softmax over the keys seen by token m (positions <= its own, within the
         window) of q.k * scale, times v; keys and values from the pages of slots[m]."""
-        _need(1 <= head_dim <= MAX_HEAD_DIM, f"head_dim {head_dim}: the attention kernel takes up to {MAX_HEAD_DIM}")
+        _need(1 <= head_dim <= MAX_HEAD_DIM,
+              lambda: f"head_dim {head_dim}: the attention kernel takes up to {MAX_HEAD_DIM}")
         _need(q_heads % kv_heads == 0, "q_heads must be a multiple of kv_heads")
         _tensor(q, "q", self.dtype, ndim=2)
         m = q.shape[0]
@@ -254,7 +268,7 @@ class Kernels:
         _need(kv_heads <= 65535, "too many kv heads for the grid")
         if max_splits > 1:
             _need(split_keys > 0 and split_keys % ATTENTION_TILE_KEYS == 0,
-                  f"split_keys must be a multiple of {ATTENTION_TILE_KEYS}")
+                  lambda: f"split_keys must be a multiple of {ATTENTION_TILE_KEYS}")
             _need(partial is not None, "partial buffer needed for split attention")
             _tensor(partial, "partial", torch.float32, ndim=1)
             _need(partial.numel() >= self.attention_partial_numel(m, q_heads, head_dim, max_splits),
@@ -296,7 +310,7 @@ class Kernels:
         _need(kv_heads <= 65535 and max_splits <= MAX_KEY_SPLITS, "too many kv heads or key splits for the grid")
         if max_splits > 1:
             _need(split_keys > 0 and split_keys % ATTENTION_TILE_KEYS == 0,
-                  f"split_keys must be a multiple of {ATTENTION_TILE_KEYS}")
+                  lambda: f"split_keys must be a multiple of {ATTENTION_TILE_KEYS}")
             _need(partial is not None, "partial buffer needed for split attention")
             _tensor(partial, "partial", torch.float32, ndim=1)
             _need(partial.numel() >= self.attention_partial_numel(m, q_heads, head_dim, max_splits),
@@ -340,6 +354,50 @@ class Kernels:
                _p(positions), _p(out), _p(group_row0), _p(group_ntok), _c_int(groups), _c_int(q_heads),
                _c_int(kv_heads), _c_int(head_dim), _c_int(page_size), _c_int(window or 0), _c_float(scale),
                _stream()), "attention_prefill")
+
+    def tiles_attention_supported(self, q_heads, kv_heads, head_dim, page_size, max_context=0, num_pages=0):
+        """The 32x32-tile kernel for prompt portions: bfloat16, head sizes up to 128 in steps of 16, pages
+        of a power of two of keys, at most 16 query heads per kv head, contexts of at most 2048 pages (it
+        keeps a group's page ids in LDS), a cache of fewer than 2^32 elements per layer (32-bit offsets)."""
+        stride = kv_heads * page_size * head_dim
+        return (self.mfma_attention_supported(q_heads, kv_heads, head_dim, page_size) and head_dim <= TILES_MAX_HEAD_DIM
+                and page_size & (page_size - 1) == 0 and max_context <= PREFILL_MAX_PAGES * page_size
+                and stride < 2 ** 24 and num_pages < 2 ** 24 and stride * num_pages < 2 ** 32)
+
+    @staticmethod
+    def tiles_group_tokens(q_heads, kv_heads, columns=TILES_COLUMNS[0]):
+        """The most tokens of a group of `attention_tiles` with workgroups of `columns` columns."""
+        return columns // (q_heads // kv_heads)
+
+    def attention_tiles(self, q, k_pages, v_pages, block_table, slots, positions, out, group_row0, group_ntok,
+                        groups, q_heads, kv_heads, head_dim, page_size, scale, window=None, max_context=None,
+                        columns=TILES_COLUMNS[0]):
+        """Attention for prompt portions: groups of up to columns // (q_heads // kv_heads) consecutive rows
+        of one request each (columns = 128, or 64 for batches that would not fill the GPU with the larger
+        workgroups); keys and values of a group are staged once through LDS in blocks of 64.  The caller
+        vouches for the groups (consecutive rows of one request, no more tokens than `tiles_group_tokens`)."""
+        _need(columns in TILES_COLUMNS, lambda: f"attention_tiles: columns must be one of {TILES_COLUMNS}")
+        _need(self.tiles_attention_supported(q_heads, kv_heads, head_dim, page_size, num_pages=k_pages.shape[0]),
+              "attention_tiles: sizes not supported")
+        _need(block_table.shape[1] <= PREFILL_MAX_PAGES or max_context is not None,
+              "attention_tiles: give max_context when the block table is wider than the kernel's page cache")
+        _need((max_context or 0) <= PREFILL_MAX_PAGES * page_size, "attention_tiles: context too long")
+        _tensor(q, "q", self.dtype, ndim=2)
+        m = q.shape[0]
+        _need(q.shape[1] == q_heads * head_dim, "q: wrong width")
+        _tensor(out, "out", self.dtype, (m, q_heads * head_dim))
+        self._check_cache(k_pages, v_pages, kv_heads, head_dim, page_size)
+        _tensor(block_table, "block_table", torch.int32, ndim=2)
+        _tensor(slots, "slots", torch.int32, (m,))
+        _tensor(positions, "positions", torch.int32, (m,))
+        _tensor(group_row0, "group_row0", torch.int32, (groups,))
+        _tensor(group_ntok, "group_ntok", torch.int32, (groups,))
+        _need(kv_heads <= 65535, "too many kv heads for the grid")
+        fn = self._lib("attention_tiles").mlr_attention_tiles
+        _ok(fn(_p(q), _p(k_pages), _p(v_pages), _p(block_table), _c_int(block_table.shape[1]), _p(slots),
+               _p(positions), _p(out), _p(group_row0), _p(group_ntok), _c_int(groups), _c_int(columns),
+               _c_int(q_heads), _c_int(kv_heads), _c_int(head_dim), _c_int(page_size), _c_int(k_pages.shape[0]),
+               _c_int(window or 0), _c_float(scale), _stream()), "attention_tiles")
 
     # -- sampling ----------------------------------------------------------------------------
     def sample_scratch(self, rows):

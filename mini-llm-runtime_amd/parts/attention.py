@@ -59,7 +59,8 @@ class GqaAttention:
         return KvSpec(self.spec.kv_heads, self.spec.head_dim, self.spec.window)
 
     def libraries(self):
-        return ["gemm", "rope_kv", "attention"]
+        tiles = ["attention_tiles"] if self.qkv is not None and self.qkv.dtype == torch.bfloat16 else []
+        return ["gemm", "rope_kv", "attention"] + tiles
 
     def forward_prenorm(self, ctx, h, delta, norm, h_out, cache_id, write_cache=True):
         """As `forward` on norm(h + delta), the residual add and the norm done inside the first
@@ -93,12 +94,23 @@ class GqaAttention:
             s.q_heads, s.kv_heads, s.head_dim, view.page_size, write_cache)
         attn = ctx.workspace.get("attn", (m, s.q_heads * s.head_dim), x.dtype)
         if k.mfma_attention_supported(s.q_heads, s.kv_heads, s.head_dim, view.page_size):
-            # prompt portions go to the LDS-staged kernel, single tokens and short portions to the one
-            # that can split a token's keys over workgroups
-            big_factor = 4 if k.prefill_attention_supported(s.q_heads, s.kv_heads, s.head_dim, view.page_size,
-                                                            ctx.max_context) else 0
-            small, big, small_rows = ctx.token_groups(max(1, 16 // (s.q_heads // s.kv_heads)), big_factor)
-            if big[2]:
+            # prompt portions go to one of the LDS-staged kernels (the 32x32-tile one where it takes the
+            # sizes), single tokens and short portions to the one that can split a token's keys over
+            # workgroups
+            sizes = (s.q_heads, s.kv_heads, s.head_dim, view.page_size, ctx.max_context)
+            g = s.q_heads // s.kv_heads
+            tq = max(1, 16 // g)
+            tiles = k.tiles_attention_supported(*sizes, num_pages=view.k_pages.shape[0])
+            # workgroups of 128 columns where the step brings enough of them for every compute unit (they
+            # are launched in pairs), else of 64
+            columns = 128 if m * g * s.kv_heads >= 2 * 128 * ctx.compute_units else 64
+            big_factor = (columns // 16 if tiles else 4) if tiles or k.prefill_attention_supported(*sizes) else 0
+            small, big, small_rows = ctx.token_groups(tq, big_factor)
+            if big[2] and tiles:
+                k.attention_tiles(q, view.k_pages, view.v_pages, view.block_table, ctx.slots, ctx.positions, attn,
+                                  big[0], big[1], big[2], s.q_heads, s.kv_heads, s.head_dim, view.page_size,
+                                  float(s.scale), window=s.window, max_context=ctx.max_context, columns=columns)
+            elif big[2]:
                 k.attention_prefill(q, view.k_pages, view.v_pages, view.block_table, ctx.slots, ctx.positions, attn,
                                     big[0], big[1], big[2], s.q_heads, s.kv_heads, s.head_dim, view.page_size,
                                     float(s.scale), window=s.window, max_context=ctx.max_context)

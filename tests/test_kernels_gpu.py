@@ -341,6 +341,22 @@ def test_paged_attention(dtype, case):
     for i in range(lengths[0]):
         torch.testing.assert_close(got[i], wants[i], **tol(dtype))
     assert torch.isnan(out3[lengths[0]:].float()).all()
+    if not k.tiles_attention_supported(hq, hkv, d, page):
+        return
+    # the 32x32-tile kernel for prompt portions, with both sizes of workgroup: groups of as many tokens as a
+    # workgroup takes, and of fewer
+    for columns, big in ((128, k.tiles_group_tokens(hq, hkv, 128)), (128, 8 * tq), (64, k.tiles_group_tokens(hq, hkv, 64)),
+                         (64, 3 * tq)):
+        first = list(range(0, lengths[0], big))
+        count = [min(big, lengths[0] - r) for r in first]
+        out4 = torch.full((m, hq * d), float("nan"), dtype=dtype, device="cuda")
+        k.attention_tiles(q.view(m, hq * d).cuda(), k_pages.cuda(), v_pages.cuda(), table.cuda(), slots, pos, out4,
+                          torch.tensor(first, dtype=torch.int32).cuda(), torch.tensor(count, dtype=torch.int32).cuda(),
+                          len(first), hq, hkv, d, page, scale, window=window, columns=columns)
+        got = out4.double().cpu().view(m, hq, d)
+        for i in range(lengths[0]):
+            torch.testing.assert_close(got[i], wants[i], **tol(dtype))
+        assert torch.isnan(out4[lengths[0]:].float()).all()
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
