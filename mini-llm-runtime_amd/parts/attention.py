@@ -101,9 +101,9 @@ class GqaAttention:
             g = s.q_heads // s.kv_heads
             tq = max(1, 16 // g)
             tiles = k.tiles_attention_supported(*sizes, num_pages=view.k_pages.shape[0])
-            # workgroups of 128 columns where the step brings enough of them for every compute unit (they
-            # are launched in pairs), else of 64
-            columns = 128 if m * g * s.kv_heads >= 2 * 128 * ctx.compute_units else 64
+            # workgroups of 128 columns (launched in pairs) unless they would leave half of the compute
+            # units idle: then of 64
+            columns = 128 if m * s.q_heads > 128 * ctx.compute_units else 64
             big_factor = (columns // 16 if tiles else 4) if tiles or k.prefill_attention_supported(*sizes) else 0
             small, big, small_rows = ctx.token_groups(tq, big_factor)
             if big[2] and tiles:
