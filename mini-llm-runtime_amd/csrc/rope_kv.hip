@@ -102,6 +102,10 @@ __global__ void qk_norm_rope_kv_kernel(
 // half (16-byte accesses); a wavefront serves 64 / (head_dim / 16) heads at once.
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 
+// Every load is asked for as early as its address is known and none sits behind a branch, so a thread
+// waits for memory twice (the row's position and its own channels; then the page id and the rotation row)
+// instead of once per table.
+template <bool HAS_NORM, bool HAS_ROPE>
 __global__ __launch_bounds__(256) void qk_norm_rope_kv_vec_kernel(
     const __bf16* __restrict__ qkv, int ld, __bf16* __restrict__ q_out, __bf16* __restrict__ k_pages,
     __bf16* __restrict__ v_pages, const int32_t* __restrict__ block_table, int max_blocks,
@@ -112,13 +116,36 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kv_vec_kernel(
     const int lph = head_dim / 16;                         // lanes per head (a power of two)
     const int half = head_dim >> 1;
     const int total = q_heads + (skip_values ? 1 : 2) * kv_heads;
-    const int head = (blockIdx.y * blockDim.x + threadIdx.x) / lph;
+    const int head_raw = (blockIdx.y * blockDim.x + threadIdx.x) / lph;
+    const bool active = head_raw < total;
+    const int head = active ? head_raw : 0;
     const int c = threadIdx.x % lph;                       // this lane: channels 8c .. 8c + 7 and half + 8c ..
     const int pos = positions[m], slot = slots[m];
-    const bool active = head < total;
-    const __bf16* src = qkv + (size_t)m * ld + (size_t)(active ? head : 0) * head_dim;
+    const __bf16* src = qkv + (size_t)m * ld + (size_t)head * head_dim;
     const bf16x8 lo8 = *reinterpret_cast<const bf16x8*>(src + 8 * c);
     const bf16x8 hi8 = *reinterpret_cast<const bf16x8*>(src + half + 8 * c);
+    const bool is_q = head < q_heads;
+    float wl[8], wh[8];
+    if (HAS_NORM) {
+        const float* w = is_q ? q_norm_w : k_norm_w;
+        const float4 w0 = *reinterpret_cast<const float4*>(w + 8 * c), w1 = *reinterpret_cast<const float4*>(w + 8 * c + 4);
+        const float4 w2 = *reinterpret_cast<const float4*>(w + half + 8 * c);
+        const float4 w3 = *reinterpret_cast<const float4*>(w + half + 8 * c + 4);
+        wl[0] = w0.x; wl[1] = w0.y; wl[2] = w0.z; wl[3] = w0.w; wl[4] = w1.x; wl[5] = w1.y; wl[6] = w1.z; wl[7] = w1.w;
+        wh[0] = w2.x; wh[1] = w2.y; wh[2] = w2.z; wh[3] = w2.w; wh[4] = w3.x; wh[5] = w3.y; wh[6] = w3.z; wh[7] = w3.w;
+    }
+    // what needs the position: the page (entry 0 of the request's row when nothing is written) and the
+    // rotation row
+    const int page = block_table[(size_t)slot * max_blocks + (write_cache ? pos / page_size : 0)];
+    float co[8], si[8];
+    if (HAS_ROPE) {
+        const float* cs = rope + (size_t)pos * head_dim;
+        const float4 c0 = *reinterpret_cast<const float4*>(cs + 8 * c), c1 = *reinterpret_cast<const float4*>(cs + 8 * c + 4);
+        const float4 s0 = *reinterpret_cast<const float4*>(cs + half + 8 * c);
+        const float4 s1 = *reinterpret_cast<const float4*>(cs + half + 8 * c + 4);
+        co[0] = c0.x; co[1] = c0.y; co[2] = c0.z; co[3] = c0.w; co[4] = c1.x; co[5] = c1.y; co[6] = c1.z; co[7] = c1.w;
+        si[0] = s0.x; si[1] = s0.y; si[2] = s0.z; si[3] = s0.w; si[4] = s1.x; si[5] = s1.y; si[6] = s1.z; si[7] = s1.w;
+    }
     float a[8], b[8];
     float sum = 0.f;
 #pragma unroll
@@ -129,15 +156,9 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kv_vec_kernel(
     }
     for (int off = 1; off < lph; off <<= 1) sum += __shfl_xor(sum, off, MLR_WAVE);
     if (!active) return;
-    size_t cache_page = 0;
-    int in_page = 0;
-    bool cache_ok = false;
-    if (write_cache) {
-        const int page = block_table[(size_t)slot * max_blocks + pos / page_size];
-        cache_ok = page >= 0;
-        cache_page = (size_t)(page < 0 ? 0 : page) * kv_heads;
-        in_page = pos % page_size;
-    }
+    const bool cache_ok = write_cache && page >= 0;
+    const size_t cache_page = (size_t)(page < 0 ? 0 : page) * kv_heads;
+    const int in_page = pos % page_size;
     if (head >= q_heads + kv_heads) {                      // a value head: into its transposed page
         if (!cache_ok) return;
         __bf16* dst = v_pages + (cache_page + (head - q_heads - kv_heads)) * head_dim * page_size + in_page;
@@ -148,23 +169,19 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kv_vec_kernel(
         }
         return;
     }
-    const bool is_q = head < q_heads;
-    const float* w = is_q ? q_norm_w : k_norm_w;
-    if (w) {
+    if (HAS_NORM) {
         const float scale = 1.0f / sqrtf(sum / (float)head_dim + eps);
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-            a[e] = (a[e] * scale) * w[8 * c + e];
-            b[e] = (b[e] * scale) * w[half + 8 * c + e];
+            a[e] = (a[e] * scale) * wl[e];
+            b[e] = (b[e] * scale) * wh[e];
         }
     }
-    if (rope) {
-        const float* cs = rope + (size_t)pos * head_dim;
+    if (HAS_ROPE) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-            const float co = cs[8 * c + e], si = cs[half + 8 * c + e];
-            const float x = a[e] * co - b[e] * si;
-            const float y = a[e] * si + b[e] * co;
+            const float x = a[e] * co[e] - b[e] * si[e];
+            const float y = a[e] * si[e] + b[e] * co[e];
             a[e] = x;
             b[e] = y;
         }
@@ -260,10 +277,18 @@ extern "C" int mlr_qk_norm_rope_kv(
         // a multiple of eight tokens
         const int split_values = write_cache && page_size % 8 == 0;
         const int threads_needed = (total_heads - (split_values ? kv_heads : 0)) * lph;
-        qk_norm_rope_kv_vec_kernel<<<dim3(rows, (threads_needed + 255) / 256), 256, 0, stream>>>(
-            (const __bf16*)qkv, ld, (__bf16*)q_out, (__bf16*)k_pages, (__bf16*)v_pages, block_table, max_blocks,
-            slots, positions, q_norm_w, k_norm_w, eps, rope, q_heads, kv_heads, head_dim, page_size, write_cache,
-            split_values);
+        const dim3 grid(rows, (threads_needed + 255) / 256);
+#define MLR_ROPE_VEC(NORM, ROPE)                                                                                   \
+        qk_norm_rope_kv_vec_kernel<NORM, ROPE><<<grid, 256, 0, stream>>>(                                          \
+            (const __bf16*)qkv, ld, (__bf16*)q_out, (__bf16*)k_pages, (__bf16*)v_pages, block_table, max_blocks,  \
+            slots, positions, q_norm_w, k_norm_w, eps, rope, q_heads, kv_heads, head_dim, page_size, write_cache, \
+            split_values)
+        const bool norm = q_norm_w != nullptr && k_norm_w != nullptr;
+        if (norm && rope) MLR_ROPE_VEC(true, true);
+        else if (norm) MLR_ROPE_VEC(true, false);
+        else if (rope) MLR_ROPE_VEC(false, true);
+        else MLR_ROPE_VEC(false, false);
+#undef MLR_ROPE_VEC
         if (split_values) {
             v_cache_write_kernel<<<dim3((rows + 15) / 16, kv_heads), 256, 16 * (head_dim + 8) * sizeof(__bf16), stream>>>(
                 (const __bf16*)qkv, ld, (__bf16*)v_pages, block_table, max_blocks, slots, positions, rows, q_heads,
