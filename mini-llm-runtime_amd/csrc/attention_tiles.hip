@@ -30,6 +30,11 @@
 // in a wavefront some column would need it in nearly every tile otherwise.  The decision is taken per
 // column from the column's own scores, so a column's arithmetic does not depend on its neighbours.
 //
+// Key splits (max_splits > 1), for a step whose groups alone would not fill the GPU (a short portion of a
+// long context): workgroup (group, kv head, split s) takes the keys [s * split_keys, (s + 1) * split_keys),
+// split_keys a multiple of 64, and leaves its columns' (values, maximum, sum) unnormalised in `partial`;
+// `tiles_combine_kernel` merges a column's splits in ascending order.
+//
 // Not handled here (the caller uses the other kernels): head sizes above 128, page sizes that are no power
 // of two, groups whose keys span more than PAGE_IDS pages.
 #include <hip/hip_runtime.h>
@@ -55,7 +60,8 @@ struct TileArgs {
     __bf16* out;                 // [M, q_heads, head_dim]
     const int32_t* group_row0;   // [groups] first batch row of a group
     const int32_t* group_ntok;   // [groups] its tokens (consecutive rows of one request)
-    int groups, max_blocks, q_heads, kv_heads, head_dim, page_size, page_shift, window;
+    float* partial;              // [M, q_heads, max_splits, head_dim + 2] when max_splits > 1
+    int groups, max_blocks, q_heads, kv_heads, head_dim, page_size, page_shift, window, split_keys, max_splits;
     float scale;
 };
 
@@ -86,7 +92,7 @@ __device__ __forceinline__ float max3(float a, float b, float c) {
 }
 
 template <int ND, int NQ>
-__device__ __forceinline__ void tile_group(const TileArgs& a, int grp, int kvh, unsigned char* lds_raw) {
+__device__ __forceinline__ void tile_group(const TileArgs& a, int grp, int kvh, int split, unsigned char* lds_raw) {
     using S = TileShape<ND, NQ>;
     constexpr int D = S::D, DB = S::DB, KPITCH = S::KPITCH, THREADS = S::THREADS;
     int32_t* page_lds = reinterpret_cast<int32_t*>(lds_raw);
@@ -103,6 +109,11 @@ __device__ __forceinline__ void tile_group(const TileArgs& a, int grp, int kvh, 
     const int slot = a.slots[row0], pos0 = a.positions[row0];
     const int lo = a.window > 0 ? max(0, pos0 + 1 - a.window) : 0;    // first key any token of the group sees
     const int ke = pos0 + ntok;                                      // one past the last
+    // the keys of this workgroup: all of them, or those of its split
+    const bool splitting = a.max_splits > 1;
+    const int lo_s = splitting ? max(lo, split * a.split_keys) : lo;
+    const int ke_s = splitting ? min(ke, (split + 1) * a.split_keys) : ke;
+    if (lo_s >= ke_s) return;                                        // no column of the group sees this split
 
     // this wavefront's tokens
     const int tf = (32 * cq) / g;
@@ -137,11 +148,11 @@ __device__ __forceinline__ void tile_group(const TileArgs& a, int grp, int kvh, 
         for (int i = 0; i < 16; ++i) o[db][i] = 0.f;
 
     // page ids of the group's key range, so that a block's loads do not wait for a load of the table
-    const int blk_begin = lo / BLOCK_KEYS, blk_end = (ke + BLOCK_KEYS - 1) / BLOCK_KEYS;
+    const int blk_begin = lo_s / BLOCK_KEYS, blk_end = (ke_s + BLOCK_KEYS - 1) / BLOCK_KEYS;
     const int first_page = (blk_begin * BLOCK_KEYS) >> pshift;
     const int32_t* table = a.block_table + (size_t)slot * a.max_blocks;
     {
-        const int n_pages = min(PAGE_IDS, ((ke + P - 1) >> pshift) - first_page);
+        const int n_pages = min(PAGE_IDS, ((ke_s + P - 1) >> pshift) - first_page);
         for (int i = threadIdx.x; i < n_pages; i += THREADS) page_lds[i] = table[first_page + i];
         __syncthreads();
     }
@@ -349,6 +360,26 @@ __device__ __forceinline__ void tile_group(const TileArgs& a, int grp, int kvh, 
         const float w0 = m_ref > -INFINITY ? __builtin_amdgcn_exp2f(m_ref - m) : 0.f;
         const float w1 = m1 > -INFINITY ? __builtin_amdgcn_exp2f(m1 - m) : 0.f;
         const float l = l_run * w0 + l1 * w1;
+        if (splitting) {
+            // only the splits that hold keys of this column are read by the merge
+            if (split * a.split_keys >= kend_c || (split + 1) * a.split_keys <= kbegin_c) return;
+            float* dst = a.partial + (((size_t)(row0 + tok) * a.q_heads + kvh * g + hh) * a.max_splits + split) * (D + 2);
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int d0 = 32 * db + 8 * j + 4 * h;
+                    if (d0 >= D) continue;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)         // (D + 2 floats a split: no 16-byte alignment)
+                        dst[d0 + r] = o[db][4 * j + r] * w0 + mine[(db * 16 + 4 * j + r) * 64] * w1;
+                }
+            if (h == 0) {
+                dst[D] = m;
+                dst[D + 1] = l;
+            }
+            return;
+        }
         const float inv = l > 0.f ? 1.f / l : 0.f;
         __bf16* dst = a.out + ((size_t)(row0 + tok) * a.q_heads + kvh * g + hh) * D;
 #pragma unroll
@@ -368,6 +399,37 @@ __device__ __forceinline__ void tile_group(const TileArgs& a, int grp, int kvh, 
     }
 }
 
+// The merge of key splits: one wavefront per (group, head, token of the group); a lane takes the channels
+// lane and lane + 64.  Splits are added in ascending order.
+__global__ __launch_bounds__(64) void tiles_combine_kernel(TileArgs a) {
+    const int grp = blockIdx.x, head = blockIdx.y, j = blockIdx.z;
+    if (j >= a.group_ntok[grp]) return;
+    const int D = a.head_dim;
+    const int m = a.group_row0[grp] + j;
+    const int pos = a.positions[m];
+    const int first = a.window > 0 ? max(0, pos + 1 - a.window) / a.split_keys : 0;
+    const int last = min(a.max_splits - 1, pos / a.split_keys);
+    const float* base = a.partial + (((size_t)m * a.q_heads + head) * a.max_splits) * (D + 2);
+    float gmax = -INFINITY;
+    for (int s = first + (int)threadIdx.x; s <= last; s += 64) gmax = fmaxf(gmax, base[(size_t)s * (D + 2) + D]);
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) gmax = fmaxf(gmax, __shfl_xor(gmax, off, 64));
+    const int d0 = min((int)threadIdx.x, D - 1), d1 = min((int)threadIdx.x + 64, D - 1);
+    float den = 0.f, n0 = 0.f, n1 = 0.f;
+    for (int s = first; s <= last; ++s) {
+        const float* p = base + (size_t)s * (D + 2);
+        const float sm = p[D];
+        const float w = sm > -INFINITY ? __builtin_amdgcn_exp2f(sm - gmax) : 0.f;   // maxima are base-2 exponents
+        den += w * p[D + 1];
+        n0 += w * p[d0];
+        n1 += w * p[d1];
+    }
+    const float inv = den > 0.f ? 1.f / den : 0.f;
+    __bf16* dst = a.out + ((size_t)m * a.q_heads + head) * D;
+    if ((int)threadIdx.x < D) dst[threadIdx.x] = (__bf16)(n0 * inv);
+    if ((int)threadIdx.x + 64 < D) dst[threadIdx.x + 64] = (__bf16)(n1 * inv);
+}
+
 // Workgroups of 128 columns take two groups, one after the other: group i and group (groups - 1 - i).
 // Within a long prompt the groups' key ranges grow with their position, so every workgroup gets about the
 // same work.  Workgroups of 64 columns take one group each, the later (longer) groups first, and two of
@@ -382,15 +444,15 @@ __global__ __launch_bounds__(128 * NQ, NQ == 2 ? 2 : 1) void attention_tiles_ker
     if (total % 8 == 0) lin = (lin % 8) * (total / 8) + lin / 8;
     const int first = lin % per_head, kvh = lin / per_head;
     const int second = a.groups - 1 - first;
-    if (NQ == 2) {
-        tile_group<ND, NQ>(a, second, kvh, lds_raw);
+    if (NQ == 2 || a.max_splits > 1) {                  // one group a workgroup, the later ones first
+        tile_group<ND, NQ>(a, second, kvh, blockIdx.z, lds_raw);
         return;
     }
     if (second > first) {
-        tile_group<ND, NQ>(a, second, kvh, lds_raw);
+        tile_group<ND, NQ>(a, second, kvh, 0, lds_raw);
         __syncthreads();
     }
-    tile_group<ND, NQ>(a, first, kvh, lds_raw);
+    tile_group<ND, NQ>(a, first, kvh, 0, lds_raw);
 }
 
 template <int ND, int NQ>
@@ -403,8 +465,12 @@ static int launch_tiles(const TileArgs& a, hipStream_t stream) {
         if (e != hipSuccess) return (int)e;
         prepared = true;
     }
-    dim3 grid(NQ == 2 ? a.groups : (a.groups + 1) / 2, a.kv_heads);
+    const bool single = NQ == 2 || a.max_splits > 1;
+    dim3 grid(single ? a.groups : (a.groups + 1) / 2, a.kv_heads, a.max_splits);
     attention_tiles_kernel<ND, NQ><<<grid, 128 * NQ, lds, stream>>>(a);
+    int err = (int)hipGetLastError();
+    if (err != 0 || a.max_splits <= 1) return err;
+    tiles_combine_kernel<<<dim3(a.groups, a.q_heads, (32 * NQ) / (a.q_heads / a.kv_heads)), 64, 0, stream>>>(a);
     return (int)hipGetLastError();
 }
 
@@ -424,24 +490,28 @@ static int launch_tiles_dim(const TileArgs& a, hipStream_t stream) {
 
 // Groups: group_row0[i] = first batch row of group i, group_ntok[i] = its tokens (consecutive rows of one
 // request, at most columns / (q_heads / kv_heads); columns = 128 or 64).  A group's keys must span at most
-// PAGE_IDS pages.  The cache of num_pages pages must hold fewer than 2^32 elements.  Returns 0, a HIP error
+// PAGE_IDS pages (per key split, with splits).  The cache of num_pages pages must hold fewer than 2^32 elements.
+// With max_splits > 1, `partial` holds M * q_heads * max_splits * (head_dim + 2) floats, M the batch's rows.  Returns 0, a HIP error
 // code, or a negative number for sizes this kernel does not take.
 extern "C" int mlr_attention_tiles(
     const void* q, const void* k_pages, const void* v_pages, const int32_t* block_table, int max_blocks,
     const int32_t* slots, const int32_t* positions, void* out, const int32_t* group_row0,
     const int32_t* group_ntok, int groups, int columns, int q_heads, int kv_heads, int head_dim, int page_size,
-    int num_pages, int window, float scale, hipStream_t stream) {
+    int num_pages, int window, float scale, int split_keys, int max_splits, float* partial, hipStream_t stream) {
     if (groups <= 0) return 0;
     if (head_dim % 16 != 0 || head_dim < 16 || head_dim > 128 || q_heads % kv_heads != 0 ||
         (columns != 128 && columns != 64) || q_heads / kv_heads > columns) return -1;
     if (page_size < 16 || (page_size & (page_size - 1)) != 0) return -2;
+    if (max_splits < 1) max_splits = 1;
+    if (max_splits > 1 && (partial == nullptr || split_keys <= 0 || split_keys % BLOCK_KEYS != 0 ||
+                           max_splits > 65535 || groups > 65535)) return -4;
     // offsets into the cache are 32-bit element counts, a page's stride and id 24-bit factors
     const uint64_t stride = (uint64_t)kv_heads * page_size * head_dim;
     if (stride >= (1u << 24) || num_pages >= (1 << 24) || stride * (uint64_t)num_pages >= (1ull << 32)) return -3;
     int shift = 0;
     while ((1 << shift) < page_size) ++shift;
     TileArgs a{(const __bf16*)q, (const __bf16*)k_pages, (const __bf16*)v_pages, block_table, slots, positions,
-               (__bf16*)out, group_row0, group_ntok, groups, max_blocks, q_heads, kv_heads, head_dim, page_size,
-               shift, window, scale};
+               (__bf16*)out, group_row0, group_ntok, partial, groups, max_blocks, q_heads, kv_heads, head_dim,
+               page_size, shift, window, split_keys, max_splits, scale};
     return columns == 128 ? launch_tiles_dim<4>(a, stream) : launch_tiles_dim<2>(a, stream);
 }

@@ -133,19 +133,34 @@ class StepContext:
         largest of base, 2 base, 4 base, ... that still gives `target_workgroups`; what a token's
         result is does not depend on the choice beyond rounding.  `rows` tokens take part; the partial
         results are indexed by batch row, of which there are `batch_rows`."""
-        base = self.split_keys
-        if base <= 0 or rows > self.split_max_tokens or self.max_context <= base:
+        if rows > self.split_max_tokens:
             return 0, 1, None
-        units = max(1, rows * kv_heads)
+        return self._split(max(1, rows * kv_heads), self.target_workgroups, batch_rows, q_heads, head_dim)
+
+    def group_split(self, groups, batch_rows, kv_heads, q_heads, head_dim, longest=None):
+        """As `attention_split` for `groups` groups of many tokens each (prompt portions), which give
+        one workgroup per (group, kv head).  `longest`: the most keys a workgroup can take without a
+        split; a longer context is split whatever the number of groups."""
+        return self._split(max(1, groups * kv_heads), self.compute_units, batch_rows, q_heads, head_dim, longest)
+
+    def _split(self, units, enough, batch_rows, q_heads, head_dim, longest=None):
+        """`units` workgroups without a split; no split when they are `enough`."""
+        base = self.split_keys
+        forced = longest is not None and self.max_context > longest
+        if base <= 0 or (self.max_context <= base and not forced):
+            return 0, 1, None
         keys = base
         while keys * 2 < self.max_context and units * (-(-self.max_context // (keys * 2))) >= self.target_workgroups:
             keys *= 2
-        if units >= self.target_workgroups:
+        if forced:
+            while keys > base and keys > longest:
+                keys //= 2
+        elif units >= enough:
             return 0, 1, None
         max_splits = -(-self.max_context // keys)
         if max_splits <= 1:
             return 0, 1, None
-        while max_splits > 1024:                     # the merge kernel's limit
+        while max_splits > 1024:                     # the merge kernels' limit
             keys *= 2
             max_splits = -(-self.max_context // keys)
         numel = self.kernels.attention_partial_numel(batch_rows, q_heads, head_dim, max_splits)

@@ -355,14 +355,21 @@ class Kernels:
                _c_int(kv_heads), _c_int(head_dim), _c_int(page_size), _c_int(window or 0), _c_float(scale),
                _stream()), "attention_prefill")
 
-    def tiles_attention_supported(self, q_heads, kv_heads, head_dim, page_size, max_context=0, num_pages=0):
+    def tiles_attention_supported(self, q_heads, kv_heads, head_dim, page_size, max_context=0, num_pages=0,
+                                  split_keys=0):
         """The 32x32-tile kernel for prompt portions: bfloat16, head sizes up to 128 in steps of 16, pages
         of a power of two of keys, at most 16 query heads per kv head, contexts of at most 2048 pages (it
         keeps a group's page ids in LDS), a cache of fewer than 2^32 elements per layer (32-bit offsets)."""
         stride = kv_heads * page_size * head_dim
         return (self.mfma_attention_supported(q_heads, kv_heads, head_dim, page_size) and head_dim <= TILES_MAX_HEAD_DIM
-                and page_size & (page_size - 1) == 0 and max_context <= PREFILL_MAX_PAGES * page_size
+                and page_size & (page_size - 1) == 0
+                and (split_keys > 0 or max_context <= PREFILL_MAX_PAGES * page_size)
                 and stride < 2 ** 24 and num_pages < 2 ** 24 and stride * num_pages < 2 ** 32)
+
+    @staticmethod
+    def tiles_longest_context(page_size):
+        """The most keys that one workgroup of `attention_tiles` can walk (it keeps their page ids in LDS)."""
+        return PREFILL_MAX_PAGES * page_size
 
     @staticmethod
     def tiles_group_tokens(q_heads, kv_heads, columns=TILES_COLUMNS[0]):
@@ -371,19 +378,31 @@ class Kernels:
 
     def attention_tiles(self, q, k_pages, v_pages, block_table, slots, positions, out, group_row0, group_ntok,
                         groups, q_heads, kv_heads, head_dim, page_size, scale, window=None, max_context=None,
-                        columns=TILES_COLUMNS[0]):
+                        columns=TILES_COLUMNS[0], split_keys=0, max_splits=1, partial=None):
         """Attention for prompt portions: groups of up to columns // (q_heads // kv_heads) consecutive rows
         of one request each (columns = 128, or 64 for batches that would not fill the GPU with the larger
-        workgroups); keys and values of a group are staged once through LDS in blocks of 64.  The caller
-        vouches for the groups (consecutive rows of one request, no more tokens than `tiles_group_tokens`)."""
+        workgroups); keys and values of a group are staged once through LDS in blocks of 64.  With
+        max_splits > 1 a group's keys are split over workgroups in ranges of split_keys (a multiple of 64)
+        and merged through `partial`.  The caller vouches for the groups (consecutive rows of one request,
+        no more tokens than `tiles_group_tokens`)."""
         _need(columns in TILES_COLUMNS, lambda: f"attention_tiles: columns must be one of {TILES_COLUMNS}")
         _need(self.tiles_attention_supported(q_heads, kv_heads, head_dim, page_size, num_pages=k_pages.shape[0]),
               "attention_tiles: sizes not supported")
-        _need(block_table.shape[1] <= PREFILL_MAX_PAGES or max_context is not None,
-              "attention_tiles: give max_context when the block table is wider than the kernel's page cache")
-        _need((max_context or 0) <= PREFILL_MAX_PAGES * page_size, "attention_tiles: context too long")
         _tensor(q, "q", self.dtype, ndim=2)
         m = q.shape[0]
+        if max_splits > 1:
+            _need(split_keys > 0 and split_keys % ATTENTION_TILE_KEYS == 0,
+                  lambda: f"split_keys must be a multiple of {ATTENTION_TILE_KEYS}")
+            _need(max_splits <= MAX_KEY_SPLITS and groups <= 65535, "too many key splits or groups for the grid")
+            _need(split_keys // page_size + 2 <= PREFILL_MAX_PAGES, "attention_tiles: a split spans too many pages")
+            _need(partial is not None, "partial buffer needed for split attention")
+            _tensor(partial, "partial", torch.float32, ndim=1)
+            _need(partial.numel() >= self.attention_partial_numel(m, q_heads, head_dim, max_splits),
+                  "partial buffer too small")
+        else:
+            _need(block_table.shape[1] <= PREFILL_MAX_PAGES or max_context is not None,
+                  "attention_tiles: give max_context when the block table is wider than the kernel's page cache")
+            _need((max_context or 0) <= PREFILL_MAX_PAGES * page_size, "attention_tiles: context too long")
         _need(q.shape[1] == q_heads * head_dim, "q: wrong width")
         _tensor(out, "out", self.dtype, (m, q_heads * head_dim))
         self._check_cache(k_pages, v_pages, kv_heads, head_dim, page_size)
@@ -397,7 +416,8 @@ class Kernels:
         _ok(fn(_p(q), _p(k_pages), _p(v_pages), _p(block_table), _c_int(block_table.shape[1]), _p(slots),
                _p(positions), _p(out), _p(group_row0), _p(group_ntok), _c_int(groups), _c_int(columns),
                _c_int(q_heads), _c_int(kv_heads), _c_int(head_dim), _c_int(page_size), _c_int(k_pages.shape[0]),
-               _c_int(window or 0), _c_float(scale), _stream()), "attention_tiles")
+               _c_int(window or 0), _c_float(scale), _c_int(split_keys), _c_int(max_splits), _p(partial),
+               _stream()), "attention_tiles")
 
     # -- sampling ----------------------------------------------------------------------------
     def sample_scratch(self, rows):

@@ -97,19 +97,24 @@ class GqaAttention:
             # prompt portions go to one of the LDS-staged kernels (the 32x32-tile one where it takes the
             # sizes), single tokens and short portions to the one that can split a token's keys over
             # workgroups
-            sizes = (s.q_heads, s.kv_heads, s.head_dim, view.page_size, ctx.max_context)
+            sizes = (s.q_heads, s.kv_heads, s.head_dim, view.page_size)
             g = s.q_heads // s.kv_heads
             tq = max(1, 16 // g)
-            tiles = k.tiles_attention_supported(*sizes, num_pages=view.k_pages.shape[0])
+            # (with key splits the 32x32-tile kernel takes any context length)
+            tiles = k.tiles_attention_supported(*sizes, num_pages=view.k_pages.shape[0], split_keys=ctx.split_keys)
             # workgroups of 128 columns (launched in pairs) unless they would leave half of the compute
             # units idle: then of 64
             columns = 128 if m * s.q_heads > 128 * ctx.compute_units else 64
-            big_factor = (columns // 16 if tiles else 4) if tiles or k.prefill_attention_supported(*sizes) else 0
+            big_factor = (columns // 16 if tiles
+                          else 4 if k.prefill_attention_supported(*sizes, ctx.max_context) else 0)
             small, big, small_rows = ctx.token_groups(tq, big_factor)
             if big[2] and tiles:
+                split_keys, max_splits, partial = ctx.group_split(
+                    big[2], m, s.kv_heads, s.q_heads, s.head_dim, longest=k.tiles_longest_context(view.page_size))
                 k.attention_tiles(q, view.k_pages, view.v_pages, view.block_table, ctx.slots, ctx.positions, attn,
                                   big[0], big[1], big[2], s.q_heads, s.kv_heads, s.head_dim, view.page_size,
-                                  float(s.scale), window=s.window, max_context=ctx.max_context, columns=columns)
+                                  float(s.scale), window=s.window, max_context=ctx.max_context, columns=columns,
+                                  split_keys=split_keys, max_splits=max_splits, partial=partial)
             elif big[2]:
                 k.attention_prefill(q, view.k_pages, view.v_pages, view.block_table, ctx.slots, ctx.positions, attn,
                                     big[0], big[1], big[2], s.q_heads, s.kv_heads, s.head_dim, view.page_size,

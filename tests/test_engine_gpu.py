@@ -76,13 +76,16 @@ def test_every_way_of_cutting_gives_the_plain_logits(model_folders, expected, na
 
 
 @pytest.mark.parametrize("dtype_name", DTYPES)
+@pytest.mark.parametrize("name", TINY)
 @pytest.mark.parametrize("split_keys,split_max_tokens", [(64, 10 ** 6), (0, 0)])
-def test_key_splits_do_not_change_the_result(model_folders, expected, dtype_name, split_keys, split_max_tokens):
-    """Attention over key ranges split across workgroups (forced on for every batch, and off)."""
-    reqs, want = expected["B"]
-    model = load(model_folders, "B", dtype_name)
-    r = runner_for(model, "B", max_tokens=192, split_keys=split_keys, split_max_tokens=split_max_tokens)
-    compare(run_steps(r, last_one_by_one(reqs)), want, dtype_name)
+def test_key_splits_do_not_change_the_result(model_folders, expected, name, dtype_name, split_keys, split_max_tokens):
+    """Attention over key ranges split across workgroups (forced on for every batch, and off): single
+    tokens, and prompt portions of changing size (the kernels for portions have splits of their own)."""
+    reqs, want = expected[name]
+    model = load(model_folders, name, dtype_name)
+    for trace in (last_one_by_one(reqs), portions(reqs, sizes=(40, 3, 64, 17, 2, 33))):
+        r = runner_for(model, name, max_tokens=192, split_keys=split_keys, split_max_tokens=split_max_tokens)
+        compare(run_steps(r, trace), want, dtype_name)
 
 
 @pytest.mark.parametrize("dtype_name", DTYPES)

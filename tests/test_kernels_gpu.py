@@ -345,14 +345,20 @@ def test_paged_attention(dtype, case):
         return
     # the 32x32-tile kernel for prompt portions, with both sizes of workgroup: groups of as many tokens as a
     # workgroup takes, and of fewer
-    for columns, big in ((128, k.tiles_group_tokens(hq, hkv, 128)), (128, 8 * tq), (64, k.tiles_group_tokens(hq, hkv, 64)),
-                         (64, 3 * tq)):
+    for columns, big, split in ((128, k.tiles_group_tokens(hq, hkv, 128), 0), (128, 8 * tq, 0),
+                                (64, k.tiles_group_tokens(hq, hkv, 64), 0), (64, 3 * tq, 0),
+                                (128, k.tiles_group_tokens(hq, hkv, 128), 64), (64, 3 * tq, 128)):
         first = list(range(0, lengths[0], big))
         count = [min(big, lengths[0] - r) for r in first]
         out4 = torch.full((m, hq * d), float("nan"), dtype=dtype, device="cuda")
+        splits, part = 1, None
+        if split:
+            splits = (max_len + split - 1) // split
+            part = torch.full((k.attention_partial_numel(m, hq, d, splits),), float("nan"), device="cuda")
         k.attention_tiles(q.view(m, hq * d).cuda(), k_pages.cuda(), v_pages.cuda(), table.cuda(), slots, pos, out4,
                           torch.tensor(first, dtype=torch.int32).cuda(), torch.tensor(count, dtype=torch.int32).cuda(),
-                          len(first), hq, hkv, d, page, scale, window=window, columns=columns)
+                          len(first), hq, hkv, d, page, scale, window=window, columns=columns,
+                          split_keys=split, max_splits=splits, partial=part)
         got = out4.double().cpu().view(m, hq, d)
         for i in range(lengths[0]):
             torch.testing.assert_close(got[i], wants[i], **tol(dtype))
