@@ -26,7 +26,7 @@ HIP_FLAGS = ["-O3", "-std=c++17", "-shared", "-fPIC", f"--offload-arch={ARCH}",
              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 HOST_FLAGS = ["-O2", "-std=c++17", "-shared", "-fPIC"]
 
-# name -> (sources relative to csrc/, headers it includes, depends on the element type)
+# name -> (sources relative to csrc/, headers it includes, depends on the element type[, extra link flags])
 HIP_LIBRARIES = {
     "elementwise": (["elementwise.hip"], ["common.h"], True),
     "rope_kv": (["rope_kv.hip"], ["common.h"], True),
@@ -34,6 +34,7 @@ HIP_LIBRARIES = {
     "gemm": (["gemm.hip"], ["common.h"], True),
     "attention_tiles": (["attention_tiles.hip"], [], False),      # bfloat16 only by nature
     "sampling": (["sampling.hip"], [], False),
+    "library_gemm": (["library_gemm.hip"], [], False, ["-lhipblaslt"]),      # host code around hipBLASLt
 }
 HOST_LIBRARIES = {
     "host": (["host/cache_manager.cpp", "host/scheduler.cpp"], []),
@@ -95,12 +96,13 @@ def _plan(name, tag):
         cmd = [_find_cxx(), *HOST_FLAGS, "-o", out] + [os.path.join(CSRC, s) for s in sources]
         flags = HOST_FLAGS
     else:
-        sources, headers, typed = HIP_LIBRARIES[name]
+        sources, headers, typed, *rest = HIP_LIBRARIES[name]
+        link = rest[0] if rest else []
         suffix = f"_{tag}" if typed else ""
         out = os.path.join(_lib_dir(), f"libmlr_{name}{suffix}.so")
         defs = [f"-DMLR_BF16={1 if tag == 'bf16' else 0}"] if typed else []
-        cmd = [_find_hipcc(), *HIP_FLAGS, *defs, "-o", out] + [os.path.join(CSRC, s) for s in sources]
-        flags = HIP_FLAGS + defs
+        cmd = [_find_hipcc(), *HIP_FLAGS, *defs, "-o", out] + [os.path.join(CSRC, s) for s in sources] + link
+        flags = HIP_FLAGS + defs + link
     h = hashlib.sha256(" ".join(flags).encode())
     for rel in sources + headers:
         with open(os.path.join(CSRC, rel), "rb") as f:

@@ -22,6 +22,7 @@ _ptr = ctypes.c_void_p
 MAX_HEAD_DIM = 256          # the attention and rotation kernels keep head_dim / 64 values per lane
 ATTENTION_TILE_KEYS = 64
 LIBRARY_GEMM_MIN_ROWS = 16    # above this many rows the bfloat16 engine's projections go to the library
+LIBRARY_GEMM_WORKSPACE = 32 << 20    # bytes of scratch memory that the library may use
 PREFILL_MAX_PAGES = 2048      # page ids of one group that the prompt-portion attention kernel keeps in LDS
 TILES_MAX_HEAD_DIM = 128      # the 32x32-tile kernel for prompt portions keeps two sets of accumulators per lane
 TILES_COLUMNS = (128, 64)     # (token, head) columns of one of its workgroups: the usual and the small one
@@ -80,6 +81,7 @@ class Kernels:
             raise KernelError("no GPU is visible: the engine's kernels are HIP only")
         self.dtype = dtype
         self.library_gemm = library_gemm
+        self._library_workspace = None      # scratch memory of the vendor library's products, allocated once
         self._libs = {}
 
     # -- libraries ---------------------------------------------------------------------------
@@ -162,9 +164,13 @@ class Kernels:
         _need(out.dtype in (self.dtype, torch.float32), lambda: f"gemm: output type {out.dtype} not supported")
         _tensor(out, "out", out.dtype, (m, n))
         if self.library_gemm and self.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and m > LIBRARY_GEMM_MIN_ROWS:
-            # many rows: a plain matrix product, handed to the vendor library (hipBLASLt through torch),
-            # as the reference hands its projections to cuBLAS (src/minillm/cuda/matrix.cpp:11-37)
-            torch.matmul(a, w.t(), out=out)
+            # many rows: a plain matrix product, handed to the vendor library (hipBLASLt), as the reference
+            # hands its projections to cuBLAS (src/minillm/cuda/matrix.cpp:11-37)
+            if self._library_workspace is None:
+                self._library_workspace = torch.empty(LIBRARY_GEMM_WORKSPACE, dtype=torch.uint8, device=a.device)
+            ws = self._library_workspace
+            _ok(self._lib("library_gemm").mlr_library_gemm(_p(a), _p(w), _p(out), _c_int(m), _c_int(n), _c_int(k),
+                                                           _p(ws), _c_size_t(ws.numel()), _stream()), "library_gemm")
             return
         fn = self._lib("gemm").mlr_gemm
         _ok(fn(_p(a), _p(w), _p(out), _c_int(m), _c_int(n), _c_int(k),

@@ -97,6 +97,8 @@ class DecoderModel:
 
     def libraries(self):
         names = {"elementwise", "gemm"}
+        if self.dtype == torch.bfloat16:
+            names.add("library_gemm")            # projections of many rows go to the vendor library
         for block in self.blocks:
             for part in block.parts().values():
                 if hasattr(part, "libraries"):

@@ -265,6 +265,11 @@ def plain_attention(q, keys, values, scale, window):
     (14, 2, 192, 16, [40], None, 0),
     (2, 1, 224, 16, [40], None, 0),
     (4, 2, 32, 16, [300], 70, 0),
+    (8, 2, 64, 64, [333, 20], None, 128),
+    (4, 2, 128, 128, [400, 130], None, 0),
+    (6, 2, 96, 256, [300], 100, 64),
+    (3, 1, 112, 32, [200], None, 0),
+    (10, 2, 16, 16, [150, 64], 64, 0),
 ])
 def test_paged_attention(dtype, case):
     """Every length is one request whose LAST token is the query (a decoded token) plus, for the

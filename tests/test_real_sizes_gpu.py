@@ -72,3 +72,33 @@ def test_prompt_of_256_tokens_every_way(folder, expected, dtype_name):
     top = np.sort(row)[-2:]
     if dtype_name == "float32" or top[1] - top[0] > 0.05 * np.abs(row).max():
         assert token == int(np.argmax(row))
+
+
+def test_graph_replays_with_library_products_match_eager(folder):
+    """24 requests decode together: their projections have more than 16 rows and go to the vendor library,
+    inside the captured graph.  Every replay (with eager work and synchronisations between the replays) must
+    give what the same steps give without a graph: a library call that records a clearing node would show
+    here as a difference on a later replay."""
+    from mini_llm_runtime_amd.engine import Entry, Runner
+    from mini_llm_runtime_amd.parts import DecoderModel
+    model = DecoderModel.load(folder, torch.bfloat16)
+    n = 24
+    prompts = make_requests(CFG["vocab_size"], [9 + (5 * i) % 23 for i in range(n)], seed=23)
+    feeds = make_requests(CFG["vocab_size"], [8] * n, seed=29)
+    outs = []
+    for use_graphs in (True, False):
+        r = Runner(model, max_tokens=n * 64, max_slots=n, page_size=16, use_graphs=use_graphs)
+        slots = [r.open_request() for _ in range(n)]
+        for s, toks in zip(slots, prompts.values()):
+            r.step([Entry(s, toks, [])])
+        steps = []
+        for j in range(8):
+            logits = r.step([Entry(s, [feeds[f"r{i}"][j]], [0]) for i, s in enumerate(slots)])
+            steps.append(logits.float().cpu().numpy().copy())
+            torch.cuda.synchronize()
+            _ = (torch.ones(1000, device="cuda") * 2).sum().item()        # eager work between the replays
+        outs.append(steps)
+        assert r.use_graphs == use_graphs
+    for j, (a, b) in enumerate(zip(*outs)):
+        assert np.isfinite(a).all(), j
+        np.testing.assert_array_equal(a, b, err_msg=f"decode step {j}")
