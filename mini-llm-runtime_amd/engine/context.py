@@ -40,6 +40,11 @@ class Workspace:
     def bytes(self):
         return sum(b.numel() * b.element_size() for b in self._buffers.values())
 
+    def buffers(self):
+        """The buffers as they are now.  A captured graph holds on to this list: it keeps using the
+        memory it was captured with, also after a larger step has made a name's buffer grow."""
+        return list(self._buffers.values())
+
 
 class Uploader:
     """Small host-to-device copies through one pinned buffer.  The copy is asynchronous; an event
@@ -85,11 +90,11 @@ class StepContext:
         self.max_context = 0          # largest position + 1 among the step's tokens
         self._groups = {}
         self._group_upload = None
-        self.single_token_groups = None
+        self.fixed_groups = None      # a captured step's groups: {key: token_groups' result}, in tensors of their own
 
     def begin_step(self):
         self._groups = {}
-        self.single_token_groups = None
+        self.fixed_groups = None
 
     def token_groups(self, tokens_per_group, big_factor=0):
         """The step's rows cut into groups of consecutive tokens of one request, as device int32 vectors
@@ -101,8 +106,8 @@ class StepContext:
         hit = self._groups.get(key)
         if hit is not None:
             return hit
-        if self.single_token_groups is not None:      # a step of single tokens with fixed buffers
-            return self.single_token_groups, (None, None, 0), self.n_tokens
+        if self.fixed_groups is not None and key in self.fixed_groups:
+            return self.fixed_groups[key]
         first, count, big_first, big_count = [], [], [], []
         small_rows = 0
         for _, row, n, _ in self.segments:
@@ -117,11 +122,18 @@ class StepContext:
                     first.append(row + i)
                     count.append(min(tokens_per_group, n - i))
         g, gb = len(first), len(big_first)
-        dev = self.workspace.get(f"token_groups_{tokens_per_group}_{big_factor}", (2 * (g + gb),), torch.int32)
-        if self._group_upload is None:
-            self._group_upload = Uploader(4096, dev.device)
-        self._group_upload.send(first + count + big_first + big_count, dev)
+        if self.fixed_groups is not None:
+            # a step that is to be captured: its groups depend on the lengths of its entries only, so they
+            # get a tensor of their own once (this is the eager run before the capture) and stay there
+            dev = torch.tensor(first + count + big_first + big_count + [0], dtype=torch.int32, device=self.workspace.device)
+        else:
+            dev = self.workspace.get(f"token_groups_{tokens_per_group}_{big_factor}", (2 * (g + gb),), torch.int32)
+            if self._group_upload is None:
+                self._group_upload = Uploader(4096, dev.device)
+            self._group_upload.send(first + count + big_first + big_count, dev)
         hit = ((dev[:g], dev[g:2 * g], g), (dev[2 * g:2 * g + gb], dev[2 * g + gb:2 * g + 2 * gb], gb), small_rows)
+        if self.fixed_groups is not None:
+            self.fixed_groups[key] = hit
         self._groups[key] = hit
         return hit
 

@@ -31,7 +31,7 @@ class Entry:
 class Runner:
     def __init__(self, model, max_tokens, max_slots=4, max_length=None, max_batch_tokens=None,
                  page_size=16, split_keys=256, split_max_tokens=256, use_graphs=True, graph_max_batch=256,
-                 target_workgroups=512):
+                 target_workgroups=512, graph_max_tokens=512, graph_after=2, max_graphs=48):
         self.model = model
         self.dtype, self.device = model.dtype, model.device
         spec = model.spec
@@ -49,11 +49,16 @@ class Runner:
         self._meta = torch.empty(4 * self.max_batch_tokens, dtype=torch.int32, device=self.device)
         self.poisoned = False
         self.steps = 0
-        # steps of single tokens (decoding) are launch-bound: after a first eager run a batch size is
-        # captured once as a HIP graph over fixed buffers and replayed from then on
+        # steps of few tokens are launch-bound: after a first eager run a step's shape is captured once
+        # as a HIP graph over fixed buffers and replayed from then on
         self.use_graphs = use_graphs and model.graph_safe()
-        self.graph_max_batch = graph_max_batch
-        self._decode_graphs = {}
+        self.graph_max_batch = graph_max_batch            # single tokens in a captured step, at most
+        self.graph_max_tokens = max(graph_max_tokens, graph_max_batch)     # tokens in a captured step, at most
+        self.graph_after = graph_after                    # a mixed shape is captured after it came this often
+        self.max_graphs = max_graphs                      # captured shapes kept (least recently used goes)
+        self._graphs = {}
+        self._seen = {}
+        self.graph_failures = 0                           # shapes whose replays did not match the eager run
 
     # -- requests ------------------------------------------------------------------------------
     def open_request(self):
@@ -68,42 +73,101 @@ class Runner:
     def free_slots(self):
         return self.cache.book.free_slots()
 
-    # -- decoding steps as graphs --------------------------------------------------------------
-    def _decode_step(self, entries, first):
-        """One token per request, logits wanted for each: the same kernels as any step, launched from a
-        captured graph.  The graph's buffers are fixed: token ids, positions, slots and wanted rows live
-        in a vector of their own per batch size, key splits are laid out for the longest context, and the
-        logits land in the usual scratch buffer."""
-        n = len(entries)
-        state = self._decode_graphs.get(n)
+    # -- steps as graphs -----------------------------------------------------------------------
+    def _signature(self, entries):
+        """What a captured step is fixed to: how many tokens every entry brings and where it wants logits."""
+        return tuple((len(e.tokens), tuple(int(w) for w in e.want)) for e in entries)
+
+    def _graph_wanted(self, entries, total, sig):
+        """Steps are launch-bound unless they bring many tokens.  Steps of single tokens with logits for
+        each (decoding) are captured the second time they come, others (portions beside decoded tokens)
+        once their shape has come `graph_after` times: a prompt's last portion rarely comes again."""
+        if not self.use_graphs or total > self.graph_max_tokens:
+            return False
+        if sig in self._graphs:
+            return True
+        if total == len(entries) and all(w == (0,) for _, w in sig):
+            return total <= self.graph_max_batch
+        seen = self._seen.get(sig, 0) + 1
+        self._seen[sig] = seen
+        if len(self._seen) > 4096:
+            self._seen.clear()
+        return seen > self.graph_after
+
+    def _graph_step(self, entries, first, total, sig):
+        """The same kernels as any step, launched from a captured graph.  The graph's buffers are fixed:
+        token ids, positions and slots live in a vector of their own per shape (the wanted rows and the
+        token groups, which depend on the shape only, are written there once), key splits are laid out
+        for the longest context, and the logits land in the scratch buffer of the capture.  A shape's
+        first run is eager (it sizes the scratch buffers), the second is captured; the capture is then
+        replayed twice on the same inputs and compared with the eager result, and a shape whose replays
+        differ (a library call that records a clearing node would do that) stays eager for good."""
+        state = self._graphs.get(sig)
         if state is None:
-            meta = torch.empty(4 * n + 2 * n, dtype=torch.int32, device=self.device)
-            meta[3 * n:4 * n] = torch.arange(n, dtype=torch.int32, device=self.device)      # wanted rows
-            meta[4 * n:5 * n] = torch.arange(n, dtype=torch.int32, device=self.device)      # groups: row i ...
-            meta[5 * n:6 * n] = 1                                                           # ... one token each
-            state = dict(meta=meta, upload=Uploader(3 * n, self.device), graph=None, logits=None, runs=0)
-            self._decode_graphs[n] = state
+            rows, base = [], 0
+            for n, want in sig:
+                rows.extend(base + w for w in want)
+                base += n
+            meta = torch.empty(3 * total + max(len(rows), 1), dtype=torch.int32, device=self.device)
+            if rows:
+                meta[3 * total:3 * total + len(rows)] = torch.tensor(rows, dtype=torch.int32, device=self.device)
+            state = dict(meta=meta, upload=Uploader(3 * total, self.device), graph=None, logits=None, runs=0,
+                         rows=len(rows), groups={}, keep=None, eager=False)
+            self._graphs[sig] = state
+            while len(self._graphs) > self.max_graphs:
+                self._graphs.pop(next(iter(self._graphs)))
+        else:
+            self._graphs[sig] = self._graphs.pop(sig)        # most recently used last
         meta = state["meta"]
-        state["upload"].send([int(e.tokens[0]) for e in entries] + list(first) + [e.slot for e in entries], meta)
+        ids, pos, slot_of, segments = [], [], [], []
+        for e, p0 in zip(entries, first):
+            n = len(e.tokens)
+            segments.append((e.slot, len(ids), n, p0))
+            ids.extend(int(t) for t in e.tokens)
+            pos.extend(range(p0, p0 + n))
+            slot_of.extend([e.slot] * n)
+        state["upload"].send(ids + pos + slot_of, meta)
         if state["graph"] is not None:
             state["graph"].replay()
             return state["logits"]
         ctx = self.ctx
         ctx.begin_step()
-        ctx.n_tokens = n
-        ctx.token_ids, ctx.positions, ctx.slots = meta[0:n], meta[n:2 * n], meta[2 * n:3 * n]
-        ctx.segments = [(e.slot, i, 1, p0) for i, (e, p0) in enumerate(zip(entries, first))]
+        ctx.n_tokens = total
+        ctx.token_ids, ctx.positions, ctx.slots = meta[0:total], meta[total:2 * total], meta[2 * total:3 * total]
+        ctx.segments = segments
+        r = state["rows"]
+        want_rows = meta[3 * total:3 * total + r] if r else None
+        if state["eager"]:                                # a shape whose capture did not hold
+            ctx.max_context = max(p0 + n for (_, _, n, p0) in segments)
+            return self.model.forward(ctx, want_rows)
         ctx.max_context = self.max_length                 # the graph must serve every later context
-        ctx.single_token_groups = (meta[4 * n:5 * n], meta[5 * n:6 * n], n)        # groups of one token each
-        want_rows = meta[3 * n:4 * n]
+        ctx.fixed_groups = state["groups"]
         state["runs"] += 1
         if state["runs"] == 1:                            # first time: eager, sizes the scratch buffers
             return self.model.forward(ctx, want_rows)
+        reference = self.model.forward(ctx, want_rows)    # (running a step again writes the same cache entries)
+        probe = reference if reference is not None else self.workspace.get("hidden", (total, self.model.spec.hidden),
+                                                                           torch.float32)
+        expect = probe.clone()
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             logits = self.model.forward(ctx, want_rows)
+        state["keep"] = self.workspace.buffers()
+        ok = True
+        for _ in range(2):
+            graph.replay()
+            got = logits if logits is not None else probe
+            scale = float(expect.abs().max())
+            ok = ok and bool(torch.isfinite(got).all() == torch.isfinite(expect).all()) and \
+                float((got - expect).abs().nan_to_num(0.0).max()) <= 1e-3 * max(scale, 1e-30)
+        if not ok:
+            state["eager"], state["keep"] = True, None
+            self.graph_failures += 1
+            ctx.fixed_groups = None
+            ctx.begin_step()
+            ctx.max_context = max(p0 + n for (_, _, n, p0) in segments)
+            return self.model.forward(ctx, want_rows)
         state["graph"], state["logits"] = graph, logits
-        graph.replay()
         return logits
 
     # -- the step ------------------------------------------------------------------------------
@@ -137,9 +201,9 @@ class Runner:
         counts = [len(e.tokens) for e in entries]
         first = self.cache.commit_first(slots, counts)    # raises with nothing changed, else takes the pages
         try:
-            if (self.use_graphs and total == len(entries) <= self.graph_max_batch
-                    and all(list(e.want) == [0] for e in entries)):
-                logits = self._decode_step(entries, first)
+            sig = self._signature(entries) if self.use_graphs and total <= self.graph_max_tokens else None
+            if sig is not None and self._graph_wanted(entries, total, sig):
+                logits = self._graph_step(entries, first, total, sig)
                 self.cache.retire(slots)
                 self.steps += 1
                 return logits

@@ -89,6 +89,33 @@ def test_key_splits_do_not_change_the_result(model_folders, expected, name, dtyp
 
 
 @pytest.mark.parametrize("dtype_name", DTYPES)
+@pytest.mark.parametrize("name", TINY)
+def test_a_step_shape_that_comes_again_is_captured_and_stays_right(model_folders, plain_models, name, dtype_name):
+    """A portion of 20 tokens of one request beside single tokens of two others, ten times over: from the
+    fifth time on the step is a replayed graph.  Every step's logits against the plain ones."""
+    vocab = TINY[name]["vocab_size"]
+    reqs = make_requests(vocab, [215, 40, 33], seed=31)
+    want = plain_logits(plain_models[name], reqs)
+    model = load(model_folders, name, dtype_name)
+    r = runner_for(model, name, max_tokens=384)
+    a, b, c = reqs["r0"], reqs["r1"], reqs["r2"]
+    steps = [dict(step=0, entries=[dict(id="r0", tokens=a[:15], want=[14]), dict(id="r1", tokens=b[:30], want=[29]),
+                                   dict(id="r2", tokens=c[:23], want=[22])], end=[])]
+    for i in range(10):
+        steps.append(dict(step=1 + i, end=[], entries=[
+            dict(id="r0", tokens=a[15 + 20 * i:35 + 20 * i], want=[0, 19]),
+            dict(id="r1", tokens=[b[30 + i]], want=[0]), dict(id="r2", tokens=[c[23 + i]], want=[0])]))
+    steps[-1]["end"] = ["r0", "r1", "r2"]
+    got = run_steps(r, steps)
+    compare(got, {k: v for k, v in want.items() if k in got}, dtype_name)
+    assert len(got) == 3 + 10 * 4
+    shape = ((20, (0, 19)), (1, (0,)), (1, (0,)))
+    assert r.graph_failures == 0 and r._graphs[shape]["graph"] is not None
+    r.cache.check()
+    assert r.cache.free_pages() == r.cache.num_pages
+
+
+@pytest.mark.parametrize("dtype_name", DTYPES)
 @pytest.mark.parametrize("name", ["A", "C"])
 def test_long_decoding(model_folders, plain_models, name, dtype_name):
     """A five-token prompt, then 600 tokens one by one (teacher-forced): crosses many pages and key tiles."""
@@ -156,7 +183,8 @@ def test_steady_steps_allocate_nothing(model_folders):
     r.step([Entry(s, list(range(40)), [39])])
     for t in range(3):                                   # eager, then captured as a graph, then replayed
         r.step([Entry(s, [t], [0])])
-    r.step([Entry(s, [5, 6], [1])])
+    for t in range(5):                                   # a shape that comes again and again is captured too
+        r.step([Entry(s, [5, 6], [1])])
     torch.cuda.synchronize()
     before = torch.cuda.memory_stats()["allocation.all.allocated"]
     for t in range(30):
