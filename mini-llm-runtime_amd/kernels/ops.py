@@ -374,8 +374,9 @@ class Kernels:
 
     @staticmethod
     def tiles_longest_context(page_size):
-        """The most keys that one workgroup of `attention_tiles` can walk (it keeps their page ids in LDS)."""
-        return PREFILL_MAX_PAGES * page_size
+        """The most keys that one workgroup of `attention_tiles` can walk (it keeps their page ids in LDS;
+        a key split that does not start at a page's edge touches one page more)."""
+        return (PREFILL_MAX_PAGES - 2) * page_size
 
     @staticmethod
     def tiles_group_tokens(q_heads, kv_heads, columns=TILES_COLUMNS[0]):

@@ -649,3 +649,43 @@ def test_norm_gemm(mnk, gated):
         else:
             want = xn @ w.double().T
         torch.testing.assert_close(out.double(), want, atol=2e-2 * float(want.abs().max()), rtol=2e-2)
+
+
+def test_prompt_portion_beyond_the_page_cache_of_a_workgroup():
+    """A portion of 70 tokens at the end of a context of 33 000 keys: more pages than a workgroup of the
+    32x32-tile kernel keeps, so the keys must be split; unsplit the call is refused."""
+    from mini_llm_runtime_amd.kernels.ops import KernelError
+    dtype = torch.bfloat16
+    k = kernels(dtype)
+    hq, hkv, d, page, L, n = 2, 1, 64, 16, 33000, 70
+    g = torch.Generator().manual_seed(77)
+    kk = torch.randn((L, hkv, d), generator=g).to(dtype)
+    vv = torch.randn((L, hkv, d), generator=g).to(dtype)
+    blocks = (L + page - 1) // page
+    perm = torch.randperm(blocks, generator=g)
+    table = perm.to(torch.int32)[None, :].contiguous()
+    k_pages = torch.zeros((blocks, hkv, page, d), dtype=dtype)
+    v_pages = torch.zeros((blocks, hkv, d, page), dtype=dtype)
+    pad = blocks * page - L
+    kp = torch.cat([kk, torch.zeros((pad, hkv, d), dtype=dtype)]).view(blocks, page, hkv, d)
+    vp = torch.cat([vv, torch.zeros((pad, hkv, d), dtype=dtype)]).view(blocks, page, hkv, d)
+    k_pages[perm] = kp.permute(0, 2, 1, 3)
+    v_pages[perm] = vp.permute(0, 2, 3, 1)
+    q = (torch.randn((n, hq, d), generator=g) * 2).to(dtype)
+    pos = torch.arange(L - n, L, dtype=torch.int32).cuda()
+    slots = torch.zeros(n, dtype=torch.int32).cuda()
+    first = torch.tensor([0, 64], dtype=torch.int32).cuda()
+    count = torch.tensor([64, 6], dtype=torch.int32).cuda()
+    out = torch.full((n, hq * d), float("nan"), dtype=dtype, device="cuda")
+    args = (q.view(n, hq * d).cuda(), k_pages.cuda(), v_pages.cuda(), table.cuda(), slots, pos, out, first, count, 2,
+            hq, hkv, d, page, 1 / math.sqrt(d))
+    with pytest.raises(KernelError):
+        k.attention_tiles(*args, max_context=L)
+    split = 16384
+    splits = (L + split - 1) // split
+    part = torch.full((k.attention_partial_numel(n, hq, d, splits),), float("nan"), device="cuda")
+    k.attention_tiles(*args, max_context=L, split_keys=split, max_splits=splits, partial=part)
+    got = out.double().cpu().view(n, hq, d)
+    for i in (0, 1, 31, 63, 64, 69):
+        want = plain_attention(q[i].double(), kk[:L - n + i + 1].double(), vv[:L - n + i + 1].double(), 1 / math.sqrt(d), None)
+        torch.testing.assert_close(got[i], want, **tol(dtype))
