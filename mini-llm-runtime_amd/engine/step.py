@@ -94,6 +94,19 @@ class Runner:
             self._seen.clear()
         return seen > self.graph_after
 
+    @staticmethod
+    def _replays_match(graph, result, expect):
+        """Replays the fresh capture twice on the inputs of the eager run that gave `expect`; `result` is
+        the tensor that the graph writes."""
+        scale = max(float(expect.abs().nan_to_num(0.0).max()), 1e-30)
+        for _ in range(2):
+            graph.replay()
+            if bool(torch.isfinite(result).all()) != bool(torch.isfinite(expect).all()):
+                return False
+            if float((result - expect).abs().nan_to_num(0.0).max()) > 1e-3 * scale:
+                return False
+        return True
+
     def _graph_step(self, entries, first, total, sig):
         """The same kernels as any step, launched from a captured graph.  The graph's buffers are fixed:
         token ids, positions and slots live in a vector of their own per shape (the wanted rows and the
@@ -153,13 +166,7 @@ class Runner:
         with torch.cuda.graph(graph):
             logits = self.model.forward(ctx, want_rows)
         state["keep"] = self.workspace.buffers()
-        ok = True
-        for _ in range(2):
-            graph.replay()
-            got = logits if logits is not None else probe
-            scale = float(expect.abs().max())
-            ok = ok and bool(torch.isfinite(got).all() == torch.isfinite(expect).all()) and \
-                float((got - expect).abs().nan_to_num(0.0).max()) <= 1e-3 * max(scale, 1e-30)
+        ok = self._replays_match(graph, logits if logits is not None else probe, expect)
         if not ok:
             state["eager"], state["keep"] = True, None
             self.graph_failures += 1

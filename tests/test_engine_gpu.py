@@ -115,6 +115,34 @@ def test_a_step_shape_that_comes_again_is_captured_and_stays_right(model_folders
     assert r.cache.free_pages() == r.cache.num_pages
 
 
+@pytest.mark.parametrize("mode", ["evict", "mismatch"])
+def test_graphs_that_are_dropped_or_do_not_hold(model_folders, plain_models, mode, monkeypatch):
+    """With room for one captured shape, two alternating shapes push each other out again and again; and a
+    shape whose replays do not match its eager run stays eager.  The logits are the plain ones either way."""
+    from mini_llm_runtime_amd.engine import Runner
+    name, dtype_name = "A", "bfloat16"
+    reqs = make_requests(TINY[name]["vocab_size"], [120, 60], seed=37)
+    want = plain_logits(plain_models[name], reqs)
+    model = load(model_folders, name, dtype_name)
+    if mode == "mismatch":
+        monkeypatch.setattr(Runner, "_replays_match", staticmethod(lambda graph, result, expect: False))
+    r = runner_for(model, name, max_tokens=256, max_graphs=1 if mode == "evict" else 48, graph_after=0)
+    a, b = reqs["r0"], reqs["r1"]
+    steps = [dict(step=0, entries=[dict(id="r0", tokens=a[:20], want=[19]), dict(id="r1", tokens=b[:30], want=[29])], end=[])]
+    for i in range(12):                                  # a portion of 8 beside a single token; then two single tokens
+        steps.append(dict(step=1 + 2 * i, end=[], entries=[dict(id="r0", tokens=a[20 + 8 * i:28 + 8 * i], want=[7]),
+                                                           dict(id="r1", tokens=[b[30 + 2 * i]], want=[0])]))
+        steps.append(dict(step=2 + 2 * i, end=[], entries=[dict(id="r1", tokens=[b[31 + 2 * i]], want=[0])]))
+    steps[-1]["end"] = ["r0", "r1"]
+    got = run_steps(r, steps)
+    compare(got, {k: v for k, v in want.items() if k in got}, dtype_name)
+    if mode == "evict":
+        assert len(r._graphs) == 1 and r.graph_failures == 0
+    else:
+        tried = [st for st in r._graphs.values() if st["runs"] > 1]
+        assert r.graph_failures == 2 == len(tried) and all(st["eager"] and st["graph"] is None for st in tried)
+
+
 @pytest.mark.parametrize("dtype_name", DTYPES)
 @pytest.mark.parametrize("name", ["A", "C"])
 def test_long_decoding(model_folders, plain_models, name, dtype_name):
