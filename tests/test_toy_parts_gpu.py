@@ -2,7 +2,8 @@
 architecture, both defined here, are registered, built, loaded from a safetensors folder and stepped --
 whole and in portions, beside each other in one batch -- without a change to the framework's files.
 A second toy architecture shows that the run order is data: a layer named twice, and a run that reads
-another run's cache."""
+another run's cache.  A third has a feed-forward with routing (three small experts, the best one per
+token) and another position encoding (a rotation with its own angles) under the framework's attention."""
 import json
 import math
 import os
@@ -62,9 +63,84 @@ def register_toys():
                     state[slot, self.hidden] = count[-1]
             return out
 
-    def attention(hidden, heads, kv_heads, head_dim, eps):
+    def attention(hidden, heads, kv_heads, head_dim, eps, position=None):
         return AttentionSpec("gqa_attention", hidden, heads, kv_heads, head_dim, 1 / math.sqrt(head_dim),
-                             NormSpec("rmsnorm", head_dim, eps), PositionSpec("rope_split_half", head_dim, 10000.0))
+                             NormSpec("rmsnorm", head_dim, eps),
+                             position or PositionSpec("rope_split_half", head_dim, 10000.0))
+
+    @dataclass(frozen=True)
+    class LinearRotationSpec:
+        kind: str
+        dim: int
+        shift: int
+
+    @register_part("position", "toy_rotation_linear")
+    class LinearRotation:
+        """Split-half rotation by the angle (position + shift) / (1 + j) for the pair j: the framework's
+        attention only asks a position encoding for its table of cosines and sines."""
+
+        def __init__(self, spec):
+            self.dim, self.shift = spec.dim, spec.shift
+            self._tables = {}
+
+        def rotation_table(self, max_positions, device):
+            key = (max_positions, str(device))
+            if key not in self._tables:
+                angle = linear_angles(np.arange(max_positions), self.dim, self.shift)
+                self._tables[key] = torch.from_numpy(np.concatenate([np.cos(angle), np.sin(angle)], axis=1)
+                                                     .astype(np.float32)).to(device)
+            return self._tables[key]
+
+    @dataclass(frozen=True)
+    class RoutedSpec:
+        kind: str
+        hidden: int
+        inner: int
+        experts: int
+
+    @register_part("ffn", "toy_routed")
+    class Routed:
+        """The expert with the largest router logit (32-bit) feeds the token forward, weighted by its softmax
+        share among all experts; an expert is a SwiGLU of its own.  Rows are gathered per expert and run
+        through the framework's projections."""
+        graph_safe = False       # which rows go to which expert is decided on the host
+
+        def __init__(self, spec):
+            self.spec = spec
+
+        def weight_specs(self):
+            s = self.spec
+            specs = {"router": WeightSpec((s.experts, s.hidden), keep_float32=True)}
+            for e in range(s.experts):
+                specs[f"expert{e}.gate_up"] = WeightSpec((2 * s.inner, s.hidden))
+                specs[f"expert{e}.down"] = WeightSpec((s.hidden, s.inner))
+            return specs
+
+        def bind(self, weights):
+            self.w = weights
+
+        def libraries(self):
+            return ["gemm", "elementwise"]
+
+        def forward(self, ctx, x):
+            s = self.spec
+            k = ctx.kernels
+            share = torch.softmax(x.float() @ self.w["router"].t(), dim=-1)
+            best = share.argmax(dim=-1)
+            out = torch.zeros_like(x)
+            for e in range(s.experts):
+                rows = (best == e).nonzero().flatten()
+                if rows.numel() == 0:
+                    continue
+                xe = x[rows].contiguous()
+                gate_up = torch.empty((rows.numel(), 2 * s.inner), dtype=x.dtype, device=x.device)
+                k.gemm(xe, self.w[f"expert{e}.gate_up"], gate_up)
+                act = torch.empty((rows.numel(), s.inner), dtype=x.dtype, device=x.device)
+                k.silu_mul(gate_up, act)
+                down = torch.empty((rows.numel(), s.hidden), dtype=x.dtype, device=x.device)
+                k.gemm(act, self.w[f"expert{e}.down"], down)
+                out[rows] = (down.float() * share[rows, e][:, None]).to(x.dtype)
+            return out
 
     class ToyBase:
         def __init__(self, data):
@@ -111,7 +187,24 @@ def register_toys():
                              (LayerRun(0, 0), LayerRun(1, 1), LayerRun(0, 2), LayerRun(1, 1, write_cache=False)),
                              norm, False, 512)
 
-    return ToyState, ToyOrder
+    @register_architecture("ToyRoutedForTests")
+    class ToyRouted(ToyBase):
+        """Two attention layers under the rotation with linear angles; the second one's feed-forward is routed."""
+
+        def model_spec(self):
+            norm = NormSpec("rmsnorm", self.hidden, 1e-5)
+            attn = attention(self.hidden, 2, 1, 16, 1e-5, LinearRotationSpec("toy_rotation_linear", 16, 3))
+            first = LayerSpec("prenorm", norm, attn, norm, MlpSpec("swiglu", self.hidden, self.inter))
+            second = LayerSpec("prenorm", norm, attn, norm, RoutedSpec("toy_routed", self.hidden, 24, 3))
+            return ModelSpec("ToyRoutedForTests", self.vocab, self.hidden, (first, second),
+                             (LayerRun(0, 0), LayerRun(1, 1)), norm, False, 512)
+
+    return ToyState, ToyOrder, ToyRouted
+
+
+def linear_angles(positions, dim, shift):
+    j = np.arange(dim // 2, dtype=np.float64)
+    return (np.asarray(positions, dtype=np.float64)[:, None] + shift) / (1.0 + j)[None, :]
 
 
 _registered = []
@@ -207,4 +300,76 @@ def test_toy_architectures_step_like_their_plain_twins(tmp_path, arch, plain, dt
     steps, peak = mixed(reqs, seed=2)
     r = Runner(model, max_tokens=peak, max_slots=4, page_size=8)
     compare(run_steps(r, steps), want, name)
+    r.cache.check()
+
+
+def plain_toy_routed(w, tokens, margins=None, chosen=None):
+    """Logits of every position; `margins` (a list) receives each token's gap between the two largest
+    router logits, `chosen` (a set) the experts that were picked."""
+    pos = np.arange(len(tokens))
+    cfg = dict(ATTN_CFG, num_key_value_heads=1)
+    angle = linear_angles(pos, 16, 3)
+    h = P.embed(tokens, w["tok.weight"])
+    for i in range(2):
+        lw = {k: w[f"layer{i}.mixer.{k}"] for k in ("q_proj", "k_proj", "v_proj", "o_proj")}
+        x = P.rms_norm(h, w[f"layer{i}.norm1.weight"], 1e-5)
+        T = len(tokens)
+        q = P.rms_norm((x @ lw["q_proj"].T).reshape(T, 2, 16), w[f"layer{i}.mixer.q_norm.weight"], 1e-5)
+        k = P.rms_norm((x @ lw["k_proj"].T).reshape(T, 1, 16), w[f"layer{i}.mixer.k_norm.weight"], 1e-5)
+        v = (x @ lw["v_proj"].T).reshape(T, 1, 16)
+        q, k = P.rope_rotate(q, np.cos(angle), np.sin(angle)), P.rope_rotate(k, np.cos(angle), np.sin(angle))
+        h = h + P.causal_attention(q, k, v, pos, 0.25).reshape(T, -1) @ lw["o_proj"].T
+        x = P.rms_norm(h, w[f"layer{i}.norm2.weight"], 1e-5)
+        if i == 0:
+            h = h + P.swiglu_mlp(x, {k: w[f"layer0.ffn.{k}"] for k in ("gate_proj", "up_proj", "down_proj")})
+            continue
+        logits = x @ w["layer1.ffn.router"].T
+        share = np.exp(logits - logits.max(axis=-1, keepdims=True))
+        share /= share.sum(axis=-1, keepdims=True)
+        best = logits.argmax(axis=-1)
+        if margins is not None:
+            top = np.sort(logits, axis=-1)
+            margins.extend((top[:, -1] - top[:, -2]).tolist())
+        if chosen is not None:
+            chosen.update(int(e) for e in best)
+        out = np.zeros_like(h)
+        for t in range(T):
+            e = best[t]
+            gu = x[t] @ w[f"layer1.ffn.expert{e}.gate_up"].T
+            g, u = gu[:24], gu[24:]
+            out[t] = share[t, e] * (((g / (1.0 + np.exp(-g))) * u) @ w[f"layer1.ffn.expert{e}.down"].T)
+        h = h + out
+    return P.output_logits(h, w["out_norm.weight"], w["out.weight"], 1e-5)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_routed_feed_forward_and_another_rotation(tmp_path, dtype):
+    """The routed layer is the last one, so a token whose two best experts are nearly tied (and may be
+    routed otherwise in bfloat16) can only change its own logits: such positions are left out."""
+    from helpers import compare, make_requests, mixed, portions, run_steps, whole
+    from mini_llm_runtime_amd.engine import Runner
+    from mini_llm_runtime_amd.parts import DecoderModel
+    folder = write_folder(tmp_path, "ToyRoutedForTests", seed=6)
+    model = DecoderModel.load(folder, dtype)
+    assert not model.graph_safe()
+    w = plain_weights(folder)
+    reqs = make_requests(97, [50, 23, 70, 9, 31], seed=12)
+    want, chosen = {}, set()
+    for rid, toks in reqs.items():
+        margins = []
+        rows = plain_toy_routed(w, toks, margins, chosen)
+        for p, row in enumerate(rows):
+            if margins[p] > (1e-4 if dtype == torch.float32 else 0.08):
+                want[(rid, p)] = row
+    assert len(want) > 120 and chosen == {0, 1, 2}       # most positions are compared; every expert is chosen by some token
+    name = "float32" if dtype == torch.float32 else "bfloat16"
+
+    def check(got):
+        compare({k: v for k, v in got.items() if k in want}, want, name)
+    r = Runner(model, max_tokens=128, max_slots=4, page_size=8)
+    check(run_steps(r, whole(reqs)))
+    check(run_steps(r, portions(reqs)))
+    steps, peak = mixed(reqs, seed=3)
+    r = Runner(model, max_tokens=peak, max_slots=4, page_size=8)
+    check(run_steps(r, steps))
     r.cache.check()
