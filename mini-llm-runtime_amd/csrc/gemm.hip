@@ -208,7 +208,11 @@ __global__ __launch_bounds__(SKINNY_WAVES * 64) void gemm_skinny_kernel(const __
         const __bf16* xrow[MT];
 #pragma unroll
         for (int i = 0; i < MT; ++i) xrow[i] = a + (size_t)min(16 * i + r16, M - 1) * K + b * (8 * W);
-        constexpr int U = (MT * NW <= 2) ? 8 : 4;         // groups whose weight loads are in flight per lane
+        // groups taken per turn of the loop.  (The compiler keeps the loads of about two of them in flight,
+        // because of the early exit below; asking for all of them up front, without the exit, measured no
+        // faster for large K and slower for small K, where a wavefront has fewer groups than a turn takes.
+        // The many wavefronts of a compute unit hide the latency between them.)
+        constexpr int U = (MT * NW <= 2) ? 8 : 4;
         for (int g0 = g_begin; g0 < g_end; g0 += U) {
             bf16x8 wf[NW][U][W];
 #pragma unroll
