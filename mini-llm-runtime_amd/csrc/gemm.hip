@@ -6,6 +6,7 @@
 // Bfloat16 engine: MFMA (v_mfma_f32_16x16x32_bf16) tiles staged through LDS; the k order of
 // every output element is fixed as well (no split over k).
 #include "common.h"
+#include <type_traits>
 
 #if !MLR_BF16
 // ------------------------------------------------------------------------------ float
@@ -208,38 +209,40 @@ __global__ __launch_bounds__(SKINNY_WAVES * 64) void gemm_skinny_kernel(const __
         const __bf16* xrow[MT];
 #pragma unroll
         for (int i = 0; i < MT; ++i) xrow[i] = a + (size_t)min(16 * i + r16, M - 1) * K + b * (8 * W);
-        // groups taken per turn of the loop.  (The compiler keeps the loads of about two of them in flight,
-        // because of the early exit below; asking for all of them up front, without the exit, measured no
-        // faster for large K and slower for small K, where a wavefront has fewer groups than a turn takes.
-        // The many wavefronts of a compute unit hide the latency between them.)
-        constexpr int U = (MT * NW <= 2) ? 8 : 4;
-        for (int g0 = g_begin; g0 < g_end; g0 += U) {
-            bf16x8 wf[NW][U][W];
+        // Full turns of U groups first: every load of a turn (the activation, which comes from the cache,
+        // before the weight that follows it in the queue) is asked for before the first product, with no
+        // branch in between.  What is left (fewer than U groups) goes one group at a time.
+        constexpr int U = (MT * NW <= 2) ? 4 : 2;
+        auto turn = [&](int g0, auto count) {
+            constexpr int C = decltype(count)::value;
+            bf16x8 xf[MT][C][W], wf[NW][C][W];
 #pragma unroll
-            for (int u = 0; u < U; ++u) {
-                const int k = min(g0 + u, g_end - 1) * (32 * W);
+            for (int u = 0; u < C; ++u)
+#pragma unroll
+                for (int i = 0; i < MT; ++i)
+#pragma unroll
+                    for (int c = 0; c < W; ++c)
+                        xf[i][u][c] = *reinterpret_cast<const bf16x8*>(xrow[i] + (g0 + u) * (32 * W) + 8 * c);
+#pragma unroll
+            for (int u = 0; u < C; ++u)
 #pragma unroll
                 for (int g = 0; g < NW; ++g)
 #pragma unroll
                     for (int c = 0; c < W; ++c)
-                        wf[g][u][c] = *reinterpret_cast<const bf16x8*>(wrow + (size_t)g * N * K + k + 8 * c);
-            }
+                        wf[g][u][c] = *reinterpret_cast<const bf16x8*>(wrow + (size_t)g * N * K + (g0 + u) * (32 * W) + 8 * c);
 #pragma unroll
-            for (int u = 0; u < U; ++u) {
-                if (g0 + u >= g_end) break;
-                const int k = (g0 + u) * (32 * W);
+            for (int u = 0; u < C; ++u)
 #pragma unroll
-                for (int i = 0; i < MT; ++i) {
+                for (int i = 0; i < MT; ++i)
 #pragma unroll
-                    for (int c = 0; c < W; ++c) {
-                        const bf16x8 xf = *reinterpret_cast<const bf16x8*>(xrow[i] + k + 8 * c);
+                    for (int c = 0; c < W; ++c)
 #pragma unroll
                         for (int g = 0; g < NW; ++g)
-                            acc[g][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[g][u][c], xf, acc[g][i], 0, 0, 0);
-                    }
-                }
-            }
-        }
+                            acc[g][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[g][u][c], xf[i][u][c], acc[g][i], 0, 0, 0);
+        };
+        int g0 = g_begin;
+        for (; g0 + U <= g_end; g0 += U) turn(g0, std::integral_constant<int, U>{});
+        for (; g0 < g_end; ++g0) turn(g0, std::integral_constant<int, 1>{});
     } else {
 #pragma unroll 4
         for (int s = s_begin; s < s_end; ++s) {
