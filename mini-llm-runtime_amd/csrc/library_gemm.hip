@@ -38,15 +38,20 @@ int make_plan(int M, int N, int K, size_t workspace_bytes, Plan& p) {
     if (hipblasLtMatmulPreferenceCreate(&pref) != HIPBLAS_STATUS_SUCCESS) return -13;
     const uint64_t ws = workspace_bytes;
     hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &ws, sizeof(ws));
-    hipblasLtMatmulHeuristicResult_t result;
+    // the library's candidates in the order of its own estimate; the first whose scratch memory fits
+    constexpr int CANDIDATES = 8;
+    hipblasLtMatmulHeuristicResult_t results[CANDIDATES];
     int found = 0;
     const hipblasStatus_t st =
-        hipblasLtMatmulAlgoGetHeuristic(g_handle, p.desc, p.a, p.b, p.c, p.c, pref, 1, &result, &found);
+        hipblasLtMatmulAlgoGetHeuristic(g_handle, p.desc, p.a, p.b, p.c, p.c, pref, CANDIDATES, results, &found);
     hipblasLtMatmulPreferenceDestroy(pref);
     if (st != HIPBLAS_STATUS_SUCCESS || found < 1) return -14;
-    if (result.workspaceSize > workspace_bytes) return -15;
-    p.algo = result.algo;
-    p.workspace = result.workspaceSize;
+    int pick = -1;
+    for (int i = 0; i < found && pick < 0; ++i)
+        if (results[i].state == HIPBLAS_STATUS_SUCCESS && results[i].workspaceSize <= workspace_bytes) pick = i;
+    if (pick < 0) return -15;
+    p.algo = results[pick].algo;
+    p.workspace = results[pick].workspaceSize;
     return 0;
 }
 }  // namespace

@@ -22,7 +22,7 @@ _ptr = ctypes.c_void_p
 MAX_HEAD_DIM = 256          # the attention and rotation kernels keep head_dim / 64 values per lane
 ATTENTION_TILE_KEYS = 64
 LIBRARY_GEMM_MIN_ROWS = 16    # above this many rows the bfloat16 engine's projections go to the library
-LIBRARY_GEMM_WORKSPACE = 32 << 20    # bytes of scratch memory that the library may use
+LIBRARY_GEMM_WORKSPACE = 128 << 20   # bytes of scratch memory that the library may use
 PREFILL_MAX_PAGES = 2048      # page ids of one group that the prompt-portion attention kernel keeps in LDS
 TILES_MAX_HEAD_DIM = 128      # the 32x32-tile kernel for prompt portions keeps two sets of accumulators per lane
 TILES_COLUMNS = (128, 64)     # (token, head) columns of one of its workgroups: the usual and the small one
