@@ -303,9 +303,24 @@ struct KvTile {
 
 #define DECODE_PAGE_CACHE 4096
 
-template <int NCH>   // ceil(head_dim / 32)
+// Decoding (every group is one new token of a request) without a kernel of its own for the per-head norm,
+// the rotation and the cache write: the attention kernel takes the raw projection, norms and rotates its
+// queries itself and walks the keys that are cached already (positions below the token's own); the merge
+// kernel, which follows anyway, norms and rotates the token's own key, adds the token's own score and
+// value as one more summand, and writes key and value into their pages for the steps to come.
+// Needs head_dim % 64 == 0 (a lane of the attention kernel then holds both channels of a rotation pair).
+struct DecodeFusion {
+    const __bf16* qkv;          // [M, ld]: q heads, k heads, v heads of every row
+    const float* q_norm_w;      // [head_dim] or null
+    const float* k_norm_w;
+    const float* rope;          // [positions, head_dim]: cosines | sines, or null
+    int ld;
+    float eps;
+};
+
+template <int NCH, bool FUSED>   // NCH: ceil(head_dim / 32)
 __global__ __launch_bounds__(256, (NCH <= 4 ? 2 : 1)) void attention_mfma_kernel(AttnArgs a, const int32_t* __restrict__ group_row0,
-                                                             const int32_t* __restrict__ group_ntok) {
+                                                             const int32_t* __restrict__ group_ntok, DecodeFusion f) {
     extern __shared__ float lds[];
     __shared__ int32_t page_lds[DECODE_PAGE_CACHE];    // the request's page ids for this workgroup's key range
     const int D = a.head_dim, P = a.page_size;
@@ -317,18 +332,20 @@ __global__ __launch_bounds__(256, (NCH <= 4 ? 2 : 1)) void attention_mfma_kernel
     const int slot = a.slots[row0], pos0 = a.positions[row0];
     const int tok = col / g, hh = col % g;
     const bool col_valid = tok < ntok;
-    const int kend_c = col_valid ? pos0 + tok + 1 : 0;
-    int kbegin_c = a.window > 0 ? max(0, kend_c - a.window) : 0;
+    const int kend_full = col_valid ? pos0 + tok + 1 : 0;
+    int kbegin_c = a.window > 0 ? max(0, kend_full - a.window) : 0;
+    const int kend_c = FUSED ? max(kend_full - 1, 0) : kend_full;     // FUSED: the token's own key is not cached yet
     const int glo = a.window > 0 ? max(0, pos0 + 1 - a.window) : 0;   // the group's key range [glo, ke)
-    const int ke = pos0 + ntok;                                         // keys below ke are written
+    const int ke = pos0 + ntok - (FUSED ? 1 : 0);                      // keys below ke are written
     int lo = glo, hi = ke;
     if (a.max_splits > 1) {
         const int first_split = glo / a.split_keys;
-        const int last_split = min(a.max_splits - 1, (ke - 1) / a.split_keys);
+        const int last_split = min(a.max_splits - 1, max(ke - 1, 0) / a.split_keys);
         if (split < first_split || split > last_split) return;          // no keys here: the whole workgroup leaves
         lo = max(lo, split * a.split_keys);
         hi = min(hi, (split + 1) * a.split_keys);
     }
+    hi = max(hi, lo);                                                   // (FUSED, first token: no key at all)
     kbegin_c = max(kbegin_c, lo);
     const int kstop_c = min(kend_c, hi);
 
@@ -346,15 +363,81 @@ __global__ __launch_bounds__(256, (NCH <= 4 ? 2 : 1)) void attention_mfma_kernel
         for (int i = threadIdx.x; i < n_pages; i += 256) page_lds[i] = table[first_page + i];
     }
 
+    // The queries.  FUSED: the raw query of this lane's column, its norm weights and its rotation row are
+    // asked for here; the arithmetic waits until the first key tile has been asked for as well (below).
     bf16x8 qf[NCH];
+    constexpr int HC = NCH / 2;
+    bf16x8 q_raw[FUSED ? NCH : 1];
+    float4 q_w[FUSED ? 2 * NCH : 1], q_cs[FUSED ? 2 * NCH : 1];
+    if (FUSED) {
+        const __bf16* src = f.qkv + (size_t)(row0 + (col_valid ? tok : 0)) * f.ld + (size_t)(kvh * g + (col_valid ? hh : 0)) * D + 8 * b;
+        const float* wq = (f.q_norm_w ? f.q_norm_w : reinterpret_cast<const float*>(f.qkv)) + 8 * b;     // (any readable address)
+        const float* cs = (f.rope ? f.rope + (size_t)(pos0 + (col_valid ? tok : 0)) * D : reinterpret_cast<const float*>(f.qkv)) + 8 * b;
 #pragma unroll
-    for (int c = 0; c < NCH; ++c) {
-        const int d0 = 32 * c + 8 * b;
-        qf[c] = zero8;
-        if (col_valid && d0 < D)
-            qf[c] = *reinterpret_cast<const bf16x8*>(q + ((size_t)(row0 + tok) * a.q_heads + kvh * g + hh) * D + d0);
+        for (int c = 0; c < NCH; ++c) {
+            q_raw[c] = *reinterpret_cast<const bf16x8*>(src + 32 * c);
+            q_w[2 * c] = *reinterpret_cast<const float4*>(wq + 32 * c);
+            q_w[2 * c + 1] = *reinterpret_cast<const float4*>(wq + 32 * c + 4);
+            // cosines of the pairs 32 c + 8 b .. for c < HC, their sines for c >= HC (the table holds cosines | sines)
+            q_cs[2 * c] = *reinterpret_cast<const float4*>(cs + 32 * c);
+            q_cs[2 * c + 1] = *reinterpret_cast<const float4*>(cs + 32 * c + 4);
+        }
+    } else {
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) {
+            const int d0 = 32 * c + 8 * b;
+            qf[c] = zero8;
+            if (col_valid && d0 < D)
+                qf[c] = *reinterpret_cast<const bf16x8*>(q + ((size_t)(row0 + tok) * a.q_heads + kvh * g + hh) * D + d0);
+        }
     }
     __syncthreads();
+    auto finish_queries = [&]() {
+        // per-head norm, rotation (a lane holds channels 32 c + 8 b .. of every chunk c, so with head_dim =
+        // 32 NCH, NCH even, the partner d + head_dim / 2 of a channel is in chunk c + NCH / 2 of the same
+        // lane), rounded to bfloat16 as the cache's keys are
+        float x[NCH][8];
+        float sq = 0.f;
+#pragma unroll
+        for (int c = 0; c < NCH; ++c)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                x[c][e] = (float)q_raw[c][e];
+                sq += x[c][e] * x[c][e];
+            }
+        sq += __shfl_xor(sq, 16, MLR_WAVE);
+        sq += __shfl_xor(sq, 32, MLR_WAVE);
+        if (f.q_norm_w) {
+            const float scale = 1.0f / sqrtf(sq / (float)D + f.eps);
+#pragma unroll
+            for (int c = 0; c < NCH; ++c) {
+                const float w8[8] = {q_w[2 * c].x, q_w[2 * c].y, q_w[2 * c].z, q_w[2 * c].w,
+                                     q_w[2 * c + 1].x, q_w[2 * c + 1].y, q_w[2 * c + 1].z, q_w[2 * c + 1].w};
+#pragma unroll
+                for (int e = 0; e < 8; ++e) x[c][e] = (x[c][e] * scale) * w8[e];
+            }
+        }
+        if (f.rope) {
+#pragma unroll
+            for (int c = 0; c < HC; ++c) {
+                const float co[8] = {q_cs[2 * c].x, q_cs[2 * c].y, q_cs[2 * c].z, q_cs[2 * c].w,
+                                     q_cs[2 * c + 1].x, q_cs[2 * c + 1].y, q_cs[2 * c + 1].z, q_cs[2 * c + 1].w};
+                const float si[8] = {q_cs[2 * (c + HC)].x, q_cs[2 * (c + HC)].y, q_cs[2 * (c + HC)].z, q_cs[2 * (c + HC)].w,
+                                     q_cs[2 * (c + HC) + 1].x, q_cs[2 * (c + HC) + 1].y, q_cs[2 * (c + HC) + 1].z,
+                                     q_cs[2 * (c + HC) + 1].w};
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float lo_v = x[c][e], hi_v = x[c + HC][e];
+                    x[c][e] = lo_v * co[e] - hi_v * si[e];
+                    x[c + HC][e] = lo_v * si[e] + hi_v * co[e];
+                }
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < NCH; ++c)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) qf[c][e] = col_valid ? (__bf16)x[c][e] : (__bf16)0.f;
+    };
 
     // Scores are kept in the base-2 domain: s * (scale * log2 e), so that a probability is one v_exp_f32.
     const float c2 = a.scale * 1.44269504088896340736f;
@@ -465,9 +548,10 @@ __global__ __launch_bounds__(256, (NCH <= 4 ? 2 : 1)) void attention_mfma_kernel
         // (clamped to the wavefront's last tile) for the reason given above
         KvTile<NCH> ta, tb2;
         int t = t_begin + wave;
+        const int t_last = t + ((t_end - 1 - t) / 4) * 4;
+        if (t < t_end) load(t, ta);
+        if (FUSED) finish_queries();
         if (t < t_end) {
-            const int t_last = t + ((t_end - 1 - t) / 4) * 4;
-            load(t, ta);
             for (;;) {
                 load(min(t + 4, t_last), tb2);
                 compute(ta);
@@ -525,7 +609,7 @@ __global__ __launch_bounds__(256, (NCH <= 4 ? 2 : 1)) void attention_mfma_kernel
             }
         }
         if (col_valid) {
-            if (a.max_splits > 1) {
+            if (a.max_splits > 1 || FUSED) {                   // (FUSED: the merge kernel always follows)
                 float* dst = a.partial + (out_row * a.max_splits + split) * (D + 2);
 #pragma unroll
                 for (int db = 0; db < 2 * NCH; ++db) {
@@ -866,6 +950,194 @@ __global__ __launch_bounds__(64) void attention_combine_groups_kernel(AttnArgs a
     }
 }
 
+// The merge for `DecodeFusion`: one wavefront per (token, head).  Besides the splits' partial results it adds
+// the token's own key and value (see `DecodeFusion`), and the first head of every kv head writes them
+// into the cache.  A lane takes the rotation pairs lane and lane + 64 and the channels lane + 64 i.
+__global__ __launch_bounds__(64) void attention_combine_fused_kernel(AttnArgs a, DecodeFusion f) {
+    // (group i is batch row i here.)  Loads are asked for as early as their addresses are known: the row's
+    // position and slot, its raw q, k, v and the norm weights at once; then what needs the position (the
+    // rotation row, the page id, the splits' maxima and sums); then the splits' values, eight at a time.
+    __shared__ float w_lds[COMBINE_MAX_SPLITS];
+    const int m = blockIdx.x, head = blockIdx.y;
+    const int D = a.head_dim, P = a.page_size, half = D >> 1;
+    const int g = a.q_heads / a.kv_heads, kvh = head / g;
+    const int lane = threadIdx.x;
+    const int pos = a.positions[m], slot = a.slots[m];
+    const __bf16* row = f.qkv + (size_t)m * f.ld;
+    const __bf16* qs = row + (size_t)head * D;
+    const __bf16* ks = row + (size_t)(a.q_heads + kvh) * D;
+    const __bf16* vs = row + (size_t)(a.q_heads + a.kv_heads + kvh) * D;
+    const bool normed = f.q_norm_w != nullptr, rotated = f.rope != nullptr;
+    const float* qw = normed ? f.q_norm_w : reinterpret_cast<const float*>(row);      // (any readable address)
+    const float* kw = normed ? f.k_norm_w : reinterpret_cast<const float*>(row);
+    float qa[2], qb[2], ka[2], kb[2], qwa[2], qwb[2], kwa[2], kwb[2], vv[MAX_DIM_REGS];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int j = min(lane + 64 * i, half - 1);
+        qa[i] = (float)qs[j];
+        qb[i] = (float)qs[j + half];
+        ka[i] = (float)ks[j];
+        kb[i] = (float)ks[j + half];
+        qwa[i] = qw[j];
+        qwb[i] = qw[j + half];
+        kwa[i] = kw[j];
+        kwb[i] = kw[j + half];
+    }
+#pragma unroll
+    for (int i = 0; i < MAX_DIM_REGS; ++i) vv[i] = (float)vs[min(lane + 64 * i, D - 1)];
+    // second round: everything that needs the position
+    const float* cs = (rotated ? f.rope : reinterpret_cast<const float*>(a.positions)) + (rotated ? (size_t)pos * D : 0);
+    float co[2], si[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int j = rotated ? min(lane + 64 * i, half - 1) : 0;
+        co[i] = cs[j];
+        si[i] = cs[rotated ? j + half : 0];
+    }
+    const int page = a.block_table[(size_t)slot * a.max_blocks + pos / P];
+    const int glo = a.window > 0 ? max(0, pos + 1 - a.window) : 0;
+    const int first = a.max_splits > 1 ? glo / a.split_keys : 0;
+    const int last = a.max_splits > 1 ? min(a.max_splits - 1, max(pos - 1, 0) / a.split_keys) : 0;
+    const int n = last - first + 1;                     // the same range of splits that the attention kernel served
+    const float* base = a.partial + (((size_t)m * a.q_heads + head) * a.max_splits + first) * (D + 2);
+    float smax[COMBINE_MAX_SPLITS / 64], ssum[COMBINE_MAX_SPLITS / 64];
+    float gmax = -INFINITY;
+#pragma unroll
+    for (int r = 0; r < COMBINE_MAX_SPLITS / 64; ++r) {
+        const int s = lane + 64 * r;
+        if (64 * r >= n) break;
+        const float* p = base + (size_t)min(s, n - 1) * (D + 2);
+        smax[r] = s < n ? p[D] : -INFINITY;
+        ssum[r] = p[D + 1];
+        gmax = fmaxf(gmax, smax[r]);
+    }
+
+    // query and key of this token: norm, rotation, rounded to bfloat16 (what the cache holds)
+    float qsum = 0.f, ksum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        if (lane + 64 * i >= half) qa[i] = qb[i] = ka[i] = kb[i] = 0.f;
+        qsum += qa[i] * qa[i] + qb[i] * qb[i];
+        ksum += ka[i] * ka[i] + kb[i] * kb[i];
+    }
+    if (normed) {
+        qsum = wave_sum(qsum);
+        ksum = wave_sum(ksum);
+        const float qscale = 1.0f / sqrtf(qsum / (float)D + f.eps), kscale = 1.0f / sqrtf(ksum / (float)D + f.eps);
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            qa[i] = (qa[i] * qscale) * qwa[i];
+            qb[i] = (qb[i] * qscale) * qwb[i];
+            ka[i] = (ka[i] * kscale) * kwa[i];
+            kb[i] = (kb[i] * kscale) * kwb[i];
+        }
+    }
+    float dot = 0.f;
+    __bf16 k_lo[2], k_hi[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        float qx = qa[i], qy = qb[i], kx = ka[i], ky = kb[i];
+        if (rotated) {
+            qx = qa[i] * co[i] - qb[i] * si[i];
+            qy = qa[i] * si[i] + qb[i] * co[i];
+            kx = ka[i] * co[i] - kb[i] * si[i];
+            ky = ka[i] * si[i] + kb[i] * co[i];
+        }
+        k_lo[i] = (__bf16)kx;
+        k_hi[i] = (__bf16)ky;
+        if (lane + 64 * i < half)
+            dot += (float)(__bf16)qx * (float)k_lo[i] + (float)(__bf16)qy * (float)k_hi[i];
+    }
+    const float s_own = wave_sum(dot) * (a.scale * 1.44269504088896340736f);     // base-2 domain, as the partial maxima
+    gmax = fmaxf(wave_max(gmax), s_own);
+    // the splits' weights (maxima are base-2 exponents) and the denominator, summed in ascending order
+#pragma unroll
+    for (int r = 0; r < COMBINE_MAX_SPLITS / 64; ++r) {
+        const int s = lane + 64 * r;
+        if (64 * r >= n) break;
+        if (s < n) w_lds[s] = smax[r] > -INFINITY ? __builtin_amdgcn_exp2f(smax[r] - gmax) * 1.0f : 0.f;
+    }
+    __syncthreads();
+    float den = 0.f;
+#pragma unroll
+    for (int r = 0; r < COMBINE_MAX_SPLITS / 64; ++r) {
+        const int s = lane + 64 * r;
+        if (64 * r >= n) break;
+        den += s < n ? w_lds[s] * ssum[r] : 0.f;
+    }
+    den = wave_sum(den);
+    float num[MAX_DIM_REGS];
+#pragma unroll
+    for (int i = 0; i < MAX_DIM_REGS; ++i) num[i] = 0.f;
+#pragma unroll 8
+    for (int s = 0; s < n; ++s) {
+        const float w = w_lds[s];
+        const float* p = base + (size_t)s * (D + 2);
+#pragma unroll
+        for (int i = 0; i < MAX_DIM_REGS; ++i) num[i] += w * p[min(lane + 64 * i, D - 1)];     // clamped: no branch around the load
+    }
+    const float w_own = __builtin_amdgcn_exp2f(s_own - gmax);
+    den += w_own;
+#pragma unroll
+    for (int i = 0; i < MAX_DIM_REGS; ++i) {
+        const int d = lane + 64 * i;
+        if (d < D) a.out[((size_t)m * a.q_heads + head) * D + d] = from_float<elem_t>((num[i] + w_own * vv[i]) / den);
+    }
+    // key and value into their pages, once per kv head
+    if (head != kvh * g || page < 0) return;
+    const size_t pk = (size_t)page * a.kv_heads + kvh;
+    __bf16* kdst = reinterpret_cast<__bf16*>(const_cast<elem_t*>(a.k_pages)) + (pk * P + pos % P) * D;
+    __bf16* vdst = reinterpret_cast<__bf16*>(const_cast<elem_t*>(a.v_pages)) + pk * D * P + pos % P;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int j = lane + 64 * i;
+        if (j < half) {
+            kdst[j] = k_lo[i];
+            kdst[j + half] = k_hi[i];
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < MAX_DIM_REGS; ++i) {
+        const int d = lane + 64 * i;
+        if (d < D) vdst[(size_t)d * P] = (__bf16)vv[i];
+    }
+}
+
+// Decoding with `DecodeFusion`: group i is the one token in batch row i (group_row0[i] = i, group_ntok[i] = 1);
+// qkv holds the raw projections
+// [rows, ld].  Key and value of every token are written into the cache.  `partial` holds at least
+// rows * q_heads * max(max_splits, 1) * (head_dim + 2) floats, also without splits.
+// Needs what `mlr_attention_mfma` needs and head_dim % 64 == 0.
+extern "C" int mlr_attention_decode_fused(
+    const void* qkv, int ld, const void* k_pages, const void* v_pages, const int32_t* block_table, int max_blocks,
+    const int32_t* slots, const int32_t* positions, void* out, float* partial, const int32_t* group_row0,
+    const int32_t* group_ntok, int groups, int q_heads, int kv_heads, int head_dim, int page_size, int window,
+    float scale, int split_keys, int max_splits, const float* q_norm_w, const float* k_norm_w, float eps,
+    const float* rope, hipStream_t stream) {
+    if (groups <= 0) return 0;
+    if (head_dim % 64 != 0 || head_dim > 256 || page_size % 16 != 0 || q_heads % kv_heads != 0 ||
+        q_heads / kv_heads > 16 || partial == nullptr || (q_norm_w == nullptr) != (k_norm_w == nullptr)) return -1;
+    if (max_splits < 1) max_splits = 1;
+    if (max_splits > 1 && (split_keys <= 0 || split_keys % MFMA_TILE_KEYS != 0 || max_splits > COMBINE_MAX_SPLITS)) return -2;
+    if ((max_splits > 1 ? split_keys / page_size + 2 : max_blocks) > DECODE_PAGE_CACHE) return -3;
+    AttnArgs a{nullptr, (const elem_t*)k_pages, (const elem_t*)v_pages, block_table, slots,
+               positions, (elem_t*)out, partial, max_blocks, q_heads, kv_heads, head_dim, page_size,
+               window, split_keys, max_splits, scale};
+    DecodeFusion f{(const __bf16*)qkv, q_norm_w, k_norm_w, rope, ld, eps};
+    dim3 grid(groups, kv_heads, max_splits);
+    const size_t lds = sizeof(float) * 3 * (16 * (size_t)head_dim + 32);
+    switch (head_dim / 32) {
+        case 2: attention_mfma_kernel<2, true><<<grid, 256, lds, stream>>>(a, group_row0, group_ntok, f); break;
+        case 4: attention_mfma_kernel<4, true><<<grid, 256, lds, stream>>>(a, group_row0, group_ntok, f); break;
+        case 6: attention_mfma_kernel<6, true><<<grid, 256, lds, stream>>>(a, group_row0, group_ntok, f); break;
+        default: attention_mfma_kernel<8, true><<<grid, 256, lds, stream>>>(a, group_row0, group_ntok, f); break;
+    }
+    int err = (int)hipGetLastError();
+    if (err != 0) return err;
+    attention_combine_fused_kernel<<<dim3(groups, q_heads), 64, 0, stream>>>(a, f);
+    return (int)hipGetLastError();
+}
+
 // Groups: group_row0[i] = first batch row of group i, group_ntok[i] = its tokens (consecutive rows of one
 // request, ntok * (q_heads / kv_heads) <= 16).  Rows outside the groups are left alone.
 // Needs page_size % 16 == 0, head_dim % 16 == 0, q_heads / kv_heads <= 16.
@@ -889,14 +1161,14 @@ extern "C" int mlr_attention_mfma(
     const size_t lds = sizeof(float) * 3 * (16 * (size_t)head_dim + 32);
     const int nch = (head_dim + 31) / 32;
     switch (nch) {
-        case 1: attention_mfma_kernel<1><<<grid, 256, lds, stream>>>(a, group_row0, group_ntok); break;
-        case 2: attention_mfma_kernel<2><<<grid, 256, lds, stream>>>(a, group_row0, group_ntok); break;
-        case 3: attention_mfma_kernel<3><<<grid, 256, lds, stream>>>(a, group_row0, group_ntok); break;
-        case 4: attention_mfma_kernel<4><<<grid, 256, lds, stream>>>(a, group_row0, group_ntok); break;
-        case 5: attention_mfma_kernel<5><<<grid, 256, lds, stream>>>(a, group_row0, group_ntok); break;
-        case 6: attention_mfma_kernel<6><<<grid, 256, lds, stream>>>(a, group_row0, group_ntok); break;
-        case 7: attention_mfma_kernel<7><<<grid, 256, lds, stream>>>(a, group_row0, group_ntok); break;
-        default: attention_mfma_kernel<8><<<grid, 256, lds, stream>>>(a, group_row0, group_ntok); break;
+        case 1: attention_mfma_kernel<1, false><<<grid, 256, lds, stream>>>(a, group_row0, group_ntok, DecodeFusion{}); break;
+        case 2: attention_mfma_kernel<2, false><<<grid, 256, lds, stream>>>(a, group_row0, group_ntok, DecodeFusion{}); break;
+        case 3: attention_mfma_kernel<3, false><<<grid, 256, lds, stream>>>(a, group_row0, group_ntok, DecodeFusion{}); break;
+        case 4: attention_mfma_kernel<4, false><<<grid, 256, lds, stream>>>(a, group_row0, group_ntok, DecodeFusion{}); break;
+        case 5: attention_mfma_kernel<5, false><<<grid, 256, lds, stream>>>(a, group_row0, group_ntok, DecodeFusion{}); break;
+        case 6: attention_mfma_kernel<6, false><<<grid, 256, lds, stream>>>(a, group_row0, group_ntok, DecodeFusion{}); break;
+        case 7: attention_mfma_kernel<7, false><<<grid, 256, lds, stream>>>(a, group_row0, group_ntok, DecodeFusion{}); break;
+        default: attention_mfma_kernel<8, false><<<grid, 256, lds, stream>>>(a, group_row0, group_ntok, DecodeFusion{}); break;
     }
     int err = (int)hipGetLastError();
     if (err != 0) return err;

@@ -148,6 +148,7 @@ class Runner:
         ctx.n_tokens = total
         ctx.token_ids, ctx.positions, ctx.slots = meta[0:total], meta[total:2 * total], meta[2 * total:3 * total]
         ctx.segments = segments
+        ctx.single_tokens = total == len(entries)
         r = state["rows"]
         want_rows = meta[3 * total:3 * total + r] if r else None
         if state["eager"]:                                # a shape whose capture did not hold
@@ -233,6 +234,7 @@ class Runner:
             ctx.positions = self._meta[total:2 * total]
             ctx.slots = self._meta[2 * total:3 * total]
             ctx.segments = segments
+            ctx.single_tokens = total == len(entries)
             ctx.max_context = max(p0 + n for (_, _, n, p0) in segments)
             want_rows = self._meta[3 * total:3 * total + r] if r else None
             logits = self.model.forward(ctx, want_rows)

@@ -329,6 +329,55 @@ class Kernels:
                _c_int(q_heads), _c_int(kv_heads), _c_int(head_dim), _c_int(page_size), _c_int(window or 0),
                _c_float(scale), _c_int(split_keys), _c_int(max_splits), _stream()), "attention_mfma")
 
+    def decode_fusion_supported(self, q_heads, kv_heads, head_dim, page_size):
+        """Attention for single new tokens that norms, rotates and caches inside itself: the matrix-core
+        kernel's sizes and head sizes that are multiples of 64."""
+        return self.mfma_attention_supported(q_heads, kv_heads, head_dim, page_size) and head_dim % 64 == 0
+
+    def attention_decode_fused(self, qkv, k_pages, v_pages, block_table, slots, positions, out, group_row0, group_ntok,
+                               groups, q_heads, kv_heads, head_dim, page_size, scale, q_norm_w, k_norm_w, eps, rope,
+                               partial, window=None, split_keys=0, max_splits=1):
+        """For a batch in which every group is ONE new token of a request (the caller vouches for that):
+        per-head RMSNorm of q and k (weights may both be None), rotation by `rope` (may be None), attention
+        over the cached keys and the token's own, and the write of the token's key and value into their
+        pages, in two launches.  `qkv` holds the raw projections; `partial` is needed also without splits."""
+        _need(self.decode_fusion_supported(q_heads, kv_heads, head_dim, page_size),
+              "attention_decode_fused: sizes not supported")
+        width = (q_heads + 2 * kv_heads) * head_dim
+        _tensor(qkv, "qkv", self.dtype, ndim=2)
+        m = qkv.shape[0]
+        _need(qkv.shape[1] == width, lambda: f"qkv: expected width {width}, got {qkv.shape[1]}")
+        _need(groups == m, "attention_decode_fused: one group per row")
+        _tensor(out, "out", self.dtype, (m, q_heads * head_dim))
+        self._check_cache(k_pages, v_pages, kv_heads, head_dim, page_size)
+        _tensor(block_table, "block_table", torch.int32, ndim=2)
+        _tensor(slots, "slots", torch.int32, (m,))
+        _tensor(positions, "positions", torch.int32, (m,))
+        _tensor(group_row0, "group_row0", torch.int32, (groups,))
+        _tensor(group_ntok, "group_ntok", torch.int32, (groups,))
+        _need((q_norm_w is None) == (k_norm_w is None), "q and k norm weights come together")
+        if q_norm_w is not None:
+            _tensor(q_norm_w, "q_norm_w", torch.float32, (head_dim,))
+            _tensor(k_norm_w, "k_norm_w", torch.float32, (head_dim,))
+        if rope is not None:
+            _tensor(rope, "rope", torch.float32, ndim=2)
+            _need(rope.shape[1] == head_dim, "rope: table width must equal head_dim")
+        max_splits = max(1, max_splits)
+        _need(kv_heads <= 65535 and max_splits <= MAX_KEY_SPLITS, "too many kv heads or key splits for the grid")
+        if max_splits > 1:
+            _need(split_keys > 0 and split_keys % ATTENTION_TILE_KEYS == 0,
+                  lambda: f"split_keys must be a multiple of {ATTENTION_TILE_KEYS}")
+        _tensor(partial, "partial", torch.float32, ndim=1)
+        _need(partial.numel() >= self.attention_partial_numel(m, q_heads, head_dim, max_splits), "partial buffer too small")
+        _need((split_keys // page_size + 2 if max_splits > 1 else block_table.shape[1]) <= 4096,
+              "attention_decode_fused: a workgroup's key range spans more than 4096 pages; split the keys")
+        fn = self._lib("attention").mlr_attention_decode_fused
+        _ok(fn(_p(qkv), _c_int(width), _p(k_pages), _p(v_pages), _p(block_table), _c_int(block_table.shape[1]),
+               _p(slots), _p(positions), _p(out), _p(partial), _p(group_row0), _p(group_ntok), _c_int(groups),
+               _c_int(q_heads), _c_int(kv_heads), _c_int(head_dim), _c_int(page_size), _c_int(window or 0),
+               _c_float(scale), _c_int(split_keys), _c_int(max_splits), _p(q_norm_w), _p(k_norm_w), _c_float(eps),
+               _p(rope), _stream()), "attention_decode_fused")
+
     def prefill_attention_supported(self, q_heads, kv_heads, head_dim, page_size, max_context=0):
         """The LDS-staged kernel for prompt portions: as the matrix-core kernel, head sizes up to 192 and
         contexts of at most 2048 pages (it keeps a group's page ids in LDS)."""

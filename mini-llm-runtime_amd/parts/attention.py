@@ -84,8 +84,27 @@ class GqaAttention:
         x = qkv
         m = qkv.shape[0]
         view = ctx.cache.kv_view(cache_id)
-        q = ctx.workspace.get("q", (m, s.q_heads * s.head_dim), x.dtype)
         rope = self.position.rotation_table(ctx.max_positions, x.device) if self.position is not None else None
+        if (ctx.single_tokens and write_cache and x.dtype == torch.bfloat16
+                and k.decode_fusion_supported(s.q_heads, s.kv_heads, s.head_dim, view.page_size)):
+            # decoding: norm, rotation and cache write ride in the attention's two launches
+            attn = ctx.workspace.get("attn", (m, s.q_heads * s.head_dim), x.dtype)
+            groups, _, _ = ctx.token_groups(max(1, 16 // (s.q_heads // s.kv_heads)), 0)
+            split_keys, max_splits, partial = ctx.attention_split(m, m, s.kv_heads, s.q_heads, s.head_dim)
+            if partial is None:
+                partial = ctx.workspace.get("attn_partial", (k.attention_partial_numel(m, s.q_heads, s.head_dim, 1),),
+                                            torch.float32)
+            k.attention_decode_fused(
+                qkv, view.k_pages, view.v_pages, view.block_table, ctx.slots, ctx.positions, attn, groups[0], groups[1],
+                groups[2], s.q_heads, s.kv_heads, s.head_dim, view.page_size, float(s.scale),
+                self.q_norm.weight if self.q_norm is not None else None,
+                self.k_norm.weight if self.k_norm is not None else None,
+                self.q_norm.eps if self.q_norm is not None else 0.0, rope, partial,
+                window=s.window, split_keys=split_keys, max_splits=max_splits)
+            out = ctx.workspace.get("mixer_out", (m, s.hidden), x.dtype)
+            k.gemm(attn, self.o, out)
+            return out
+        q = ctx.workspace.get("q", (m, s.q_heads * s.head_dim), x.dtype)
         k.qk_norm_rope_kv(
             qkv, q, view.k_pages, view.v_pages, view.block_table, ctx.slots, ctx.positions,
             self.q_norm.weight if self.q_norm is not None else None,

@@ -689,3 +689,77 @@ def test_prompt_portion_beyond_the_page_cache_of_a_workgroup():
     for i in (0, 1, 31, 63, 64, 69):
         want = plain_attention(q[i].double(), kk[:L - n + i + 1].double(), vv[:L - n + i + 1].double(), 1 / math.sqrt(d), None)
         torch.testing.assert_close(got[i], want, **tol(dtype))
+
+
+@pytest.mark.parametrize("case", [
+    # (q heads, kv heads, head_dim, page, context lengths of the requests, window, split_keys, norm, rotation)
+    (16, 8, 128, 16, [1, 2, 17, 300, 4096], None, 512, True, True),
+    (4, 4, 64, 16, [1, 33, 64, 65, 130], None, 0, True, True),
+    (8, 2, 64, 32, [5, 100, 257], 40, 64, True, True),
+    (6, 1, 192, 16, [1, 70], None, 0, False, True),
+    (2, 1, 256, 16, [129, 1], 1, 64, True, False),
+    (32, 8, 128, 64, [513, 512, 511], 512, 256, True, True),
+])
+def test_decode_attention_that_norms_rotates_and_caches_itself(case):
+    """Every request brings one new token.  The fused pair of launches against the separate ones (per-head
+    norm + rotation + cache write, then attention): the same output within bfloat16 rounding, the same key and
+    value in the cache bit for bit, nothing else in the cache touched; and against the plain attention."""
+    hq, hkv, d, page, lengths, window, split_keys, with_norm, with_rope = case
+    dtype = torch.bfloat16
+    k = kernels(dtype)
+    gen = torch.Generator().manual_seed(41)
+    n = len(lengths)
+    max_len = max(lengths)
+    max_blocks = (max_len + page - 1) // page
+    n_pages = sum((L + page - 1) // page for L in lengths) + 3
+    perm = torch.randperm(n_pages, generator=gen).tolist()
+    table = torch.full((n, max_blocks), -1, dtype=torch.int32)
+    k_pages = torch.full((n_pages, hkv, page, d), float("nan"), dtype=dtype)
+    v_pages = torch.full((n_pages, hkv, d, page), float("nan"), dtype=dtype)
+    keys, values = [], []
+    for s, L in enumerate(lengths):
+        kk = torch.randn((L - 1, hkv, d), generator=gen).to(dtype)
+        vv = torch.randn((L - 1, hkv, d), generator=gen).to(dtype)
+        keys.append(kk)
+        values.append(vv)
+        for b in range((L + page - 1) // page):
+            pg = perm.pop()
+            table[s, b] = pg
+            cnt = max(0, min(page, L - 1 - b * page))
+            if cnt:
+                k_pages[pg, :, :cnt] = kk[b * page:b * page + cnt].transpose(0, 1)
+                v_pages[pg, :, :, :cnt] = vv[b * page:b * page + cnt].permute(1, 2, 0)
+    qkv = (torch.randn((n, (hq + 2 * hkv) * d), generator=gen) * 1.5).to(dtype).cuda()
+    qw = (1 + 0.2 * torch.randn(d, generator=gen)).cuda() if with_norm else None
+    kw = (1 + 0.2 * torch.randn(d, generator=gen)).cuda() if with_norm else None
+    eps, base, scale = 1e-5, 10000.0, 1 / math.sqrt(d)
+    rope = rope_table(max_len, d, base).cuda() if with_rope else None
+    slots = torch.arange(n, dtype=torch.int32).cuda()
+    pos = torch.tensor([L - 1 for L in lengths], dtype=torch.int32).cuda()
+    first = torch.arange(n, dtype=torch.int32).cuda()
+    ones = torch.ones(n, dtype=torch.int32).cuda()
+    max_splits = (max_len + split_keys - 1) // split_keys if split_keys else 1
+    partial = torch.full((k.attention_partial_numel(n, hq, d, max_splits),), float("nan"), device="cuda")
+    # the separate launches
+    k1, v1 = k_pages.clone().cuda(), v_pages.clone().cuda()
+    q1 = torch.empty((n, hq * d), dtype=dtype, device="cuda")
+    k.qk_norm_rope_kv(qkv, q1, k1, v1, table.cuda(), slots, pos, qw, kw, eps, rope, hq, hkv, d, page)
+    out1 = torch.full((n, hq * d), float("nan"), dtype=dtype, device="cuda")
+    k.attention_mfma(q1, k1, v1, table.cuda(), slots, pos, out1, first, ones, n, hq, hkv, d, page, scale, window=window,
+                     split_keys=split_keys, max_splits=max_splits, partial=partial if max_splits > 1 else None)
+    # the fused ones
+    k2, v2 = k_pages.clone().cuda(), v_pages.clone().cuda()
+    out2 = torch.full((n, hq * d), float("nan"), dtype=dtype, device="cuda")
+    partial.fill_(float("nan"))
+    k.attention_decode_fused(qkv, k2, v2, table.cuda(), slots, pos, out2, first, ones, n, hq, hkv, d, page, scale,
+                             qw, kw, eps, rope, partial, window=window, split_keys=split_keys, max_splits=max_splits)
+    same = lambda x, y: torch.equal(x.view(torch.int16), y.view(torch.int16))     # NaN-filled entries compare too
+    assert same(k1, k2) and same(v1, v2)
+    torch.testing.assert_close(out2.float(), out1.float(), atol=2e-2, rtol=2e-2)
+    # and the plain attention over the cached keys plus the new one, as the separate launches cached it
+    for s, L in enumerate(lengths):
+        pg, at = table[s, (L - 1) // page].item(), (L - 1) % page
+        kk = torch.cat([keys[s], k1[pg, :, at].cpu()[None]]).double()
+        vv = torch.cat([values[s], v1[pg, :, :, at].cpu()[None]]).double()
+        want = plain_attention(q1[s].double().cpu().view(hq, d), kk, vv, scale, window)
+        torch.testing.assert_close(out2[s].double().cpu().view(hq, d), want, **tol(dtype))
