@@ -1,8 +1,9 @@
-"""The engine at the widths of the benchmark model (hidden 1024, 16 q / 8 kv heads of 128, feed-forward
-3072, vocabulary 151936, tied), with two layers so that the plain implementation stays quick: a 256-token
-prompt whole, in portions and with its last tokens decoded one by one, in 32-bit and in bfloat16, against
-the plain logits.  Tiny models cannot show a fault that needs a head of 128 channels, sixteen query heads
-or a vocabulary that fills many workgroups."""
+"""The engine at the widths of the benchmark models, with few layers so that the plain implementation stays
+quick: hidden 1024, 16 q / 8 kv heads of 128, feed-forward 3072, vocabulary 151936, tied (two layers); and
+hidden 4096, 32 q / 8 kv heads of 128, feed-forward 12288, untied, with a small vocabulary (one layer).  A
+256-token prompt whole, in portions and with its last tokens decoded one by one, in 32-bit and in bfloat16,
+against the plain logits.  Tiny models cannot show a fault that needs a head of 128 channels, four query
+heads per kv head on the matrix cores, rows of 4096 or a vocabulary that fills many workgroups."""
 import numpy as np
 import pytest
 import torch
@@ -14,35 +15,44 @@ pytestmark = pytest.mark.gpu
 CFG = dict(architectures=["Qwen3ForCausalLM"], hidden_size=1024, num_hidden_layers=2, num_attention_heads=16,
            num_key_value_heads=8, head_dim=128, intermediate_size=3072, vocab_size=151936,
            max_position_embeddings=4096, rms_norm_eps=1e-6, rope_theta=1000000.0, tie_word_embeddings=True)
+WIDE = dict(architectures=["Qwen3ForCausalLM"], hidden_size=4096, num_hidden_layers=1, num_attention_heads=32,
+            num_key_value_heads=8, head_dim=128, intermediate_size=12288, vocab_size=8192,
+            max_position_embeddings=4096, rms_norm_eps=1e-6, rope_theta=1000000.0, tie_word_embeddings=False)
+CONFIGS = {"narrow": CFG, "wide": WIDE}
 WANT = [0, 1, 15, 16, 17, 32, 127, 128, 255]          # the reference's probe positions (tests/data/qwen3_validation_cases.json)
 
 
 @pytest.fixture(scope="module")
-def folder(tmp_path_factory):
+def folders(tmp_path_factory):
     from mini_llm_runtime_amd.config import config_from_dict
     from mini_llm_runtime_amd.weights import write_random_model
-    path = str(tmp_path_factory.mktemp("real-sizes"))
-    # N(0, 0.02) as in the benchmark; norm weights 1 + N(0, 0.1)
-    write_random_model(path, config_from_dict(CFG), seed=7)
-    return path
+    out = {}
+    for name, cfg in CONFIGS.items():
+        out[name] = str(tmp_path_factory.mktemp(f"real-sizes-{name}"))
+        # N(0, 0.02) as in the benchmark; norm weights 1 + N(0, 0.1)
+        write_random_model(out[name], config_from_dict(cfg), seed=7)
+    return out
 
 
 @pytest.fixture(scope="module")
-def expected(folder):
+def expectations(folders):
     from plain.qwen3_plain import PlainQwen3
-    toks = make_requests(CFG["vocab_size"], [256], seed=17)["r0"]
-    plain = PlainQwen3(folder)
-    rows = plain.logits(toks, WANT)
-    return toks, {("r0", p): rows[i] for i, p in enumerate(WANT)}
+    out = {}
+    for name, cfg in CONFIGS.items():
+        toks = make_requests(cfg["vocab_size"], [256], seed=17)["r0"]
+        rows = PlainQwen3(folders[name]).logits(toks, WANT)
+        out[name] = (toks, {("r0", p): rows[i] for i, p in enumerate(WANT)})
+    return out
 
 
 @pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
-def test_prompt_of_256_tokens_every_way(folder, expected, dtype_name):
+@pytest.mark.parametrize("name", list(CONFIGS))
+def test_prompt_of_256_tokens_every_way(folders, expectations, name, dtype_name):
     from helpers import run_steps
     from mini_llm_runtime_amd.engine import Runner
     from mini_llm_runtime_amd.parts import DecoderModel
-    toks, want = expected
-    model = DecoderModel.load(folder, torch.float32 if dtype_name == "float32" else torch.bfloat16)
+    toks, want = expectations[name]
+    model = DecoderModel.load(folders[name], torch.float32 if dtype_name == "float32" else torch.bfloat16)
     r = Runner(model, max_tokens=512, max_slots=2, page_size=16)
 
     def wanted(lo, hi):
@@ -74,17 +84,19 @@ def test_prompt_of_256_tokens_every_way(folder, expected, dtype_name):
         assert token == int(np.argmax(row))
 
 
-def test_graph_replays_with_library_products_match_eager(folder):
+@pytest.mark.parametrize("name", list(CONFIGS))
+def test_graph_replays_with_library_products_match_eager(folders, name):
     """24 requests decode together: their projections have more than 16 rows and go to the vendor library,
     inside the captured graph.  Every replay (with eager work and synchronisations between the replays) must
     give what the same steps give without a graph: a library call that records a clearing node would show
     here as a difference on a later replay."""
     from mini_llm_runtime_amd.engine import Entry, Runner
     from mini_llm_runtime_amd.parts import DecoderModel
-    model = DecoderModel.load(folder, torch.bfloat16)
+    model = DecoderModel.load(folders[name], torch.bfloat16)
     n = 24
-    prompts = make_requests(CFG["vocab_size"], [9 + (5 * i) % 23 for i in range(n)], seed=23)
-    feeds = make_requests(CFG["vocab_size"], [8] * n, seed=29)
+    vocab = CONFIGS[name]["vocab_size"]
+    prompts = make_requests(vocab, [9 + (5 * i) % 23 for i in range(n)], seed=23)
+    feeds = make_requests(vocab, [8] * n, seed=29)
     outs = []
     for use_graphs in (True, False):
         r = Runner(model, max_tokens=n * 64, max_slots=n, page_size=16, use_graphs=use_graphs)
