@@ -48,8 +48,10 @@ def main():
     ap.add_argument("--attn-workgroups", type=int, default=512,
                     help="tuning aid: workgroups that the split of a token's keys aims for")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points and the prefill")
-    ap.add_argument("--only", default="all", choices=["all", "decode", "prefill"],
-                    help="profiling aid: run just the decode steps or just the prefill")
+    ap.add_argument("--only", default="all", choices=["all", "decode", "prefill", "engine"],
+                    help="profiling aid: run just the decode steps or just the prefill; engine: the scheduler "
+                         "over a burst of requests (3 x batch requests of 512 prompt and 128 output tokens, "
+                         "batch slots), printed as one line of its own")
     ap.add_argument("--fill", default="prefill", choices=["prefill", "random"],
                     help="how the requests' caches are filled before the timed steps: by real prefill "
                          "(default) or, as a profiling aid, with random keys and values")
@@ -154,6 +156,28 @@ def main():
 
     if args.only == "prefill":
         print(json.dumps({"prefill": prefill_run()}))
+        return 0
+    if args.only == "engine":
+        from mini_llm_runtime_amd.engine import Engine, EngineOptions
+        slots, prompt, output = args.batch, 512, 128
+        engine = Engine(model, EngineOptions(context_tokens=slots * 1024, max_model_len=1024, max_active=slots,
+                                             batch_tokens=max(256, 16 * slots), prefill_chunk=max(128, 8 * slots),
+                                             block_size=args.page_size))
+        requests = 3 * slots
+        for _ in range(requests):
+            engine.submit(torch.randint(0, c.vocab_size, (prompt,), generator=g).tolist(), max_tokens=output,
+                          ignore_eos=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        engine.run_until_done()
+        torch.cuda.synchronize()
+        seconds = time.perf_counter() - t0
+        print(json.dumps({"engine": {"requests": requests, "slots": slots, "prompt_tokens": prompt,
+                                     "output_tokens": output, "seconds": round(seconds, 3),
+                                     "generated_tok_s": round(requests * output / seconds, 1),
+                                     "total_tok_s": round(requests * (prompt + output) / seconds, 1),
+                                     "batches": engine.stats["batches"],
+                                     "mixed_batches": engine.stats["mixed_batches"]}}))
         return 0
     seconds, mean_context = decode_run(args.batch, args.steps, args.warmup)
     ms_per_step = seconds / args.steps * 1e3

@@ -31,7 +31,7 @@ class Entry:
 class Runner:
     def __init__(self, model, max_tokens, max_slots=4, max_length=None, max_batch_tokens=None,
                  page_size=16, split_keys=256, split_max_tokens=256, use_graphs=True, graph_max_batch=256,
-                 target_workgroups=512, graph_max_tokens=512, graph_after=2, max_graphs=48):
+                 target_workgroups=512, graph_max_tokens=512, graph_after=4, max_graphs=48):
         self.model = model
         self.dtype, self.device = model.dtype, model.device
         spec = model.spec
