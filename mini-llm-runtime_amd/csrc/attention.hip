@@ -328,7 +328,8 @@ __global__ __launch_bounds__(256, (NCH <= 4 ? 2 : 1)) void attention_mfma_kernel
     const int grp = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int col = lane & 15, b = lane >> 4;
-    const int row0 = group_row0[grp], ntok = group_ntok[grp];
+    // (FUSED: group i is the one token in batch row i; no need to wait for the group vectors)
+    const int row0 = FUSED ? grp : group_row0[grp], ntok = FUSED ? 1 : group_ntok[grp];
     const int slot = a.slots[row0], pos0 = a.positions[row0];
     const int tok = col / g, hh = col % g;
     const bool col_valid = tok < ntok;
