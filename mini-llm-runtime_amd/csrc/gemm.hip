@@ -322,6 +322,14 @@ __global__ __launch_bounds__(SKINNY_WAVES * 64) void gemm_skinny_norm_kernel(
         for (int g = 0; g < NW; ++g)
             wf[g][i] = *reinterpret_cast<const bf16x8*>(w + ((size_t)g * N + min(n0 + r16, N - 1)) * K + k);
     }
+    // the norm's weights too (they depend on nothing; asked for after the sums they would cost a round trip more)
+    float4 nw0[PW], nw1[PW];
+#pragma unroll
+    for (int i = 0; i < PW; ++i) {
+        const int k = min(s_begin + i, steps - 1) * 32 + b * 8;
+        nw0[i] = *reinterpret_cast<const float4*>(norm_w + k);
+        nw1[i] = *reinterpret_cast<const float4*>(norm_w + k + 4);
+    }
     float x[PW][8];
     float sq = 0.f;
 #pragma unroll
@@ -364,10 +372,7 @@ __global__ __launch_bounds__(SKINNY_WAVES * 64) void gemm_skinny_norm_kernel(
     for (int i = 0; i < PW; ++i) {
         const int s = s_begin + i;
         if (s >= s_end) break;
-        const int k = s * 32 + b * 8;
-        const float4 w0 = *reinterpret_cast<const float4*>(norm_w + k);
-        const float4 w1 = *reinterpret_cast<const float4*>(norm_w + k + 4);
-        const float nw[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+        const float nw[8] = {nw0[i].x, nw0[i].y, nw0[i].z, nw0[i].w, nw1[i].x, nw1[i].y, nw1[i].z, nw1[i].w};
         bf16x8 xf;
 #pragma unroll
         for (int e = 0; e < 8; ++e) xf[e] = (__bf16)((x[i][e] * scale) * nw[e]);
