@@ -18,11 +18,13 @@ Interfaces (B = the tokens of a step, E = the model width, T = the engine's elem
                   write_cache) -> the next pending delta: a block adds `pending` (the previous
                   block's last output) into h itself, fused with its first norm.
 
-A part whose forward only launches work over the step's device vectors (ctx.token_ids, positions,
-slots, the cache views) may set the class attribute `graph_safe = True`: steps of single tokens are
-then captured once as a HIP graph and replayed.  A part that reads host-side facts of the step
-(ctx.segments, ctx.max_context) to decide what to launch must leave it unset; a model with such a part
-runs every step eagerly.
+A part may set the class attribute `graph_safe = True` when what it launches depends only on the step's
+SHAPE -- how many tokens each entry brings (ctx.n_tokens, the lengths in ctx.segments, ctx.single_tokens,
+ctx.token_groups) and ctx.max_context, which is the runner's max_length in a step that is to be captured --
+and everything else reaches its kernels through device memory (ctx.token_ids, positions, slots, the cache
+views).  Steps of a shape that comes again are then captured once as a HIP graph and replayed.  A part
+that reads the slots or positions of ctx.segments on the host, or keeps host-side state per request, must
+leave it unset; a model with such a part runs every step eagerly.
 
 No part is told which model it is in; sizes and constants arrive through its spec.
 """
