@@ -174,14 +174,21 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_bf16_kernel(
 // consecutive n of one m.
 // GATED: w holds two stacked matrices [gate; up] of N rows each; the workgroup computes the same 16
 // columns of both and writes silu(gate) * up (the feed-forward's activation fused into the projection).
+// STAGE (M <= 16, K a multiple of 64): a wavefront reads its part of the activation as M rows of
+// consecutive bytes, puts them into a piece of LDS of its own and takes its operand from there.  Read
+// straight into the operand layout, the activation costs as many requests to the cache as the weight
+// does to memory, and the weight's rate drops by a tenth to a third (measured; more with more rows).
 #define SKINNY_WAVES 8
-template <int MT, bool OUT_FLOAT, bool GATED>
+#define SKINNY_STAGE_PITCH(U) ((U) * 128 + 16)        // bytes a row of the staged activation takes
+#define SKINNY_STAGE_LDS (66 * 1024)                  // the most dynamic LDS a workgroup asks for
+template <int MT, bool OUT_FLOAT, bool GATED, int UMAX = 4, bool STAGE = false>   // UMAX: the most groups of k a turn takes
 __global__ __launch_bounds__(SKINNY_WAVES * 64) void gemm_skinny_kernel(const __bf16* __restrict__ a,
-                                                                         const __bf16* __restrict__ w,
-                                                                         void* __restrict__ out_raw, int M, int N,
-                                                                         int K) {
+                                                               const __bf16* __restrict__ w,
+                                                               void* __restrict__ out_raw, int M, int N, int K) {
     constexpr int NW = GATED ? 2 : 1;
+    static_assert(!STAGE || MT == 1, "the activation is staged for at most 16 rows");
     __shared__ float part[SKINNY_WAVES - 1][NW][MT][64][4];
+    extern __shared__ __attribute__((aligned(16))) char staged[];   // [SKINNY_WAVES][M][pitch] when STAGE
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r16 = lane & 15, b = lane >> 4;
     const int n0 = blockIdx.x * 16;
@@ -211,18 +218,30 @@ __global__ __launch_bounds__(SKINNY_WAVES * 64) void gemm_skinny_kernel(const __
         for (int i = 0; i < MT; ++i) xrow[i] = a + (size_t)min(16 * i + r16, M - 1) * K + b * (8 * W);
         // Full turns of U groups first: every load of a turn (the activation, which comes from the cache,
         // before the weight that follows it in the queue) is asked for before the first product, with no
-        // branch in between.  What is left (fewer than U groups) goes one group at a time.
-        constexpr int U = (MT * NW <= 2) ? 4 : 2;
+        // branch in between.  What is left (fewer than U groups) makes one shorter turn.
+        constexpr int U = (MT * NW <= 2 && UMAX >= 4) ? 4 : 2;
+        constexpr int PITCH = SKINNY_STAGE_PITCH(U);
+        char* mine = staged + (size_t)wave * M * PITCH;
         auto turn = [&](int g0, auto count) {
             constexpr int C = decltype(count)::value;
-            bf16x8 xf[MT][C][W], wf[NW][C][W];
+            constexpr int PPR = C * 8;                        // 16-byte pieces in a row of this turn's chunk
+            bf16x8 xf[MT][C][W], wf[NW][C][W], xg[STAGE ? C * W : 1];
+            if constexpr (STAGE) {
+                // piece p of the chunk: row p / PPR, bytes 16 * (p % PPR); a lane takes pieces lane, lane + 64, ...
 #pragma unroll
-            for (int u = 0; u < C; ++u)
+                for (int i = 0; i < C * W; ++i) {
+                    const int p = min(i * 64 + lane, M * PPR - 1);
+                    xg[i] = *reinterpret_cast<const bf16x8*>(a + (size_t)(p / PPR) * K + (g0 * (32 * W) + (p % PPR) * 8));
+                }
+            } else {
 #pragma unroll
-                for (int i = 0; i < MT; ++i)
+                for (int u = 0; u < C; ++u)
 #pragma unroll
-                    for (int c = 0; c < W; ++c)
-                        xf[i][u][c] = *reinterpret_cast<const bf16x8*>(xrow[i] + (g0 + u) * (32 * W) + 8 * c);
+                    for (int i = 0; i < MT; ++i)
+#pragma unroll
+                        for (int c = 0; c < W; ++c)
+                            xf[i][u][c] = *reinterpret_cast<const bf16x8*>(xrow[i] + (g0 + u) * (32 * W) + 8 * c);
+            }
 #pragma unroll
             for (int u = 0; u < C; ++u)
 #pragma unroll
@@ -230,6 +249,22 @@ __global__ __launch_bounds__(SKINNY_WAVES * 64) void gemm_skinny_kernel(const __
 #pragma unroll
                     for (int c = 0; c < W; ++c)
                         wf[g][u][c] = *reinterpret_cast<const bf16x8*>(wrow + (size_t)g * N * K + (g0 + u) * (32 * W) + 8 * c);
+            __builtin_amdgcn_sched_barrier(0);            // or the compiler spreads the loads among the products
+            if constexpr (STAGE) {
+                // LDS serves a wavefront's accesses in their order: the reads below see these writes, and
+                // the next turn's writes come after these reads.  Rows from M on read row M - 1.
+#pragma unroll
+                for (int i = 0; i < C * W; ++i) {
+                    const int p = i * 64 + lane;
+                    if (p < M * PPR) *reinterpret_cast<bf16x8*>(mine + (p / PPR) * PITCH + (p % PPR) * 16) = xg[i];
+                }
+                const char* row = mine + min(r16, M - 1) * PITCH + b * (16 * W);
+#pragma unroll
+                for (int u = 0; u < C; ++u)
+#pragma unroll
+                    for (int c = 0; c < W; ++c)
+                        xf[0][u][c] = *reinterpret_cast<const bf16x8*>(row + u * (64 * W) + 16 * c);
+            }
 #pragma unroll
             for (int u = 0; u < C; ++u)
 #pragma unroll
@@ -242,7 +277,10 @@ __global__ __launch_bounds__(SKINNY_WAVES * 64) void gemm_skinny_kernel(const __
         };
         int g0 = g_begin;
         for (; g0 + U <= g_end; g0 += U) turn(g0, std::integral_constant<int, U>{});
-        for (; g0 < g_end; ++g0) turn(g0, std::integral_constant<int, 1>{});
+        const int rest = g_end - g0;                      // the same in every lane of a wavefront
+        if (U > 2 && rest == 3) turn(g0, std::integral_constant<int, 3>{});
+        else if (U > 2 && rest == 2) turn(g0, std::integral_constant<int, 2>{});
+        else if (rest == 1) turn(g0, std::integral_constant<int, 1>{});
     } else {
 #pragma unroll 4
         for (int s = s_begin; s < s_end; ++s) {
@@ -403,17 +441,42 @@ __global__ __launch_bounds__(SKINNY_WAVES * 64) void gemm_skinny_norm_kernel(
     }
 }
 
+template <int MT, bool OUT_FLOAT, bool GATED, int UMAX, bool STAGE>
+static int launch_skinny_kernel(const void* a, const void* w, void* out, int M, int N, int K, size_t lds,
+                                hipStream_t stream) {
+    auto* kernel = gemm_skinny_kernel<MT, OUT_FLOAT, GATED, UMAX, STAGE>;
+    if (STAGE) {                                          // static and dynamic LDS together may pass 64 KB
+        static const hipError_t allowed = hipFuncSetAttribute(
+            reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, SKINNY_STAGE_LDS);
+        if (allowed != hipSuccess) return (int)allowed;
+    }
+    kernel<<<dim3((N + 15) / 16), SKINNY_WAVES * 64, lds, stream>>>((const __bf16*)a, (const __bf16*)w, out, M, N, K);
+    return (int)hipGetLastError();
+}
+
+template <int MT, bool GATED, int UMAX, bool STAGE>
+static int launch_skinny_as(const void* a, const void* w, void* out, int M, int N, int K, int out_float,
+                            size_t lds, hipStream_t stream) {
+    if (out_float) return launch_skinny_kernel<MT, true, GATED, UMAX, STAGE>(a, w, out, M, N, K, lds, stream);
+    return launch_skinny_kernel<MT, false, GATED, UMAX, STAGE>(a, w, out, M, N, K, lds, stream);
+}
+
 template <int MT, bool GATED>
 static int launch_skinny(const void* a, const void* w, void* out, int M, int N, int K, int out_float,
                          hipStream_t stream) {
-    dim3 grid((N + 15) / 16);
-    if (out_float)
-        gemm_skinny_kernel<MT, true, GATED><<<grid, SKINNY_WAVES * 64, 0, stream>>>(
-            (const __bf16*)a, (const __bf16*)w, out, M, N, K);
-    else
-        gemm_skinny_kernel<MT, false, GATED><<<grid, SKINNY_WAVES * 64, 0, stream>>>(
-            (const __bf16*)a, (const __bf16*)w, out, M, N, K);
-    return (int)hipGetLastError();
+    // A short k (at most two groups of 64 a wavefront) takes the variant whose turns hold two groups: it
+    // needs fewer registers, so more of its short-lived workgroups fit a compute unit.
+    const bool short_k = MT * (GATED ? 2 : 1) <= 2 && K <= 64 * 2 * SKINNY_WAVES;
+    if constexpr (MT == 1 && !GATED) {
+        // Two rows or more and a long k: the activation goes through LDS.  (Measured: with a short k the
+        // extra step costs what it saves, and the gated variant, whose turns would have to shrink to stay
+        // within the registers of two workgroups a compute unit, gains nothing.)
+        const size_t lds = (size_t)SKINNY_WAVES * M * SKINNY_STAGE_PITCH(4);
+        if (M >= 2 && K % 64 == 0 && K > 2048 && lds <= SKINNY_STAGE_LDS)
+            return launch_skinny_as<MT, GATED, 4, true>(a, w, out, M, N, K, out_float, lds, stream);
+    }
+    if (short_k) return launch_skinny_as<MT, GATED, 2, false>(a, w, out, M, N, K, out_float, 0, stream);
+    return launch_skinny_as<MT, GATED, 4, false>(a, w, out, M, N, K, out_float, 0, stream);
 }
 
 template <int WM, int WN, int TM, int TN>

@@ -117,7 +117,8 @@ def test_silu_mul_and_residual(dtype):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("mnk", [(7, 19, 33), (5, 37, 131), (1, 311, 80), (16, 64, 64), (17, 130, 100),
                                  (64, 200, 76), (65, 257, 256), (200, 300, 1024), (2, 2048, 1024),
-                                 (33, 48, 520), (48, 1000, 264), (8, 6144, 1024), (129, 100, 40)])
+                                 (33, 48, 520), (48, 1000, 264), (8, 6144, 1024), (129, 100, 40),
+                                 (5, 40, 192), (11, 72, 4160), (16, 33, 1024), (9, 130, 3072), (2, 24, 8192), (16, 40, 4096)])
 def test_gemm(dtype, mnk):
     """Odd shapes as in the reference's GEMM test (tests/cuda_unit_tests.cu:207-209)."""
     from mini_llm_runtime_amd.kernels import Kernels
@@ -521,7 +522,8 @@ def test_attention_window_edge(dtype, window):
             assert bool((out.float().cpu()[0] - vv[hot].to(dtype).float()).abs().max() < 0.05) == inside
 
 
-@pytest.mark.parametrize("mnk", [(1, 48, 64), (8, 3072, 1024), (17, 100, 76), (40, 208, 80), (64, 136, 264)])
+@pytest.mark.parametrize("mnk", [(1, 48, 64), (8, 3072, 1024), (17, 100, 76), (40, 208, 80), (64, 136, 264),
+                                 (3, 56, 192), (16, 40, 4160), (13, 72, 2048)])
 def test_gemm_gated_silu(mnk):
     """The feed-forward's activation fused into its first projection (few rows, bfloat16):
     silu(a Wgate^T) * (a Wup^T) with the sums kept in 32-bit until the product."""
