@@ -350,8 +350,29 @@ __global__ __launch_bounds__(SKINNY_WAVES * 64) void gemm_skinny_norm_kernel(
     const int s_begin = wave * PW, s_end = min(steps, s_begin + PW);
     const bool row_ok = r16 < M;
 
-    // the weight first: its loads fly while the norm is computed (no branch around a load; a wavefront
-    // beyond the end of k re-reads the last step and ignores it)
+    // Every load is asked for here, before anything waits and with no branch in between, in the order of
+    // need (loads come back in the order they were asked for): the rows, which the sums of squares wait
+    // for and which come from the cache; the norm's weights; the weight, which comes from memory and
+    // flies while the norm is computed.  A step beyond the end of k and a row beyond M read a valid
+    // place and count as zero; without a delta the load reads the rows' own memory (which is longer)
+    // and its value is dropped.
+    const __bf16* delta_or_any = delta ? delta : reinterpret_cast<const __bf16*>(h_in);
+    float4 a0[PW], a1[PW];
+    bf16x8 d8[PW];
+#pragma unroll
+    for (int i = 0; i < PW; ++i) {
+        const size_t at = (size_t)min(r16, M - 1) * K + min(s_begin + i, steps - 1) * 32 + b * 8;
+        a0[i] = *reinterpret_cast<const float4*>(h_in + at);
+        a1[i] = *reinterpret_cast<const float4*>(h_in + at + 4);
+        d8[i] = *reinterpret_cast<const bf16x8*>(delta_or_any + at);
+    }
+    float4 nw0[PW], nw1[PW];
+#pragma unroll
+    for (int i = 0; i < PW; ++i) {
+        const int k = min(s_begin + i, steps - 1) * 32 + b * 8;
+        nw0[i] = *reinterpret_cast<const float4*>(norm_w + k);
+        nw1[i] = *reinterpret_cast<const float4*>(norm_w + k + 4);
+    }
     bf16x8 wf[NW][PW];
 #pragma unroll
     for (int i = 0; i < PW; ++i) {
@@ -360,39 +381,25 @@ __global__ __launch_bounds__(SKINNY_WAVES * 64) void gemm_skinny_norm_kernel(
         for (int g = 0; g < NW; ++g)
             wf[g][i] = *reinterpret_cast<const bf16x8*>(w + ((size_t)g * N + min(n0 + r16, N - 1)) * K + k);
     }
-    // the norm's weights too (they depend on nothing; asked for after the sums they would cost a round trip more)
-    float4 nw0[PW], nw1[PW];
-#pragma unroll
-    for (int i = 0; i < PW; ++i) {
-        const int k = min(s_begin + i, steps - 1) * 32 + b * 8;
-        nw0[i] = *reinterpret_cast<const float4*>(norm_w + k);
-        nw1[i] = *reinterpret_cast<const float4*>(norm_w + k + 4);
-    }
+    __builtin_amdgcn_sched_barrier(0);
     float x[PW][8];
     float sq = 0.f;
 #pragma unroll
     for (int i = 0; i < PW; ++i) {
-        const int s = s_begin + i;
+        const bool valid = s_begin + i < s_end && row_ok;
+        const float a[8] = {a0[i].x, a0[i].y, a0[i].z, a0[i].w, a1[i].x, a1[i].y, a1[i].z, a1[i].w};
 #pragma unroll
-        for (int e = 0; e < 8; ++e) x[i][e] = 0.f;
-        if (s < s_end && row_ok) {
-            const size_t at = (size_t)r16 * K + s * 32 + b * 8;
-            const float4 a0 = *reinterpret_cast<const float4*>(h_in + at);
-            const float4 a1 = *reinterpret_cast<const float4*>(h_in + at + 4);
-            x[i][0] = a0.x; x[i][1] = a0.y; x[i][2] = a0.z; x[i][3] = a0.w;
-            x[i][4] = a1.x; x[i][5] = a1.y; x[i][6] = a1.z; x[i][7] = a1.w;
-            if (delta) {
-                const bf16x8 d8 = *reinterpret_cast<const bf16x8*>(delta + at);
-#pragma unroll
-                for (int e = 0; e < 8; ++e) x[i][e] += (float)d8[e];
-            }
-            if (h_out && blockIdx.x == 0) {
-                *reinterpret_cast<float4*>(h_out + at) = make_float4(x[i][0], x[i][1], x[i][2], x[i][3]);
-                *reinterpret_cast<float4*>(h_out + at + 4) = make_float4(x[i][4], x[i][5], x[i][6], x[i][7]);
-            }
-#pragma unroll
-            for (int e = 0; e < 8; ++e) sq += x[i][e] * x[i][e];
+        for (int e = 0; e < 8; ++e) {
+            const float v = delta ? a[e] + (float)d8[i][e] : a[e];
+            x[i][e] = valid ? v : 0.f;
         }
+        if (h_out && blockIdx.x == 0 && valid) {
+            const size_t at = (size_t)r16 * K + (s_begin + i) * 32 + b * 8;
+            *reinterpret_cast<float4*>(h_out + at) = make_float4(x[i][0], x[i][1], x[i][2], x[i][3]);
+            *reinterpret_cast<float4*>(h_out + at + 4) = make_float4(x[i][4], x[i][5], x[i][6], x[i][7]);
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) sq += x[i][e] * x[i][e];
     }
     sq += __shfl_xor(sq, 16, MLR_WAVE);
     sq += __shfl_xor(sq, 32, MLR_WAVE);
