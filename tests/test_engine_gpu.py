@@ -221,3 +221,41 @@ def test_steady_steps_allocate_nothing(model_folders):
             r.step([Entry(s, [t, t + 1], [1])])          # a portion between decoded tokens
     torch.cuda.synchronize()
     assert torch.cuda.memory_stats()["allocation.all.allocated"] == before
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_configurations_drawn_at_random(seed, tmp_path):
+    """Sizes nobody chose: head sizes in steps of 16 up to 256, any number of heads and groups, widths
+    and vocabularies that are multiples of nothing in particular, pages of 8 to 64, tied or not.  Whole,
+    last tokens one by one, portions and mixed, in both engines, against the plain implementation."""
+    from mini_llm_runtime_amd.config import config_from_dict
+    from mini_llm_runtime_amd.engine import Runner
+    from mini_llm_runtime_amd.parts import DecoderModel
+    from mini_llm_runtime_amd.weights import write_random_model
+    from plain.qwen3_plain import PlainQwen3
+    rng = np.random.default_rng(1000 + seed)
+    kv_heads = int(rng.integers(1, 5))
+    cfg = dict(architectures=["Qwen3ForCausalLM"],
+               hidden_size=int(rng.integers(16, 150)) * 2 if seed % 2 else int(rng.integers(4, 40)) * 8,
+               num_hidden_layers=int(rng.integers(1, 4)),
+               num_attention_heads=kv_heads * int(rng.choice([1, 2, 3, 4, 5, 8])), num_key_value_heads=kv_heads,
+               head_dim=int(rng.choice([16, 32, 48, 64, 80, 96, 112, 128, 144, 256])),
+               intermediate_size=int(rng.integers(8, 200)) * 2, vocab_size=int(rng.integers(20, 700)),
+               max_position_embeddings=2048, rms_norm_eps=float(rng.choice([1e-6, 1e-5, 3e-6])),
+               rope_theta=float(rng.choice([1e4, 1e6, 5e5])), tie_word_embeddings=bool(rng.random() < 0.5))
+    page = int(rng.choice([8, 16, 32, 64]))
+    folder = str(tmp_path)
+    write_random_model(folder, config_from_dict(cfg), seed=seed, matrix_std=0.12, norm_std=0.2)
+    reqs = make_requests(cfg["vocab_size"], [int(x) for x in rng.integers(2, 160, 5)] + [int(rng.integers(260, 400))],
+                         seed=seed)
+    want = plain_logits(PlainQwen3(folder), reqs)
+    for dtype_name, dtype in DTYPES.items():
+        model = DecoderModel.load(folder, dtype)
+        r = Runner(model, max_tokens=448, max_slots=4, page_size=page)
+        for steps in (whole(reqs), last_one_by_one(reqs), portions(reqs)):
+            compare(run_steps(r, steps), want, dtype_name)
+        steps, peak = mixed(reqs, seed=seed)
+        r = Runner(model, max_tokens=peak, max_slots=4, page_size=page)
+        compare(run_steps(r, steps), want, dtype_name)
+        r.cache.check()
+        assert r.cache.free_pages() == r.cache.num_pages
