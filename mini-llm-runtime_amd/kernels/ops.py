@@ -163,7 +163,7 @@ class Kernels:
         _need(k == k2, lambda: f"gemm: inner sizes differ ({k} and {k2})")
         _need(out.dtype in (self.dtype, torch.float32), lambda: f"gemm: output type {out.dtype} not supported")
         _tensor(out, "out", out.dtype, (m, n))
-        if self.library_gemm and self.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and m > LIBRARY_GEMM_MIN_ROWS:
+        if self.library_gemm and self.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and not self.streams_weight(m, k):
             # many rows: a plain matrix product, handed to the vendor library (hipBLASLt), as the reference
             # hands its projections to cuBLAS (src/minillm/cuda/matrix.cpp:11-37)
             if self._library_workspace is None:
@@ -176,11 +176,21 @@ class Kernels:
         _ok(fn(_p(a), _p(w), _p(out), _c_int(m), _c_int(n), _c_int(k),
                _c_int(1 if out.dtype == torch.float32 else 0), _stream()), "gemm")
 
-    def gated_silu_fused(self, rows):
-        """Whether `gemm_gated_silu` is the path for this many rows: the bfloat16 engine, up to 16 rows with
-        the library in use (above that the library's product and a separate activation are faster), up to
-        64 without."""
-        return self.dtype == torch.bfloat16 and rows <= (LIBRARY_GEMM_MIN_ROWS if self.library_gemm else 64)
+    def streams_weight(self, rows, k):
+        """Whether a projection of this many rows and inner size goes to the kernels that stream the weight
+        once into the matrix cores, and not to the vendor library: up to 16 rows always; up to 64 rows while
+        the rows, which every workgroup reads again, stay small beside its strip of the weight (measured on
+        weights that do not sit in a cache: k = 1024 up to 64 rows, k = 2048 up to 32)."""
+        if self.dtype != torch.bfloat16:
+            return False
+        if not self.library_gemm:
+            return rows <= 64
+        return rows <= LIBRARY_GEMM_MIN_ROWS or (rows <= 64 and k * ((rows + 15) // 16) <= 4096)
+
+    def gated_silu_fused(self, rows, k=None):
+        """Whether `gemm_gated_silu` is the path for this many rows and inner size: the bfloat16 engine, where
+        `streams_weight` says so (elsewhere the library's product and a separate activation are faster)."""
+        return self.streams_weight(rows, k if k is not None else 1 << 30)
 
     def gemm_gated_silu(self, a, w, out):
         """out[M, N] = silu(a . w[:N]^T) * (a . w[N:]^T), w = [gate; up] stacked, for few rows."""

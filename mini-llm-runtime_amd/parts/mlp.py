@@ -45,7 +45,7 @@ class SwiGluMlp:
         s = self.spec
         m = x.shape[0]
         act = ctx.workspace.get("act", (m, s.intermediate), x.dtype)
-        if ctx.kernels.gated_silu_fused(m):           # few rows: the activation rides on the projection
+        if ctx.kernels.gated_silu_fused(m, s.hidden):  # few rows: the activation rides on the projection
             ctx.kernels.gemm_gated_silu(x, self.gate_up, act)
         else:
             gate_up = ctx.workspace.get("gate_up", (m, 2 * s.intermediate), x.dtype)

@@ -532,6 +532,8 @@ def test_gemm_gated_silu(mnk):
     k = Kernels(torch.bfloat16, library_gemm=False)
     assert k.gated_silu_fused(m) and not k.gated_silu_fused(65)
     assert kernels(torch.bfloat16).gated_silu_fused(16) and not kernels(torch.bfloat16).gated_silu_fused(17)
+    # with the library at hand, more rows stay here only while the inner size is small
+    assert kernels(torch.bfloat16).gated_silu_fused(64, 1024) and not kernels(torch.bfloat16).gated_silu_fused(33, 2048)
     a = rnd((m, kk), torch.bfloat16, 50)
     w = rnd((2 * n, kk), torch.bfloat16, 51, 0.3)
     out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
