@@ -85,10 +85,6 @@ class Kernels:
         self._libs = {}
 
     # -- libraries ---------------------------------------------------------------------------
-    @staticmethod
-    def libraries_for(parts=("elementwise", "rope_kv", "attention", "gemm")):
-        return list(parts)
-
     def prepare(self, names):
         """Build (if need be) and load several libraries at once."""
         typed = [n for n in names if build.HIP_LIBRARIES[n][2]]
