@@ -114,3 +114,49 @@ def test_graph_replays_with_library_products_match_eager(folders, name):
     for j, (a, b) in enumerate(zip(*outs)):
         assert np.isfinite(a).all(), j
         np.testing.assert_array_equal(a, b, err_msg=f"decode step {j}")
+
+
+LONG = {
+    # heads as in the 0.6B sizes (two query heads a kv head, 128 channels), narrow otherwise
+    "pairs": dict(architectures=["Qwen3ForCausalLM"], hidden_size=256, num_hidden_layers=2, num_attention_heads=4,
+                  num_key_value_heads=2, head_dim=128, intermediate_size=512, vocab_size=1000,
+                  max_position_embeddings=8192, rms_norm_eps=1e-6, rope_theta=1000000.0, tie_word_embeddings=True),
+    # four query heads a kv head, as in the 8B sizes
+    "fours": dict(architectures=["Qwen3ForCausalLM"], hidden_size=192, num_hidden_layers=1, num_attention_heads=8,
+                  num_key_value_heads=2, head_dim=128, intermediate_size=384, vocab_size=777,
+                  max_position_embeddings=8192, rms_norm_eps=1e-6, rope_theta=1000000.0, tie_word_embeddings=False),
+}
+LONG_TOKENS = 4700
+LONG_WANT = [0, 100, 2047, 2048, 4095, 4096, 4600] + list(range(LONG_TOKENS - 33, LONG_TOKENS))
+
+
+@pytest.mark.parametrize("name", list(LONG))
+def test_a_context_of_4700_tokens(tmp_path, name):
+    """A context beyond 4096 with heads of 128 channels: the prompt in portions of 1500, 1700 and the rest
+    (the later portions attend to thousands of cached keys, in key splits where the engine chooses them),
+    the last 32 tokens one by one (decoding over 4700 keys in key splits).  Both engines against the plain
+    logits at the first, some middle and the last positions."""
+    from helpers import run_steps
+    from mini_llm_runtime_amd.config import config_from_dict
+    from mini_llm_runtime_amd.engine import Runner
+    from mini_llm_runtime_amd.parts import DecoderModel
+    from mini_llm_runtime_amd.weights import write_random_model
+    from plain.qwen3_plain import PlainQwen3
+    cfg = LONG[name]
+    folder = str(tmp_path)
+    write_random_model(folder, config_from_dict(cfg), seed=3, matrix_std=0.06, norm_std=0.1)
+    toks = make_requests(cfg["vocab_size"], [LONG_TOKENS], seed=31)["r0"]
+    rows = PlainQwen3(folder).logits(toks, LONG_WANT)
+    want = {("r0", p): rows[i] for i, p in enumerate(LONG_WANT)}
+    cuts = [0, 1500, 3200, LONG_TOKENS - 32]
+    steps = [dict(step=i, entries=[dict(id="r0", tokens=toks[lo:hi], want=[p - lo for p in LONG_WANT if lo <= p < hi])],
+                  end=[]) for i, (lo, hi) in enumerate(zip(cuts, cuts[1:]))]
+    steps += [dict(step=10 + p, entries=[dict(id="r0", tokens=[toks[p]], want=[0] if p in LONG_WANT else [])], end=[])
+              for p in range(LONG_TOKENS - 32, LONG_TOKENS)]
+    steps[-1]["end"] = ["r0"]
+    for dtype_name, dtype in (("float32", torch.float32), ("bfloat16", torch.bfloat16)):
+        model = DecoderModel.load(folder, dtype)
+        r = Runner(model, max_tokens=4800, max_slots=2, max_length=4800, max_batch_tokens=2048, page_size=16)
+        compare(run_steps(r, steps), want, dtype_name)
+        r.cache.check()
+        assert r.cache.free_pages() == r.cache.num_pages
