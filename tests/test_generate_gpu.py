@@ -51,6 +51,25 @@ def test_greedy_generation_through_the_python_entry_point(model_folders, plain_m
         assert one == outs[0] == plain_models[name].greedy(prompts[0], 8)
 
 
+def test_many_requests_on_a_pool_that_holds_three(model_folders, plain_models):
+    """Thirty requests of every length on a cache of 192 tokens: most of them wait for pages, pages and slots
+    are used again and again, portions of prompts run beside decoding requests; every request still gets
+    the plain implementation's greedy tokens, and everything is given back at the end."""
+    from mini_llm_runtime_amd.api import LLM
+    rng = np.random.default_rng(41)
+    llm = LLM(model_folders["A"], dtype="float32", context_tokens=192, max_model_len=64, max_active=8,
+              batch_tokens=24, prefill_chunk=16, block_size=PAGE_SIZE["A"])
+    lengths = [int(x) for x in rng.integers(1, 50, 30)]
+    prompts = prompts_for("A", lengths)
+    outs = llm.generate(prompts, max_tokens=9)
+    for prompt, out in zip(prompts, outs):
+        assert out == plain_models["A"].greedy(prompt, 9)
+    stats = llm.engine.stats
+    assert stats["mixed_batches"] > 0
+    assert llm.engine.runner.cache.free_pages() == llm.engine.total_pages
+    llm.engine.runner.cache.check()
+
+
 def test_temperature_sampling_is_per_request(model_folders, plain_models):
     """Same seed, same tokens, alone or beside others; each token is the inverse-CDF draw of the plain
     distribution at the request's own uniform number."""
