@@ -25,9 +25,10 @@ __device__ __forceinline__ void chunk_range(int vocab, int chunk, int* begin, in
     *end = min(vocab, *begin + per);
 }
 
+// (Also clears the status words, which the next pass sets: one launch less than a kernel of its own.)
 __global__ __launch_bounds__(THREADS) void chunk_max_kernel(const float* __restrict__ logits, int vocab,
                                                             float* __restrict__ cmax, int32_t* __restrict__ cidx,
-                                                            int32_t* __restrict__ cbad) {
+                                                            int32_t* __restrict__ cbad, int32_t* __restrict__ status) {
     __shared__ float vals[THREADS];
     __shared__ int idxs[THREADS];
     __shared__ int bad;
@@ -35,14 +36,18 @@ __global__ __launch_bounds__(THREADS) void chunk_max_kernel(const float* __restr
     const float* row = logits + (size_t)r * vocab;
     int cb, ce;
     chunk_range(vocab, chunk, &cb, &ce);
-    const int per = (ce - cb + THREADS - 1) / THREADS;
-    const int begin = min(ce, cb + t * per), end = min(ce, begin + per);
     if (t == 0) bad = 0;
+    if (t == 0 && r == 0 && chunk == 0) {
+        status[0] = 0;
+        status[1] = 0x7fffffff;
+    }
     __syncthreads();
+    // neighbouring threads read neighbouring elements; a thread meets its elements in ascending order, so
+    // the first of equal maxima it keeps is the lowest, and the merge below prefers the lower index
     float best = -INFINITY;
     int best_i = 0x7fffffff;
     bool nonfinite = false;
-    for (int i = begin; i < end; ++i) {
+    for (int i = cb + t; i < ce; i += THREADS) {
         const float x = row[i];
         if (!(fabsf(x) <= 3.402823466e38f)) nonfinite = true;
         if (x > best) { best = x; best_i = i; }
@@ -173,11 +178,6 @@ __global__ __launch_bounds__(THREADS) void pick_kernel(const float* __restrict__
     if (t == 0 && chosen >= 0) tokens[r] = chosen;
 }
 
-__global__ void reset_status_kernel(int32_t* status) {
-    status[0] = 0;
-    status[1] = 0x7fffffff;
-}
-
 extern "C" int mlr_sample_scratch_floats(int rows) { return rows * (2 * CHUNKS + 1); }
 extern "C" int mlr_sample_scratch_ints(int rows) { return rows * 2 * CHUNKS; }
 
@@ -193,8 +193,7 @@ extern "C" int mlr_sample(const float* logits, int rows, int vocab, const float*
     float* rmax = scratch_f + (size_t)rows * 2 * CHUNKS;
     int32_t* cidx = scratch_i;
     int32_t* cbad = scratch_i + (size_t)rows * CHUNKS;
-    reset_status_kernel<<<1, 1, 0, stream>>>(status);
-    chunk_max_kernel<<<dim3(rows, CHUNKS), THREADS, 0, stream>>>(logits, vocab, cmax, cidx, cbad);
+    chunk_max_kernel<<<dim3(rows, CHUNKS), THREADS, 0, stream>>>(logits, vocab, cmax, cidx, cbad, status);
     row_max_kernel<<<rows, 64, 0, stream>>>(cmax, cidx, cbad, temperature, rmax, tokens, status);
     if (any_sampling) {
         chunk_sum_kernel<<<dim3(rows, CHUNKS), THREADS, 0, stream>>>(logits, vocab, temperature, rmax, csum);
