@@ -75,7 +75,17 @@ int mlr_cache_add_group(void* h, int page_size, int num_pages, int window) {
     g.num_pages = num_pages;
     g.window = window > 0 ? window : 0;
     g.max_blocks = blocks_for(c->max_length, page_size);
+    // A fresh pool hands its pages out in a fixed shuffled order.  In ascending order, requests of equal
+    // length that start together lie a power of two apart, and the workgroups that read block i of each of
+    // them at the same moment meet in the same memory channels (measured: decoding attention over 64 such
+    // requests streams at 4.7 TB/s, over pages that lie anywhere at 5.7).
     for (int p = num_pages - 1; p >= 0; --p) g.free_list.push_back(p);
+    uint64_t state = 0x9E3779B97F4A7C15ull;
+    for (int i = num_pages - 1; i > 0; --i) {
+        state = state * 6364136223846793005ull + 1442695040888963407ull;
+        const int j = (int)((state >> 33) % (uint64_t)(i + 1));
+        std::swap(g.free_list[i], g.free_list[j]);
+    }
     g.table.assign((size_t)c->max_slots * g.max_blocks, -1);
     g.owner.assign(num_pages, -1);
     g.first_block.assign(c->max_slots, 0);
