@@ -118,7 +118,7 @@ def test_silu_mul_and_residual(dtype):
 @pytest.mark.parametrize("mnk", [(7, 19, 33), (5, 37, 131), (1, 311, 80), (16, 64, 64), (17, 130, 100),
                                  (64, 200, 76), (65, 257, 256), (200, 300, 1024), (2, 2048, 1024),
                                  (33, 48, 520), (48, 1000, 264), (8, 6144, 1024), (129, 100, 40),
-                                 (5, 40, 192), (11, 72, 4160), (16, 33, 1024), (9, 130, 3072), (2, 24, 8192), (16, 40, 4096)])
+                                 (5, 40, 192), (11, 72, 4160), (16, 33, 1024), (9, 130, 3072), (2, 24, 8192), (16, 40, 4096), (40, 96, 4096), (24, 56, 2048)])
 def test_gemm(dtype, mnk):
     """Odd shapes as in the reference's GEMM test (tests/cuda_unit_tests.cu:207-209)."""
     from mini_llm_runtime_amd.kernels import Kernels
