@@ -1,5 +1,5 @@
 // Plain matrix products of many rows, handed to the vendor library (hipBLASLt) without a detour through
-// another framework's dispatcher: out[M, N] = a[M, K] . w[N, K]^T, bfloat16 in and out, 32-bit sums.
+// another framework's dispatcher: out[M, N] = a[M, K] . w[N, K]^T, bfloat16 in, bfloat16 or float out, 32-bit sums.
 // (The reference hands its projections to cuBLAS the same way, src/minillm/cuda/matrix.cpp:11-37.)
 //
 // Row-major out[M, N] is the column-major N x M matrix w^T(as stored: K x N, ld K)^T . a(as stored: K x M,
@@ -21,10 +21,10 @@ struct Plan {
     size_t workspace = 0;
 };
 hipblasLtHandle_t g_handle = nullptr;
-std::map<std::tuple<int, int, int, size_t>, Plan> g_plans;
+std::map<std::tuple<int, int, int, size_t, int>, Plan> g_plans;
 std::mutex g_mutex;
 
-int make_plan(int M, int N, int K, size_t workspace_bytes, Plan& p) {
+int make_plan(int M, int N, int K, size_t workspace_bytes, int out_float, Plan& p) {
     if (hipblasLtMatmulDescCreate(&p.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F) != HIPBLAS_STATUS_SUCCESS) return -10;
     const hipblasOperation_t ta = HIPBLAS_OP_T, tb = HIPBLAS_OP_N;
     if (hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_TRANSA, &ta, sizeof(ta)) != HIPBLAS_STATUS_SUCCESS ||
@@ -32,7 +32,7 @@ int make_plan(int M, int N, int K, size_t workspace_bytes, Plan& p) {
         return -11;
     if (hipblasLtMatrixLayoutCreate(&p.a, HIP_R_16BF, K, N, K) != HIPBLAS_STATUS_SUCCESS ||
         hipblasLtMatrixLayoutCreate(&p.b, HIP_R_16BF, K, M, K) != HIPBLAS_STATUS_SUCCESS ||
-        hipblasLtMatrixLayoutCreate(&p.c, HIP_R_16BF, N, M, N) != HIPBLAS_STATUS_SUCCESS)
+        hipblasLtMatrixLayoutCreate(&p.c, out_float ? HIP_R_32F : HIP_R_16BF, N, M, N) != HIPBLAS_STATUS_SUCCESS)
         return -12;
     hipblasLtMatmulPreference_t pref = nullptr;
     if (hipblasLtMatmulPreferenceCreate(&pref) != HIPBLAS_STATUS_SUCCESS) return -13;
@@ -58,17 +58,17 @@ int make_plan(int M, int N, int K, size_t workspace_bytes, Plan& p) {
 
 // Returns 0, or a negative number that names the library call that failed (-1: bad sizes, -2: no handle,
 // -10 .. -15: setting up the product, -20: the product itself).
-extern "C" int mlr_library_gemm(const void* a, const void* w, void* out, int M, int N, int K, void* workspace,
-                                size_t workspace_bytes, hipStream_t stream) {
+extern "C" int mlr_library_gemm(const void* a, const void* w, void* out, int M, int N, int K, int out_float,
+                                void* workspace, size_t workspace_bytes, hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
     if (K <= 0) return -1;
     std::lock_guard<std::mutex> lock(g_mutex);
     if (g_handle == nullptr && hipblasLtCreate(&g_handle) != HIPBLAS_STATUS_SUCCESS) return -2;
-    const auto key = std::make_tuple(M, N, K, workspace_bytes);
+    const auto key = std::make_tuple(M, N, K, workspace_bytes, out_float ? 1 : 0);
     auto it = g_plans.find(key);
     if (it == g_plans.end()) {
         Plan p;
-        const int rc = make_plan(M, N, K, workspace_bytes, p);
+        const int rc = make_plan(M, N, K, workspace_bytes, out_float, p);
         if (rc != 0) return rc;
         it = g_plans.emplace(key, p).first;
     }

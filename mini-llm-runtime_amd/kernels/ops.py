@@ -159,13 +159,16 @@ class Kernels:
         _need(k == k2, lambda: f"gemm: inner sizes differ ({k} and {k2})")
         _need(out.dtype in (self.dtype, torch.float32), lambda: f"gemm: output type {out.dtype} not supported")
         _tensor(out, "out", out.dtype, (m, n))
-        if self.library_gemm and self.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and not self.streams_weight(m, k):
+        if self.library_gemm and self.dtype == torch.bfloat16 and m > LIBRARY_GEMM_MIN_ROWS and \
+                (out.dtype == torch.float32 or not self.streams_weight(m, k)):
             # many rows: a plain matrix product, handed to the vendor library (hipBLASLt), as the reference
-            # hands its projections to cuBLAS (src/minillm/cuda/matrix.cpp:11-37)
+            # hands its projections to cuBLAS (src/minillm/cuda/matrix.cpp:11-37).  (Float outputs are
+            # logits, a vocabulary wide: there the library wins from 17 rows on at any inner size.)
             if self._library_workspace is None:
                 self._library_workspace = torch.empty(LIBRARY_GEMM_WORKSPACE, dtype=torch.uint8, device=a.device)
             ws = self._library_workspace
             _ok(self._lib("library_gemm").mlr_library_gemm(_p(a), _p(w), _p(out), _c_int(m), _c_int(n), _c_int(k),
+                                                           _c_int(1 if out.dtype == torch.float32 else 0),
                                                            _p(ws), _c_size_t(ws.numel()), _stream()), "library_gemm")
             return
         fn = self._lib("gemm").mlr_gemm
