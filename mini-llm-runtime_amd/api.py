@@ -57,6 +57,8 @@ class LLM:
                                           seed=None if seed is None else seed + i, ignore_eos=ignore_eos))
         done = self.engine.run_until_done()
         out = [done[i] for i in ids]
+        for i in ids:
+            self.engine.finished.pop(i, None)      # handed over: a long-lived engine keeps no record of them
         return out[0] if single else out
 
 
