@@ -102,6 +102,64 @@ __global__ void qk_norm_rope_kv_kernel(
 // half (16-byte accesses); a wavefront serves 64 / (head_dim / 16) heads at once.
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 
+// Values into their transposed pages, sixteen batch rows at a time: the rows' values of one kv head go
+// through LDS so that a thread ends up with eight consecutive rows of one channel.  When those rows are
+// eight consecutive positions of one request inside one page (the usual case in a prompt portion that
+// starts at a multiple of eight) they are one 16-byte store; otherwise element by element.  Done by extra
+// workgroups of the kernel below (the two jobs share nothing; one launch instead of two).
+__device__ __forceinline__ void write_values_transposed(
+    const __bf16* __restrict__ qkv, int ld, __bf16* __restrict__ v_pages, const int32_t* __restrict__ block_table,
+    int max_blocks, const int32_t* __restrict__ slots, const int32_t* __restrict__ positions, int rows, int q_heads,
+    int kv_heads, int head_dim, int page_size, int r0, int kvh) {
+    extern __shared__ __attribute__((aligned(16))) __bf16 tile[];   // [16 rows][head_dim + 8]
+    __shared__ long long row_base[16];                     // element offset of (page, kv head) for each row, or -1
+    __shared__ int row_in_page[16];
+    const int pitch = head_dim + 8;
+    const int chunks = head_dim / 8;                       // 16-byte chunks per row
+    for (int i = threadIdx.x; i < 16 * chunks; i += 256) {
+        const int r = i / chunks, c = i % chunks;
+        bf16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (r0 + r < rows)
+            v = *reinterpret_cast<const bf16x8*>(qkv + (size_t)(r0 + r) * ld + (size_t)(q_heads + kv_heads + kvh) * head_dim + 8 * c);
+        *reinterpret_cast<bf16x8*>(&tile[r * pitch + 8 * c]) = v;
+    }
+    if (threadIdx.x < 16) {
+        const int r = r0 + threadIdx.x;
+        long long base = -1;
+        int in_page = 0;
+        if (r < rows) {
+            const int pos = positions[r];
+            const int page = block_table[(size_t)slots[r] * max_blocks + pos / page_size];
+            if (page >= 0) base = ((long long)page * kv_heads + kvh) * head_dim * page_size;
+            in_page = pos % page_size;
+        }
+        row_base[threadIdx.x] = base;
+        row_in_page[threadIdx.x] = in_page;
+    }
+    __syncthreads();
+    // thread -> (channel d, rows 8 h .. 8 h + 7)
+    for (int i = threadIdx.x; i < 2 * head_dim; i += 256) {
+        const int d = i % head_dim, h = i / head_dim;
+        const long long base = row_base[8 * h];
+        const int in_page = row_in_page[8 * h];
+        bool run = base >= 0 && (in_page & 7) == 0;
+#pragma unroll
+        for (int e = 1; e < 8; ++e) run = run && row_base[8 * h + e] == base && row_in_page[8 * h + e] == in_page + e;
+        if (run) {
+            bf16x8 v;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] = tile[(8 * h + e) * pitch + d];
+            *reinterpret_cast<bf16x8*>(v_pages + base + (long long)d * page_size + in_page) = v;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const long long b = row_base[8 * h + e];
+                if (b >= 0) v_pages[b + (long long)d * page_size + row_in_page[8 * h + e]] = tile[(8 * h + e) * pitch + d];
+            }
+        }
+    }
+}
+
 // Every load is asked for as early as its address is known and none sits behind a branch, so a thread
 // waits for memory twice (the row's position and its own channels; then the page id and the rotation row)
 // instead of once per table.
@@ -111,7 +169,14 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kv_vec_kernel(
     __bf16* __restrict__ v_pages, const int32_t* __restrict__ block_table, int max_blocks,
     const int32_t* __restrict__ slots, const int32_t* __restrict__ positions, const float* __restrict__ q_norm_w,
     const float* __restrict__ k_norm_w, float eps, const float* __restrict__ rope, int q_heads, int kv_heads,
-    int head_dim, int page_size, int write_cache, int skip_values) {
+    int head_dim, int page_size, int write_cache, int skip_values, int rows) {
+    if (blockIdx.x >= (unsigned)rows) {                    // a workgroup beyond the rows: sixteen rows' values of one kv head
+        if (blockIdx.y != 0) return;
+        const int job = blockIdx.x - rows;
+        write_values_transposed(qkv, ld, v_pages, block_table, max_blocks, slots, positions, rows, q_heads, kv_heads,
+                                head_dim, page_size, (job / kv_heads) * 16, job % kv_heads);
+        return;
+    }
     const int m = blockIdx.x;
     const int lph = head_dim / 16;                         // lanes per head (a power of two)
     const int half = head_dim >> 1;
@@ -203,63 +268,6 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kv_vec_kernel(
     *reinterpret_cast<bf16x8*>(dst + half + 8 * c) = o_hi;
 }
 
-// Values into their transposed pages, sixteen batch rows at a time: the rows' values of one kv head go
-// through LDS so that a thread ends up with eight consecutive rows of one channel.  When those rows are
-// eight consecutive positions of one request inside one page (the usual case in a prompt portion that
-// starts at a multiple of eight) they are one 16-byte store; otherwise element by element.
-__global__ __launch_bounds__(256) void v_cache_write_kernel(
-    const __bf16* __restrict__ qkv, int ld, __bf16* __restrict__ v_pages, const int32_t* __restrict__ block_table,
-    int max_blocks, const int32_t* __restrict__ slots, const int32_t* __restrict__ positions, int rows, int q_heads,
-    int kv_heads, int head_dim, int page_size) {
-    extern __shared__ __attribute__((aligned(16))) __bf16 tile[];   // [16 rows][head_dim + 8]
-    __shared__ long long row_base[16];                     // element offset of (page, kv head) for each row, or -1
-    __shared__ int row_in_page[16];
-    const int r0 = blockIdx.x * 16, kvh = blockIdx.y;
-    const int pitch = head_dim + 8;
-    const int chunks = head_dim / 8;                       // 16-byte chunks per row
-    for (int i = threadIdx.x; i < 16 * chunks; i += 256) {
-        const int r = i / chunks, c = i % chunks;
-        bf16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
-        if (r0 + r < rows)
-            v = *reinterpret_cast<const bf16x8*>(qkv + (size_t)(r0 + r) * ld + (size_t)(q_heads + kv_heads + kvh) * head_dim + 8 * c);
-        *reinterpret_cast<bf16x8*>(&tile[r * pitch + 8 * c]) = v;
-    }
-    if (threadIdx.x < 16) {
-        const int r = r0 + threadIdx.x;
-        long long base = -1;
-        int in_page = 0;
-        if (r < rows) {
-            const int pos = positions[r];
-            const int page = block_table[(size_t)slots[r] * max_blocks + pos / page_size];
-            if (page >= 0) base = ((long long)page * kv_heads + kvh) * head_dim * page_size;
-            in_page = pos % page_size;
-        }
-        row_base[threadIdx.x] = base;
-        row_in_page[threadIdx.x] = in_page;
-    }
-    __syncthreads();
-    // thread -> (channel d, rows 8 h .. 8 h + 7)
-    for (int i = threadIdx.x; i < 2 * head_dim; i += 256) {
-        const int d = i % head_dim, h = i / head_dim;
-        const long long base = row_base[8 * h];
-        const int in_page = row_in_page[8 * h];
-        bool run = base >= 0 && (in_page & 7) == 0;
-#pragma unroll
-        for (int e = 1; e < 8; ++e) run = run && row_base[8 * h + e] == base && row_in_page[8 * h + e] == in_page + e;
-        if (run) {
-            bf16x8 v;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) v[e] = tile[(8 * h + e) * pitch + d];
-            *reinterpret_cast<bf16x8*>(v_pages + base + (long long)d * page_size + in_page) = v;
-        } else {
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const long long b = row_base[8 * h + e];
-                if (b >= 0) v_pages[b + (long long)d * page_size + row_in_page[8 * h + e]] = tile[(8 * h + e) * pitch + d];
-            }
-        }
-    }
-}
 #endif
 
 extern "C" int mlr_qk_norm_rope_kv(
@@ -273,27 +281,24 @@ extern "C" int mlr_qk_norm_rope_kv(
 #if MLR_BF16
     const int lph = head_dim / 16;
     if (rows >= 64 && head_dim % 16 == 0 && (lph & (lph - 1)) == 0 && ld % 8 == 0) {
-        // values take a kernel of their own (stores of 16 bytes into the transposed pages) when pages hold
+        // values take workgroups of their own (stores of 16 bytes into the transposed pages) when pages hold
         // a multiple of eight tokens
         const int split_values = write_cache && page_size % 8 == 0;
         const int threads_needed = (total_heads - (split_values ? kv_heads : 0)) * lph;
-        const dim3 grid(rows, (threads_needed + 255) / 256);
+        const int value_jobs = split_values ? ((rows + 15) / 16) * kv_heads : 0;
+        const dim3 grid(rows + value_jobs, (threads_needed + 255) / 256);
+        const size_t lds = split_values ? 16 * (head_dim + 8) * sizeof(__bf16) : 0;
 #define MLR_ROPE_VEC(NORM, ROPE)                                                                                   \
-        qk_norm_rope_kv_vec_kernel<NORM, ROPE><<<grid, 256, 0, stream>>>(                                          \
+        qk_norm_rope_kv_vec_kernel<NORM, ROPE><<<grid, 256, lds, stream>>>(                                        \
             (const __bf16*)qkv, ld, (__bf16*)q_out, (__bf16*)k_pages, (__bf16*)v_pages, block_table, max_blocks,  \
             slots, positions, q_norm_w, k_norm_w, eps, rope, q_heads, kv_heads, head_dim, page_size, write_cache, \
-            split_values)
+            split_values, rows)
         const bool norm = q_norm_w != nullptr && k_norm_w != nullptr;
         if (norm && rope) MLR_ROPE_VEC(true, true);
         else if (norm) MLR_ROPE_VEC(true, false);
         else if (rope) MLR_ROPE_VEC(false, true);
         else MLR_ROPE_VEC(false, false);
 #undef MLR_ROPE_VEC
-        if (split_values) {
-            v_cache_write_kernel<<<dim3((rows + 15) / 16, kv_heads), 256, 16 * (head_dim + 8) * sizeof(__bf16), stream>>>(
-                (const __bf16*)qkv, ld, (__bf16*)v_pages, block_table, max_blocks, slots, positions, rows, q_heads,
-                kv_heads, head_dim, page_size);
-        }
         return (int)hipGetLastError();
     }
 #endif
