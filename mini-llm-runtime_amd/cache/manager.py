@@ -52,9 +52,9 @@ class StateSpec:
 
 @dataclass
 class KvView:
-    k_pages: torch.Tensor             # [num_pages, kv_heads, page_size, head_dim]
-    v_pages: torch.Tensor             # [num_pages, kv_heads, head_dim, page_size]
-    block_table: torch.Tensor         # device int32 [max_slots, max_blocks]
+    k_pages: torch.Tensor             # [num_pages + 1, kv_heads, page_size, head_dim] (the last page: scratch)
+    v_pages: torch.Tensor             # [num_pages + 1, kv_heads, head_dim, page_size]
+    block_table: torch.Tensor         # device int32 [max_slots + 1, max_blocks] (the last row: the scratch request)
     page_size: int
     window: Optional[int]
     group: int
@@ -233,14 +233,20 @@ class CacheManager:
         self.group_specs = [None] * len(members)
         for spec, g in self._group_of_spec.items():
             self.group_specs[g] = spec
+        # Beyond the pool and the slots of the bookkeeping, every group has one page more and every block
+        # table one row more: a scratch request of one token (slot `scratch_slot`, its only block mapped to
+        # that page), with which a step may fill a batch up to a size it has a captured graph for.  Models
+        # with per-request state have no such request (its state would have to be kept apart too).
+        self.scratch_slot = max_slots if all(not isinstance(s, StateSpec) for s in self.entry_specs) else None
         self._k, self._v, self._tables = [], [], []
         for g, spec in enumerate(self.group_specs):
-            shape = (len(members[g]), self.num_pages, spec.kv_heads, page_size, spec.head_dim)
-            v_shape = (len(members[g]), self.num_pages, spec.kv_heads, spec.head_dim, page_size)
+            shape = (len(members[g]), self.num_pages + 1, spec.kv_heads, page_size, spec.head_dim)
+            v_shape = (len(members[g]), self.num_pages + 1, spec.kv_heads, spec.head_dim, page_size)
             self._k.append(torch.full(shape, float("nan"), dtype=dtype, device=self.device))
             self._v.append(torch.full(v_shape, float("nan"), dtype=dtype, device=self.device))
-            self._tables.append(torch.full((max_slots, self.book.max_blocks(g)), -1, dtype=torch.int32,
-                                           device=self.device))
+            table = torch.full((max_slots + 1, self.book.max_blocks(g)), -1, dtype=torch.int32, device=self.device)
+            table[max_slots, 0] = self.num_pages
+            self._tables.append(table)
         self._states = {}
         for cid, spec in enumerate(self.entry_specs):
             if isinstance(spec, StateSpec):
@@ -298,7 +304,7 @@ class CacheManager:
                 continue
             host = torch.from_numpy(self.book.table(g))
             if len(rows) * 4 >= self.max_slots:
-                dev.copy_(host)
+                dev[:self.max_slots].copy_(host)
             else:
                 for s in rows:
                     dev[s].copy_(host[s])

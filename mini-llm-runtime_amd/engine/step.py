@@ -31,7 +31,7 @@ class Entry:
 class Runner:
     def __init__(self, model, max_tokens, max_slots=4, max_length=None, max_batch_tokens=None,
                  page_size=16, split_keys=256, split_max_tokens=256, use_graphs=True, graph_max_batch=256,
-                 target_workgroups=512, graph_max_tokens=512, graph_after=4, max_graphs=48):
+                 target_workgroups=512, graph_max_tokens=512, graph_after=4, max_graphs=64):
         self.model = model
         self.dtype, self.device = model.dtype, model.device
         spec = model.spec
@@ -78,6 +78,20 @@ class Runner:
         """What a captured step is fixed to: how many tokens every entry brings and where it wants logits."""
         return tuple((len(e.tokens), tuple(int(w) for w in e.want)) for e in entries)
 
+    def _decode_fill(self, entries):
+        """How many rows of the scratch request fill a batch of single tokens (each wanting its logits) up to
+        a size that comes again: every size up to 8, even sizes up to 16, multiples of 4 up to 64, of 8
+        beyond.  So that a server whose requests come and go captures a few dozen graphs, not one for every
+        number of live requests."""
+        n = len(entries)
+        if self.cache.scratch_slot is None or not self.use_graphs:
+            return 0
+        if any(len(e.tokens) != 1 or list(e.want) != [0] for e in entries):
+            return 0
+        step = 1 if n <= 8 else 2 if n <= 16 else 4 if n <= 64 else 8
+        filled = -(-n // step) * step
+        return filled - n if filled <= min(self.graph_max_batch, self.max_batch_tokens) else 0
+
     def _graph_wanted(self, entries, total, sig):
         """Steps are launch-bound unless they bring many tokens.  Steps of single tokens with logits for
         each (decoding) are captured the second time they come, others (portions beside decoded tokens)
@@ -86,7 +100,7 @@ class Runner:
             return False
         if sig in self._graphs:
             return True
-        if total == len(entries) and all(w == (0,) for _, w in sig):
+        if total == len(sig) and all(w == (0,) for _, w in sig):
             return total <= self.graph_max_batch
         seen = self._seen.get(sig, 0) + 1
         self._seen[sig] = seen
@@ -107,7 +121,7 @@ class Runner:
                 return False
         return True
 
-    def _graph_step(self, entries, first, total, sig):
+    def _graph_step(self, entries, first, total, sig, fill=0):
         """The same kernels as any step, launched from a captured graph.  The graph's buffers are fixed:
         token ids, positions and slots live in a vector of their own per shape (the wanted rows and the
         token groups, which depend on the shape only, are written there once), key splits are laid out
@@ -139,6 +153,11 @@ class Runner:
             ids.extend(int(t) for t in e.tokens)
             pos.extend(range(p0, p0 + n))
             slot_of.extend([e.slot] * n)
+        for _ in range(fill):                             # rows of the scratch request: token 0 at position 0
+            segments.append((self.cache.scratch_slot, len(ids), 1, 0))
+            ids.append(0)
+            pos.append(0)
+            slot_of.append(self.cache.scratch_slot)
         state["upload"].send(ids + pos + slot_of, meta)
         if state["graph"] is not None:
             state["graph"].replay()
@@ -148,7 +167,7 @@ class Runner:
         ctx.n_tokens = total
         ctx.token_ids, ctx.positions, ctx.slots = meta[0:total], meta[total:2 * total], meta[2 * total:3 * total]
         ctx.segments = segments
-        ctx.single_tokens = total == len(entries)
+        ctx.single_tokens = total == len(segments)
         r = state["rows"]
         want_rows = meta[3 * total:3 * total + r] if r else None
         if state["eager"]:                                # a shape whose capture did not hold
@@ -210,11 +229,14 @@ class Runner:
         first = self.cache.commit_first(slots, counts)    # raises with nothing changed, else takes the pages
         try:
             sig = self._signature(entries) if self.use_graphs and total <= self.graph_max_tokens else None
-            if sig is not None and self._graph_wanted(entries, total, sig):
-                logits = self._graph_step(entries, first, total, sig)
+            fill = self._decode_fill(entries) if sig is not None else 0
+            if fill:
+                sig = sig + ((1, (0,)),) * fill
+            if sig is not None and self._graph_wanted(entries, total + fill, sig):
+                logits = self._graph_step(entries, first, total + fill, sig, fill)
                 self.cache.retire(slots)
                 self.steps += 1
-                return logits
+                return logits[:len(entries)] if fill else logits
             ids, pos, slot_of, rows = [], [], [], []
             segments = []
             for e, p0 in zip(entries, first):

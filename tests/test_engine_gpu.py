@@ -115,6 +115,50 @@ def test_a_step_shape_that_comes_again_is_captured_and_stays_right(model_folders
     assert r.cache.free_pages() == r.cache.num_pages
 
 
+@pytest.mark.parametrize("dtype_name", DTYPES)
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_decode_batches_are_filled_up_to_a_size_that_comes_again(model_folders, plain_models, name, dtype_name):
+    """Eleven requests decode together, then ten, then nine: the steps run as graphs of twelve and of ten
+    rows, the rows beyond the live requests being tokens of a scratch request that owns a page outside the
+    pool.  Every step's logits against the plain ones, and against the same steps without graphs."""
+    from mini_llm_runtime_amd.engine import Entry
+    vocab = TINY[name]["vocab_size"]
+    n = 11
+    reqs = make_requests(vocab, [5 + (7 * i) % 19 + 12 for i in range(n)], seed=37)
+    want = plain_logits(plain_models[name], reqs)
+    model = load(model_folders, name, dtype_name)
+    outs = []
+    for use_graphs in (True, False):
+        from mini_llm_runtime_amd.engine import Runner
+        r = Runner(model, max_tokens=n * 64, max_slots=n, page_size=PAGE_SIZE[name], use_graphs=use_graphs)
+        slots, at, got = {}, {}, {}
+        for rid, toks in reqs.items():
+            slots[rid] = r.open_request()
+            at[rid] = len(toks) - 12
+            r.step([Entry(slots[rid], toks[:at[rid]], [])])
+        live = list(reqs)
+        for step in range(12):
+            if step in (4, 8):                              # one request ends: eleven -> ten -> nine
+                r.close_request(slots.pop(live.pop()))
+            logits = r.step([Entry(slots[rid], [reqs[rid][at[rid]]], [0]) for rid in live])
+            assert logits.shape[0] == len(live)
+            rows = logits.double().cpu().numpy()
+            for rid, row in zip(live, rows):
+                got[(rid, at[rid])] = row
+                at[rid] += 1
+        compare(got, {k: want[k] for k in got}, dtype_name)
+        if use_graphs:
+            sizes = sorted(len(sig) for sig, st in r._graphs.items() if st["graph"] is not None)
+            assert sizes == [10, 12] and r.graph_failures == 0
+        for rid in live:
+            r.close_request(slots[rid])
+        r.cache.check()
+        assert r.cache.free_pages() == r.cache.num_pages
+        outs.append(got)
+    limit = 2e-5 if dtype_name == "float32" else 0.03 * max(float(np.abs(v).max()) for v in outs[0].values())
+    assert max_difference(outs[0], outs[1]) <= limit
+
+
 @pytest.mark.parametrize("mode", ["evict", "mismatch"])
 def test_graphs_that_are_dropped_or_do_not_hold(model_folders, plain_models, mode, monkeypatch):
     """With room for one captured shape, two alternating shapes push each other out again and again; and a
