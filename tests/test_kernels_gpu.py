@@ -767,3 +767,37 @@ def test_decode_attention_that_norms_rotates_and_caches_itself(case):
         vv = torch.cat([values[s], v1[pg, :, :, at].cpu()[None]]).double()
         want = plain_attention(q1[s].double().cpu().view(hq, d), kk, vv, scale, window)
         torch.testing.assert_close(out2[s].double().cpu().view(hq, d), want, **tol(dtype))
+
+
+def test_bfloat16_widening_and_rounding():
+    """Every one of the 65536 bfloat16 patterns widens to the float of the same value (the embedding gather
+    is the kernel that does nothing else), and a 32-bit sum that lies exactly between two bfloat16 values
+    is rounded to the even one (the projections' epilogue), below and above one, in both signs -- the
+    reference checks its 16-bit conversions the same way (tests/core_tests.cpp:244-254,
+    tests/cuda_ops_tests.cu:75-101)."""
+    from mini_llm_runtime_amd.kernels import Kernels
+    k = kernels(torch.bfloat16)
+    patterns = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16).view(512, 128).cuda()
+    ids = torch.arange(512, dtype=torch.int32, device="cuda")
+    h = torch.empty((512, 128), dtype=torch.float32, device="cuda")
+    k.embed_gather(ids, patterns, h)
+    want = patterns.float()
+    assert torch.equal(h.view(torch.int32), want.view(torch.int32))          # bit for bit, NaN payloads too
+    # sums a0 * 1 + a1 * 1 with a0 a bfloat16 value and a1 half a unit in its last place
+    cases = []
+    for exponent in (-20, -1, 0, 1, 7, 30):
+        for mantissa in (0, 1, 2, 126, 127):
+            base = (1.0 + mantissa / 128.0) * 2.0 ** exponent
+            half_ulp = 2.0 ** (exponent - 8)
+            even = base if mantissa % 2 == 0 else base + 2 * half_ulp
+            for sign in (1.0, -1.0):
+                cases.append((sign * base, sign * half_ulp, sign * even))
+    a = torch.tensor([[c[0], c[1]] for c in cases], dtype=torch.float32)
+    assert torch.equal(a.to(torch.bfloat16).float(), a)                      # the summands are exact in bfloat16
+    w = torch.ones((8, 2), dtype=torch.bfloat16, device="cuda")
+    want = torch.tensor([c[2] for c in cases], dtype=torch.float32)
+    for engine in (k, Kernels(torch.bfloat16, library_gemm=False)):
+        for rows in (len(cases), 16, 5):                                     # many rows (the library, or tiles) and few
+            out = torch.empty((rows, 8), dtype=torch.bfloat16, device="cuda")
+            engine.gemm(a[:rows].to(torch.bfloat16).cuda(), w, out)
+            assert torch.equal(out.float().cpu(), want[:rows, None].expand(rows, 8)), rows
