@@ -160,3 +160,33 @@ def test_a_context_of_4700_tokens(tmp_path, name):
         compare(run_steps(r, steps), want, dtype_name)
         r.cache.check()
         assert r.cache.free_pages() == r.cache.num_pages
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", list(CONFIGS))
+def test_six_requests_decode_together(folders, name, dtype_name):
+    """Six requests of different lengths decode side by side at the benchmark models' widths: projections of
+    six rows (with an inner size of 4096 and 12288 in the wide model, where the rows are staged through LDS),
+    decoding attention over contexts of different lengths in one launch.  Against the plain logits."""
+    from helpers import plain_logits, run_steps
+    from mini_llm_runtime_amd.engine import Runner
+    from mini_llm_runtime_amd.parts import DecoderModel
+    from plain.qwen3_plain import PlainQwen3
+    cfg = CONFIGS[name]
+    reqs = make_requests(cfg["vocab_size"], [21, 40, 33, 17, 52, 28], seed=43)
+    plain = PlainQwen3(folders[name])
+    want = {}
+    for rid, toks in reqs.items():
+        rows = plain.logits(toks, list(range(len(toks) - 5, len(toks))))
+        for i, p in enumerate(range(len(toks) - 5, len(toks))):
+            want[(rid, p)] = rows[i]
+    model = DecoderModel.load(folders[name], torch.float32 if dtype_name == "float32" else torch.bfloat16)
+    r = Runner(model, max_tokens=6 * 64, max_slots=6, page_size=16)
+    steps = [dict(step=i, entries=[dict(id=rid, tokens=toks[:len(toks) - 5], want=[])], end=[])
+             for i, (rid, toks) in enumerate(reqs.items())]
+    for j in range(5):
+        steps.append(dict(step=10 + j, end=[], entries=[
+            dict(id=rid, tokens=[toks[len(toks) - 5 + j]], want=[0]) for rid, toks in reqs.items()]))
+    steps[-1]["end"] = list(reqs)
+    compare(run_steps(r, steps), want, dtype_name)
+    r.cache.check()
