@@ -106,3 +106,14 @@ def test_load_config_from_folder(tmp_path):
                                                           sliding_window=None, max_window_layers=2,
                                                           use_cache=True, bos_token_id=1)))
     assert load_config(str(tmp_path)).vocab_size == 517
+
+
+def test_the_benchmark_refuses_more_than_one_gpu():
+    """One line and exit code 2, before anything touches a GPU."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    done = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
+                          timeout=120)
+    assert done.returncode == 2 and len(done.stdout.strip().splitlines()) == 1 and "--gpus 2" in done.stdout
