@@ -46,15 +46,17 @@ class LLM:
     def runner(self):
         return self.engine.runner
 
-    def generate(self, prompts, max_tokens=32, temperature=0.0, seed=None, ignore_eos=False):
+    def generate(self, prompts, max_tokens=32, temperature=0.0, seed=None, ignore_eos=False, timeout_ms=None):
         """`prompts`: one list of token ids or a list of such lists.  Returns the generated ids
-        (without the prompt), in the same shape."""
+        (without the prompt), in the same shape.  A request that runs out of `timeout_ms` returns what it
+        has generated until then."""
         single = len(prompts) > 0 and not isinstance(prompts[0], (list, tuple))
         batch = [prompts] if single else list(prompts)
         ids = []
         for i, prompt in enumerate(batch):
             ids.append(self.engine.submit(prompt, max_tokens=max_tokens, temperature=temperature,
-                                          seed=None if seed is None else seed + i, ignore_eos=ignore_eos))
+                                          seed=None if seed is None else seed + i, ignore_eos=ignore_eos,
+                                          timeout_ms=timeout_ms))
         done = self.engine.run_until_done()
         out = [done[i] for i in ids]
         for i in ids:

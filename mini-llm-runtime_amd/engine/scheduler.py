@@ -120,6 +120,8 @@ class Request:
     generated: List[int] = field(default_factory=list)
     rng: Optional[RequestRng] = None
     finish_reason: Optional[str] = None
+    deadline: Optional[float] = None  # on the engine's clock; None: no time limit
+    cancelled: bool = False
 
 
 class Engine:
@@ -147,7 +149,11 @@ class Engine:
                           max_batch_tokens=0, max_batch_sequences=0, admission_waits=0)
 
     # -- submit ----------------------------------------------------------------------------------
-    def submit(self, prompt, max_tokens=64, temperature=0.0, seed=None, ignore_eos=False, priority=0):
+    def submit(self, prompt, max_tokens=64, temperature=0.0, seed=None, ignore_eos=False, priority=0,
+               timeout_ms=None):
+        """Queues a request and returns its id.  `timeout_ms` (1 .. 300000, as the reference allows,
+        src/engine.cpp:658): the request ends with the reason "timeout" at the first step boundary after
+        that long, waiting or running, and keeps what it has generated."""
         o = self.options
         if self.failed:
             raise RuntimeError("the engine stopped after a failed step")
@@ -167,6 +173,8 @@ class Engine:
             raise ValueError("priority must be in 0..3")
         if temperature < 0:
             raise ValueError("temperature must not be negative")
+        if timeout_ms is not None and not 1 <= timeout_ms <= 300000:
+            raise ValueError("timeout_ms must be in 1..300000")
         if len(self.waiting) >= o.queue_capacity:
             raise RuntimeError("the waiting queue is full")
         now = self.clock()
@@ -175,9 +183,35 @@ class Engine:
         req = Request(rid, prompt, max_tokens, float(temperature), rid if seed is None else int(seed),
                       bool(ignore_eos), priority, order=self._order, created=now, last_scheduled=now)
         req.rng = RequestRng(req.seed)
+        req.deadline = None if timeout_ms is None else now + timeout_ms / 1000.0
         self._order += 1
         self.waiting.append(req)
         return rid
+
+    def cancel(self, request_id):
+        """Asks a waiting or running request to end; it does at the next step boundary, with the reason
+        "cancelled" (src/engine.cpp:262-284, 709-716).  False when no such request waits or runs."""
+        for req in self.waiting + self.active:
+            if req.id == request_id:
+                req.cancelled = True
+                return True
+        return False
+
+    def _expire(self):
+        """Ends what was cancelled or has run out of time, before the next batch is formed: a waiting request
+        leaves the queue, a running one gives back its slot, its pages and its reservation."""
+        now = self.clock()
+        events = []
+        for req in [r for r in self.waiting + self.active if r.cancelled or (r.deadline is not None and now >= r.deadline)]:
+            reason = "cancelled" if req.cancelled else "timeout"
+            if req.slot is None:
+                self.waiting.remove(req)
+                req.finish_reason = reason
+                self.finished[req.id] = req
+            else:
+                self._finish(req, reason)
+            events.append((req.id, None, reason))
+        return events
 
     def _pages_for(self, tokens):
         return (tokens + self.options.block_size - 1) // self.options.block_size
@@ -220,16 +254,17 @@ class Engine:
 
     # -- one iteration ---------------------------------------------------------------------------
     def step(self):
-        """Admit, form one batch, run it, sample, finish.  Returns the events of this iteration:
-        [(request id, token, finish reason or None)]."""
+        """End what was cancelled or timed out, admit, form one batch, run it, sample, finish.  Returns the
+        events of this iteration: [(request id, token or None, finish reason or None)]."""
         if self.failed:
             raise RuntimeError("the engine stopped after a failed step")
         o = self.options
+        expired = self._expire()
         self._admit_waiting()
         if not self.active:
             if self.waiting:
                 raise RuntimeError("no request fits an otherwise idle KV pool")
-            return []
+            return expired
         now = self.clock()
         items = [(i, len(r.prompt) - r.processed, r.priority, int((now - r.last_scheduled) * 1000), r.order)
                  for i, r in enumerate(self.active)]
@@ -290,7 +325,7 @@ class Engine:
         for rid, _, reason in events:
             if reason is not None:
                 self._finish(next(r for r in self.active if r.id == rid), reason)
-        return events
+        return expired + events
 
     def has_work(self):
         return bool(self.waiting or self.active)

@@ -70,6 +70,26 @@ def test_many_requests_on_a_pool_that_holds_three(model_folders, plain_models):
     llm.engine.runner.cache.check()
 
 
+def test_a_cancelled_request_leaves_the_others_alone(model_folders, plain_models):
+    from mini_llm_runtime_amd.engine import Engine, EngineOptions
+    from mini_llm_runtime_amd.parts import DecoderModel
+    import torch
+    model = DecoderModel.load(model_folders["A"], torch.float32)
+    eng = Engine(model, EngineOptions(context_tokens=256, max_model_len=64, max_active=3, batch_tokens=16,
+                                      prefill_chunk=8, block_size=PAGE_SIZE["A"]))
+    prompts = prompts_for("A", (20, 9, 14))
+    ids = [eng.submit(p, max_tokens=12) for p in prompts]
+    for _ in range(4):
+        eng.step()
+    assert eng.cancel(ids[0])
+    done = eng.run_until_done()
+    assert eng.finished[ids[0]].finish_reason == "cancelled" and len(done[ids[0]]) < 12
+    for i in (1, 2):
+        assert done[ids[i]] == plain_models["A"].greedy(prompts[i], 12)
+    assert eng.runner.cache.free_pages() == eng.total_pages and eng.runner.free_slots() == 3
+    eng.runner.cache.check()
+
+
 def test_temperature_sampling_is_per_request(model_folders, plain_models):
     """Same seed, same tokens, alone or beside others; each token is the inverse-CDF draw of the plain
     distribution at the request's own uniform number."""

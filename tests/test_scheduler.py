@@ -277,3 +277,45 @@ def test_option_parser():
             Options(["--t", text], {"--t"}).number("--t", 0.0, 0.0, 10.0)
     with pytest.raises(OptionError):
         Options(["--p", "1,a"], {"--p"}).integers("--p")
+
+
+def test_cancelled_requests_end_at_the_next_step_and_give_everything_back():
+    """The reference's engine_bounded_queue_and_cancellation (tests/core_tests.cpp:969-981): a cancelled request
+    ends with the reason "cancelled", the engine is idle afterwards, and an unknown id is not cancelled."""
+    eng, now = engine(context_tokens=128, max_active=2)
+    a = eng.submit(list(range(1, 30)), max_tokens=20)
+    b = eng.submit(list(range(40, 50)), max_tokens=20)
+    c = eng.submit(list(range(60, 70)), max_tokens=20)       # waits: two slots
+    for _ in range(3):
+        eng.step()
+    assert eng.cancel(a) and eng.cancel(c) and not eng.cancel(12345)
+    events = eng.step()
+    assert (a, None, "cancelled") in events and (c, None, "cancelled") in events
+    assert eng.finished[a].finish_reason == "cancelled" and eng.finished[c].generated == []
+    done = eng.run_until_done()
+    assert done[b] == serial(list(range(40, 50)), 20)          # the neighbour is not disturbed
+    assert len(done[a]) < 20
+    assert eng.free_credits == eng.total_pages and eng.runner.book.free_pages() == 128 // 16
+    assert eng.runner.free_slots() == 2 and not eng.has_work()
+    assert not eng.cancel(b)                                    # finished: nothing to cancel
+
+
+def test_a_request_out_of_time_ends_waiting_or_running():
+    """tests/core_tests.cpp:983-997: the reason is "timeout" and the resources come back."""
+    eng, now = engine(context_tokens=128, max_active=1)
+    a = eng.submit(list(range(1, 20)), max_tokens=40, timeout_ms=50)
+    b = eng.submit(list(range(30, 40)), max_tokens=5, timeout_ms=20)     # waits behind a; runs out of time there
+    c = eng.submit(list(range(50, 60)), max_tokens=5)
+    eng.step()
+    now[0] += 0.03
+    events = eng.step()
+    assert (b, None, "timeout") in events and eng.finished[b].generated == []
+    now[0] += 0.03
+    events = eng.step()
+    assert (a, None, "timeout") in events and eng.finished[a].finish_reason == "timeout"
+    done = eng.run_until_done()
+    assert done[c] == serial(list(range(50, 60)), 5)
+    assert eng.free_credits == eng.total_pages and eng.runner.free_slots() == 1
+    for bad in (0, 300001):
+        with pytest.raises(ValueError):
+            eng.submit([1, 2], max_tokens=2, timeout_ms=bad)
