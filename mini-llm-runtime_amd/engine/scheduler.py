@@ -156,7 +156,7 @@ class Engine:
         that long, waiting or running, and keeps what it has generated."""
         o = self.options
         if self.failed:
-            raise RuntimeError("the engine stopped after a failed step")
+            raise RuntimeError("the engine stopped (a failed step, or shut down)")
         prompt = [int(t) for t in prompt]
         vocab = self.model.spec.vocab_size
         if not prompt:
@@ -196,6 +196,15 @@ class Engine:
                 req.cancelled = True
                 return True
         return False
+
+    def shutdown(self):
+        """Ends every waiting and running request with the reason "cancelled" and takes no new ones
+        (src/engine.cpp:637).  Returns the events."""
+        for req in self.waiting + self.active:
+            req.cancelled = True
+        events = self._expire()
+        self.failed = True
+        return events
 
     def _expire(self):
         """Ends what was cancelled or has run out of time, before the next batch is formed: a waiting request

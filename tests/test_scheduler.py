@@ -319,3 +319,16 @@ def test_a_request_out_of_time_ends_waiting_or_running():
     for bad in (0, 300001):
         with pytest.raises(ValueError):
             eng.submit([1, 2], max_tokens=2, timeout_ms=bad)
+
+
+def test_shutdown_ends_queued_and_running_requests():
+    """tests/core_tests.cpp:1054: everything ends as cancelled, everything comes back, nothing new is taken."""
+    eng, now = engine(context_tokens=128, max_active=2)
+    ids = [eng.submit(list(range(1 + 10 * i, 9 + 10 * i)), max_tokens=30) for i in range(4)]
+    for _ in range(3):
+        eng.step()
+    events = eng.shutdown()
+    assert sorted(e[0] for e in events) == ids and all(e[2] == "cancelled" for e in events)
+    assert not eng.has_work() and eng.free_credits == eng.total_pages and eng.runner.free_slots() == 2
+    with pytest.raises(RuntimeError):
+        eng.submit([1, 2, 3])
