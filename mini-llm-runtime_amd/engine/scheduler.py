@@ -146,7 +146,7 @@ class Engine:
         self._order = 0
         self.failed = False
         self.stats = dict(batches=0, mixed_batches=0, prefill_tokens=0, decode_tokens=0, generated_tokens=0,
-                          max_batch_tokens=0, max_batch_sequences=0, admission_waits=0)
+                          max_batch_tokens=0, max_batch_sequences=0, admission_waits=0, cancelled=0, timeouts=0)
 
     # -- submit ----------------------------------------------------------------------------------
     def submit(self, prompt, max_tokens=64, temperature=0.0, seed=None, ignore_eos=False, priority=0,
@@ -213,6 +213,7 @@ class Engine:
         events = []
         for req in [r for r in self.waiting + self.active if r.cancelled or (r.deadline is not None and now >= r.deadline)]:
             reason = "cancelled" if req.cancelled else "timeout"
+            self.stats["cancelled" if req.cancelled else "timeouts"] += 1
             if req.slot is None:
                 self.waiting.remove(req)
                 req.finish_reason = reason

@@ -313,6 +313,7 @@ def test_a_request_out_of_time_ends_waiting_or_running():
     now[0] += 0.03
     events = eng.step()
     assert (a, None, "timeout") in events and eng.finished[a].finish_reason == "timeout"
+    assert eng.stats["timeouts"] == 2 and eng.stats["cancelled"] == 0
     done = eng.run_until_done()
     assert done[c] == serial(list(range(50, 60)), 5)
     assert eng.free_credits == eng.total_pages and eng.runner.free_slots() == 1
