@@ -15,7 +15,8 @@ import time
 USAGE = """mini-llm (--model DIR | --random-weights CONFIG.json [--seed 0]) --prompt-ids 1,2,3
          [--tokens 32] [--context 2048] [--batch 128] [--chunk 128] [--sequences 4]
          [--dtype bfloat16|float32] [--temperature 0] [--sample-seed 0] [--page-size 16]
-         [--device 0] [--ignore-eos] [--device-time] [--output NEW_REPORT.json]
+         [--device 0] [--device-budget-bytes 0] [--ignore-eos] [--device-time] [--output NEW_REPORT.json]
+         [--cuda-precision f32-pedantic] [--kv-layout paged]
 """
 
 
@@ -25,7 +26,8 @@ def main(argv=None):
     try:
         opts = Options(argv, {"--model", "--random-weights", "--seed", "--prompt-ids", "--tokens", "--context",
                               "--batch", "--chunk", "--sequences", "--dtype", "--temperature", "--sample-seed",
-                              "--page-size", "--device", "--output"},
+                              "--page-size", "--device", "--output", "--device-budget-bytes", "--cuda-precision",
+                              "--kv-layout"},
                        {"--help", "--ignore-eos", "--device-time"})
         if opts.has("--help") or not (opts.has("--model") or opts.has("--random-weights")):
             sys.stdout.write(USAGE)
@@ -45,6 +47,17 @@ def main(argv=None):
         temperature = opts.number("--temperature", 0.0, 0.0, 1e6)
         sample_seed = opts.integer("--sample-seed", 0, 0, 2 ** 63 - 1)
         prompt = opts.integers("--prompt-ids")
+        budget = opts.integer("--device-budget-bytes", 0, 0, 2 ** 63 - 1)
+        # the reference's names for what is a choice of one here (apps/cuda_main.cpp:18-47): its 32-bit mode
+        # is --dtype float32; its FP16-matrix mode and its contiguous cache layout are not built
+        if opts.get("--kv-layout", "paged") != "paged":
+            raise OptionError("--kv-layout: only the paged cache is built")
+        if opts.has("--cuda-precision"):
+            if opts.get("--cuda-precision") != "f32-pedantic":
+                raise OptionError("--cuda-precision: only f32-pedantic (= --dtype float32) is built; "
+                                  "the reduced-precision engine is --dtype bfloat16")
+            if opts.has("--dtype") and opts.get("--dtype") not in ("float32", "fp32"):
+                raise OptionError("--cuda-precision f32-pedantic contradicts --dtype")
 
         import torch
         from .api import parse_dtype
@@ -53,7 +66,7 @@ def main(argv=None):
         from .parts import DecoderModel
         from .sampling import RequestRng, Sampler
         from .weights import write_random_model
-        dtype = parse_dtype(opts.get("--dtype", "bfloat16"))
+        dtype = parse_dtype("float32" if opts.has("--cuda-precision") else opts.get("--dtype", "bfloat16"))
         scratch = None
         if opts.has("--random-weights"):
             with open(opts.get("--random-weights")) as f:
@@ -70,6 +83,14 @@ def main(argv=None):
         if len(prompt) > limit or count - 1 > limit - len(prompt):
             raise OptionError("prompt and the output tokens written to the cache exceed the context")
         pages = sequences * ((limit + page - 1) // page)
+        # the budget gate, before the cache is allocated (src/minillm/cuda/storage.cpp:168-175)
+        element = 4 if dtype == torch.float32 else 2
+        cache_bytes = sum(2 * spec.kv_heads * spec.head_dim * element for spec in model.cache_entry_specs
+                          if hasattr(spec, "kv_heads")) * (pages + 1) * page
+        weight_bytes = model.weight_bytes()
+        if budget and weight_bytes + cache_bytes > budget:
+            raise OptionError(f"weights ({weight_bytes} bytes) and cache ({cache_bytes} bytes) exceed "
+                              f"--device-budget-bytes {budget}")
         runner = Runner(model, max_tokens=pages * page, max_slots=sequences, max_length=limit,
                         max_batch_tokens=batch, page_size=page)
         sampler = Sampler(runner.kernels, runner.device, max_rows=1)
@@ -123,6 +144,7 @@ def main(argv=None):
             "output_tokens_per_second": len(generated) / elapsed if elapsed > 0 else None,
             "limits": {"max_sequences": sequences, "max_model_len": limit, "batch_tokens": batch,
                        "page_size": page},
+            "device_bytes": {"weights": weight_bytes, "cache": runner.cache.kv_bytes(), "budget": budget},
             "used_kv_pages_before_release": pages_before,
             "used_kv_pages_after_release": runner.cache.num_pages - runner.cache.free_pages(),
             "forwards": forwards,

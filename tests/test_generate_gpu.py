@@ -164,12 +164,23 @@ def test_command_line(model_folders, plain_models, tmp_path):
     a = run_cli(["--random-weights", cfg_path, "--seed", "3", "--prompt-ids", "1,2,3", "--tokens", "5"])
     b = run_cli(["--random-weights", cfg_path, "--seed", "3", "--prompt-ids", "1,2,3", "--tokens", "5"])
     assert a.returncode == 0 and json.loads(a.stdout)["token_ids"] == json.loads(b.stdout)["token_ids"]
+    # the reference's names for what is one choice here, and its budget gate
+    c = run_cli(["--model", model_folders["A"], "--prompt-ids", ids, "--tokens", "6", "--cuda-precision", "f32-pedantic",
+                 "--kv-layout", "paged", "--context", "64", "--sequences", "1", "--device-budget-bytes", "100000000"])
+    assert c.returncode == 0, c.stderr
+    rc = json.loads(c.stdout)
+    assert rc["token_ids"] == report["token_ids"] and rc["dtype"] == "float32"
+    assert rc["device_bytes"]["cache"] == 2 * 2 * 2 * 16 * 4 * (4 + 1) * 16      # 2 layers x (k, v) x 2 heads x 16 x float x 5 pages x 16
     # errors: one line on stderr, exit code 1
     for args, text in [(["--model", model_folders["A"], "--prompt-ids", ids, "--output", report_path], "new file"),
                        (["--model", model_folders["A"], "--prompt-ids", "1,2", "--tokens", "0"], "out-of-range"),
                        (["--model", model_folders["A"], "--prompt-ids", "999"], "vocabulary"),
                        (["--model", model_folders["A"], "--prompt-ids", ids, "--context", "15", "--tokens", "4"], "exceed"),
                        (["--model", model_folders["A"], "--bogus"], "unknown option"),
+                       (["--model", model_folders["A"], "--prompt-ids", ids, "--kv-layout", "contiguous"], "paged"),
+                       (["--model", model_folders["A"], "--prompt-ids", ids, "--cuda-precision", "f16-matrix-f32acc"],
+                        "f32-pedantic"),
+                       (["--model", model_folders["A"], "--prompt-ids", ids, "--device-budget-bytes", "1000"], "exceed"),
                        (["--model", str(tmp_path), "--prompt-ids", "1"], "config.json")]:
         bad = run_cli(args)
         assert bad.returncode == 1 and text in bad.stderr, (args, bad.stderr)
