@@ -17,7 +17,38 @@ USAGE = """mini-llm (--model DIR | --random-weights CONFIG.json [--seed 0]) --pr
          [--dtype bfloat16|float32] [--temperature 0] [--sample-seed 0] [--page-size 16]
          [--device 0] [--device-budget-bytes 0] [--ignore-eos] [--device-time] [--output NEW_REPORT.json]
          [--cuda-precision f32-pedantic] [--kv-layout paged]
+mini-llm --model DIR --inspect
 """
+
+
+def inspect(opts):
+    """What the model folder holds, without a GPU: architecture, configuration, files, tensors, and whether
+    the tensors are the ones the architecture expects (apps/mini_main.cpp:54-69 prints the same of its file)."""
+    from .config import load_config
+    from .options import OptionError
+    from .parts.model import expected_tensors
+    from .weights.loader import WeightError, check_names, open_model_folder
+    if not opts.has("--model"):
+        raise OptionError("--inspect needs --model")
+    folder = opts.get("--model")
+    config = load_config(folder)
+    names, files = open_model_folder(folder)
+    found = {name: f.entries[name] for name, f in names.items()}
+    try:
+        check_names(expected_tensors(config), found)
+        problems = None
+    except WeightError as error:
+        problems = str(error)
+    dimensions = config.to_dict()
+    report = {"architecture": (dimensions.get("architectures") or [type(config).__name__])[0], "dimensions": dimensions,
+              "files": [os.path.basename(f.path) for f in files],
+              "bytes": sum(os.path.getsize(f.path) for f in files), "tensors": len(found),
+              "tensor_types": sorted({str(dtype).replace("torch.", "") for dtype, _ in found.values()}),
+              "complete": problems is None, "problems": problems}
+    for f in files:
+        f.close()
+    print(json.dumps(report, indent=2))
+    return 0
 
 
 def main(argv=None):
@@ -28,12 +59,14 @@ def main(argv=None):
                               "--batch", "--chunk", "--sequences", "--dtype", "--temperature", "--sample-seed",
                               "--page-size", "--device", "--output", "--device-budget-bytes", "--cuda-precision",
                               "--kv-layout"},
-                       {"--help", "--ignore-eos", "--device-time"})
+                       {"--help", "--ignore-eos", "--device-time", "--inspect"})
         if opts.has("--help") or not (opts.has("--model") or opts.has("--random-weights")):
             sys.stdout.write(USAGE)
             return 0 if opts.has("--help") else 1
         if opts.has("--model") and opts.has("--random-weights"):
             raise OptionError("give --model or --random-weights, not both")
+        if opts.has("--inspect"):
+            return inspect(opts)
         output = opts.get("--output")
         if opts.has("--output") and (not output or os.path.exists(output)):
             raise OptionError("--output must be a new file")

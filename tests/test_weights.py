@@ -208,3 +208,35 @@ def test_random_mode_is_seeded(tmp_path):
     assert torch.equal(fd.tensor("model.embed_tokens.weight").clone(), fa.tensor("model.embed_tokens.weight").clone())
     for f in (fa, fb, fc, fd):
         f.close()
+
+
+def test_the_command_line_inspects_a_folder_without_a_gpu(tmp_path):
+    """`mini-llm --model DIR --inspect` (the reference's --inspect, apps/mini_main.cpp:54-69): architecture,
+    configuration, files, tensor count, and whether the tensors are the expected ones."""
+    import json
+    import os
+    import subprocess
+    import sys
+    from safetensors.torch import load_file, save_file
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    folder = str(tmp_path / "m")
+    config = config_from_dict(dict(architectures=["Qwen3ForCausalLM"], hidden_size=32, num_hidden_layers=2,
+                                   num_attention_heads=2, num_key_value_heads=1, head_dim=16, intermediate_size=48,
+                                   vocab_size=50, max_position_embeddings=128, rms_norm_eps=1e-6, rope_theta=10000.0,
+                                   tie_word_embeddings=True))
+    write_random_model(folder, config, seed=1)
+
+    def inspect():
+        done = subprocess.run([sys.executable, os.path.join(root, "bin", "mini-llm"), "--model", folder, "--inspect"],
+                              capture_output=True, text=True, timeout=120)
+        assert done.returncode == 0, done.stderr
+        return json.loads(done.stdout)
+    report = inspect()
+    assert report["architecture"] == "Qwen3ForCausalLM" and report["dimensions"]["head_dim"] == 16
+    assert report["tensors"] == 2 + 2 * 11 and report["complete"] and report["files"] == ["model.safetensors"]
+    path = os.path.join(folder, "model.safetensors")
+    tensors = load_file(path)
+    del tensors["model.layers.1.mlp.up_proj.weight"]
+    save_file(tensors, path)
+    report = inspect()
+    assert not report["complete"] and "model.layers.1.mlp.up_proj.weight" in report["problems"]
