@@ -52,6 +52,9 @@ def main():
                     help="profiling aid: run just the decode steps or just the prefill; engine: the scheduler "
                          "over a burst of requests (3 x batch requests of 512 prompt and 128 output tokens, "
                          "batch slots), printed as one line of its own")
+    ap.add_argument("--prefill-graph", type=int, default=1,
+                    help="1: the prefill step may be captured as a graph once its shape has come often enough")
+    ap.add_argument("--prefill-reps", type=int, default=10, help="prefill steps; the fastest but the first counts")
     ap.add_argument("--fill", default="prefill", choices=["prefill", "random"],
                     help="how the requests' caches are filled before the timed steps: by real prefill "
                          "(default) or, as a profiling aid, with random keys and values")
@@ -135,10 +138,11 @@ def main():
 
     def prefill_run():
         runner = Runner(model, max_tokens=PREFILL_TOKENS, max_slots=1, max_length=PREFILL_TOKENS,
-                        max_batch_tokens=PREFILL_TOKENS, page_size=args.page_size)
+                        max_batch_tokens=PREFILL_TOKENS, page_size=args.page_size,
+                        graph_max_tokens=PREFILL_TOKENS if args.prefill_graph else 512)
         ids = torch.randint(0, c.vocab_size, (PREFILL_TOKENS,), generator=g).tolist()
         times = []
-        for i in range(4):
+        for i in range(args.prefill_reps):
             s = runner.open_request()
             torch.cuda.synchronize()
             t0 = time.perf_counter()

@@ -3,8 +3,13 @@
 // (The reference hands its projections to cuBLAS the same way, src/minillm/cuda/matrix.cpp:11-37.)
 //
 // Row-major out[M, N] is the column-major N x M matrix w^T(as stored: K x N, ld K)^T . a(as stored: K x M,
-// ld K).  The library's choice of algorithm for a shape is looked up once and kept; the caller brings the
-// workspace (the same for every call, so that calls on one stream may follow each other without clearing it).
+// ld K).  The algorithm for a shape is chosen once and kept: the library lists its candidates in the order of
+// its own estimate, and the first call of a shape runs each of them on the caller's operands and keeps the
+// fastest (the estimate is off by up to 2x at a few hundred rows and by 5-10 % on some large shapes); only
+// row counts that are likely to come again are timed, see below.  While the stream
+// is being captured nothing can be timed; then the library's first candidate is taken, and the choice is
+// made again by the next call outside a capture.  The caller brings the workspace (the same for every
+// call, so that calls on one stream may follow each other without clearing it).
 #include <hip/hip_runtime.h>
 #include <hipblaslt/hipblaslt.h>
 #include <stdint.h>
@@ -19,6 +24,9 @@ struct Plan {
     hipblasLtMatrixLayout_t a = nullptr, b = nullptr, c = nullptr;
     hipblasLtMatmulAlgo_t algo;
     size_t workspace = 0;
+    bool timed = false;  // the algorithm was chosen by measurement
+    hipblasLtMatmulHeuristicResult_t candidates[16];
+    int found = 0;
 };
 hipblasLtHandle_t g_handle = nullptr;
 std::map<std::tuple<int, int, int, size_t, int>, Plan> g_plans;
@@ -39,22 +47,74 @@ int make_plan(int M, int N, int K, size_t workspace_bytes, int out_float, Plan& 
     const uint64_t ws = workspace_bytes;
     hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &ws, sizeof(ws));
     // the library's candidates in the order of its own estimate; the first whose scratch memory fits
-    constexpr int CANDIDATES = 8;
+    constexpr int CANDIDATES = sizeof(p.candidates) / sizeof(p.candidates[0]);
     hipblasLtMatmulHeuristicResult_t results[CANDIDATES];
     int found = 0;
     const hipblasStatus_t st =
         hipblasLtMatmulAlgoGetHeuristic(g_handle, p.desc, p.a, p.b, p.c, p.c, pref, CANDIDATES, results, &found);
     hipblasLtMatmulPreferenceDestroy(pref);
     if (st != HIPBLAS_STATUS_SUCCESS || found < 1) return -14;
-    int pick = -1;
-    for (int i = 0; i < found && pick < 0; ++i)
-        if (results[i].state == HIPBLAS_STATUS_SUCCESS && results[i].workspaceSize <= workspace_bytes) pick = i;
-    if (pick < 0) return -15;
-    p.algo = results[pick].algo;
-    p.workspace = results[pick].workspaceSize;
+    for (int i = 0; i < found; ++i)
+        if (results[i].state == HIPBLAS_STATUS_SUCCESS && results[i].workspaceSize <= workspace_bytes)
+            p.candidates[p.found++] = results[i];
+    if (p.found < 1) return -15;
+    p.algo = p.candidates[0].algo;
+    p.workspace = p.candidates[0].workspaceSize;
     return 0;
 }
+
+int g_tuning = 1;
+
+// Runs every candidate on the caller's operands (each writes the same product into `out`) and keeps the
+// fastest.  A candidate that fails is passed over.
+void choose_by_time(Plan& p, const void* a, const void* w, void* out, void* workspace, hipStream_t stream) {
+    p.timed = true;
+    if (p.found < 2) return;
+    hipEvent_t t0 = nullptr, t1 = nullptr;
+    if (hipEventCreate(&t0) != hipSuccess || hipEventCreate(&t1) != hipSuccess) {
+        if (t0) (void)hipEventDestroy(t0);
+        return;
+    }
+    const float one = 1.0f, zero = 0.0f;
+    float best = 0.0f;
+    int pick = -1;
+    for (int i = 0; i < p.found; ++i) {
+        const hipblasLtMatmulHeuristicResult_t& c = p.candidates[i];
+        float fastest = 0.0f;
+        bool ok = true;
+        // launches follow each other closely, as in a step: one untimed group, then the faster of two
+        for (int group = 0; group < 3 && ok; ++group) {
+            if (hipEventRecord(t0, stream) != hipSuccess) ok = false;
+            for (int run = 0; run < 8 && ok; ++run)
+                if (hipblasLtMatmul(g_handle, p.desc, &one, w, p.a, a, p.b, &zero, out, p.c, out, p.c, &c.algo,
+                                    workspace, c.workspaceSize, stream) != HIPBLAS_STATUS_SUCCESS)
+                    ok = false;
+            float ms = 0.0f;
+            if (ok && (hipEventRecord(t1, stream) != hipSuccess || hipEventSynchronize(t1) != hipSuccess ||
+                       hipEventElapsedTime(&ms, t0, t1) != hipSuccess))
+                ok = false;
+            if (ok && group > 0 && (fastest == 0.0f || ms < fastest)) fastest = ms;
+        }
+        if (ok && (pick < 0 || fastest < best)) {
+            best = fastest;
+            pick = i;
+        }
+    }
+    (void)hipEventDestroy(t0);
+    (void)hipEventDestroy(t1);
+    (void)hipGetLastError();
+    if (pick >= 0) {
+        p.algo = p.candidates[pick].algo;
+        p.workspace = p.candidates[pick].workspaceSize;
+    }
+}
 }  // namespace
+
+// Whether the first call of a shape times the library's candidates (1, the default) or takes the first (0).
+extern "C" void mlr_library_gemm_tuning(int on) {
+    std::lock_guard<std::mutex> lock(g_mutex);
+    g_tuning = on;
+}
 
 // Returns 0, or a negative number that names the library call that failed (-1: bad sizes, -2: no handle,
 // -10 .. -15: setting up the product, -20: the product itself).
@@ -72,7 +132,14 @@ extern "C" int mlr_library_gemm(const void* a, const void* w, void* out, int M, 
         if (rc != 0) return rc;
         it = g_plans.emplace(key, p).first;
     }
-    const Plan& p = it->second;
+    Plan& p = it->second;
+    // Row counts that come again (few rows: decoding batches are filled up to a few sizes; multiples of 64:
+    // prompt portions) are worth the 16 x 24 launches; a mixed step's odd row count may never return.
+    if (!p.timed && g_tuning && (M <= 64 || M % 64 == 0)) {
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(stream, &capturing) == hipSuccess && capturing == hipStreamCaptureStatusNone)
+            choose_by_time(p, a, w, out, workspace, stream);
+    }
     const float one = 1.0f, zero = 0.0f;
     const hipblasStatus_t st = hipblasLtMatmul(g_handle, p.desc, &one, w, p.a, a, p.b, &zero, out, p.c, out, p.c,
                                                &p.algo, workspace, p.workspace, stream);
