@@ -486,6 +486,266 @@ static int launch_skinny(const void* a, const void* w, void* out, int M, int N, 
     return launch_skinny_as<MT, GATED, 4, false>(a, w, out, M, N, K, out_float, 0, stream);
 }
 
+// Many rows (prompt portions), K a multiple of 64: 32x32 tiles of v_mfma_f32_32x32x16_bf16, the operands
+// staged through LDS in blocks of 64 k, double-buffered: the loads of block i + 1 are asked for before the
+// products of block i and written to the other buffer after them, one barrier per block.
+// A workgroup has WM x WN wavefronts, each TM x TN tiles: it owns BM = 32 WM TM rows and BN = 32 WN TN
+// columns of the output.  The weight is the A operand of the instruction (its rows are output columns),
+// the activation the B operand, so a lane ends up with four consecutive columns n of one row m, as in the
+// kernels above (lane = 32 h + i: A holds row i, k slots 8 h .. 8 h + 7, B column i, the same k slots,
+// C column i, rows 8 j + 4 h + r in register 4 j + r).
+// Rows of a staged block lie 144 bytes apart (128 of data): the eight lanes that the LDS serves in one
+// cycle of a 16-byte read then hit different banks.  Every output element is one sum over k in ascending
+// order whatever M is.  GATED: w = [gate; up] of N rows each; a wavefront's weight tiles alternate between
+// the two, and silu(gate) * up is written (N columns).
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
+#define WIDE_BK 64
+#define WIDE_PITCH (WIDE_BK + 8)
+
+template <int WM, int WN, int TM, int TN>
+struct WideShape {
+    static constexpr int BM = 32 * WM * TM, BN = 32 * WN * TN, THREADS = 64 * WM * WN;
+    static constexpr int ROWS = BM + BN;                          // staged rows per block: weight, then activation
+    static constexpr int PER_THREAD = ROWS * (WIDE_BK / 8) / THREADS;      // 16-byte pieces a thread stages
+    static constexpr size_t lds_bytes = 2 * (size_t)ROWS * WIDE_PITCH * sizeof(__bf16);
+    static_assert(ROWS * (WIDE_BK / 8) % THREADS == 0, "the staged pieces must divide among the threads");
+};
+
+template <int WM, int WN, int TM, int TN, bool OUT_FLOAT, bool GATED>
+__global__ __launch_bounds__(64 * WM * WN) void gemm_wide_kernel(const __bf16* __restrict__ a,
+                                                                 const __bf16* __restrict__ w,
+                                                                 void* __restrict__ out_raw, int M, int N, int K,
+                                                                 int tiles_m, int tiles_n) {
+    using S = WideShape<WM, WN, TM, TN>;
+    constexpr int BM = S::BM, BN = S::BN, THREADS = S::THREADS, ROWS = S::ROWS, PT = S::PER_THREAD;
+    static_assert(!GATED || TN % 2 == 0, "gate and up tiles come in pairs");
+    extern __shared__ __attribute__((aligned(16))) __bf16 wide_lds[];
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int li = lane & 31, h = lane >> 5;
+    const int wm = wave / WN, wn = wave % WN;
+    // Workgroups go to the 8 XCDs in turn; each XCD gets a contiguous range of tiles, and within it
+    // consecutive tiles share their columns, so a strip of the weight is fetched into one L2 once.
+    const int total = tiles_m * tiles_n;
+    int tile = blockIdx.x;
+    if (total % 8 == 0) tile = (tile % 8) * (total / 8) + tile / 8;
+    const int m0 = (tile % tiles_m) * BM, n0 = (tile / tiles_m) * BN;
+    // In the gated case a workgroup's BN staged weight rows are BN / 2 gate rows and BN / 2 up rows of the
+    // same output columns: staged row 32 j + i of wavefront column wn is gate (j even) or up (j odd).
+    constexpr int NOUT = GATED ? BN / 2 : BN;                     // output columns of the workgroup
+    const int c0 = GATED ? (tile / tiles_m) * NOUT : n0;
+
+    // What a thread stages per block: pieces t, t + THREADS, ... of 16 bytes; piece c is row c / 8 of the
+    // staged block (weight rows first), k 8 (c % 8) ..  The first PW pieces of a thread are weight, the
+    // others activation; their places are kept as 32-bit element offsets from the matrices' bases (the host
+    // refuses matrices of 2^31 elements and more), which keeps the loads' addresses out of the registers.
+    constexpr int STEP = THREADS / 8;                             // staged rows between a thread's pieces
+    static_assert(BN % STEP == 0, "a thread's pieces must not straddle weight and activation");
+    constexpr int PW = BN / STEP;
+    uint32_t src[PT];
+    const int dst0 = (t >> 3) * WIDE_PITCH + (t & 7) * 8;
+#pragma unroll
+    for (int i = 0; i < PT; ++i) {
+        const int row = (t >> 3) + STEP * i, kc = (t & 7) * 8;
+        if (i < PW) {
+            int n;
+            if (GATED) {
+                // staged weight row -> (wavefront column, tile j, row in tile); tile pairs (2 p, 2 p + 1) are
+                // gate and up of output columns c0 + wn_ * (TN / 2) * 32 + p * 32 ..
+                const int wn_ = row / (32 * TN), j = (row / 32) % TN, r = row % 32;
+                const int col = c0 + (wn_ * (TN / 2) + j / 2) * 32 + r;
+                n = min(col, N - 1) + (j & 1) * N;
+            } else {
+                n = min(n0 + row, N - 1);
+            }
+            src[i] = (uint32_t)n * (uint32_t)K + kc;
+        } else {
+            src[i] = (uint32_t)min(m0 + row - BN, M - 1) * (uint32_t)K + kc;
+        }
+    }
+    // Two blocks are in flight from memory while a third is multiplied: with one, a compute unit has 64 KB
+    // on its way at any time, and the latency of the loads bounds the whole GPU at about 7 TB/s of operands.
+    bf16x8 stage0[PT], stage1[PT];
+    const int blocks = K / WIDE_BK;
+    auto fetch = [&](int kb, auto which) {                    // (blocks past the end fetch the last one again)
+        const __bf16* wk = w + (size_t)min(kb, blocks - 1) * WIDE_BK;
+        const __bf16* ak = a + (size_t)min(kb, blocks - 1) * WIDE_BK;
+#pragma unroll
+        for (int i = 0; i < PT; ++i) {
+            const bf16x8 v = *reinterpret_cast<const bf16x8*>((i < PW ? wk : ak) + src[i]);
+            if constexpr (decltype(which)::value == 0) stage0[i] = v; else stage1[i] = v;
+        }
+    };
+    auto stash = [&](int buf, auto which) {
+        __bf16* base = wide_lds + (size_t)buf * ROWS * WIDE_PITCH;
+#pragma unroll
+        for (int i = 0; i < PT; ++i) {
+            if constexpr (decltype(which)::value == 0) *reinterpret_cast<bf16x8*>(base + dst0 + i * STEP * WIDE_PITCH) = stage0[i];
+            else *reinterpret_cast<bf16x8*>(base + dst0 + i * STEP * WIDE_PITCH) = stage1[i];
+        }
+    };
+    constexpr std::integral_constant<int, 0> S0{};
+    constexpr std::integral_constant<int, 1> S1{};
+
+    floatx16 acc[TN][TM];
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[j][i][e] = 0.f;
+
+    auto products = [&](int buf) {
+        const __bf16* base = wide_lds + (size_t)buf * ROWS * WIDE_PITCH;
+        const __bf16* wb = base + (wn * TN * 32 + li) * WIDE_PITCH + 8 * h;
+        const __bf16* ab = base + (BN + wm * TM * 32 + li) * WIDE_PITCH + 8 * h;
+#pragma unroll
+        for (int ks = 0; ks < WIDE_BK / 16; ++ks) {
+            bf16x8 wf[TN], af[TM];
+#pragma unroll
+            for (int j = 0; j < TN; ++j) wf[j] = *reinterpret_cast<const bf16x8*>(wb + j * 32 * WIDE_PITCH + 16 * ks);
+#pragma unroll
+            for (int i = 0; i < TM; ++i) af[i] = *reinterpret_cast<const bf16x8*>(ab + i * 32 * WIDE_PITCH + 16 * ks);
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+                    acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[j], af[i], acc[j][i], 0, 0, 0);
+        }
+    };
+
+    fetch(0, S0);
+    fetch(1, S1);
+    stash(0, S0);
+    fetch(2, S0);
+    __syncthreads();
+    // block kb is multiplied out of buffer kb % 2; block kb + 1 goes from stage[(kb + 1) % 2] into the other
+    // buffer, whose readers passed the last barrier; block kb + 3 takes its place in the registers
+    // (two blocks per turn of the loop and no branch inside: the register stages keep their names, and
+    // the compiler counts the loads in flight exactly; with a branch it waits for all of them)
+    int kb = 0;
+#pragma unroll 1
+    for (; kb + 2 <= blocks; kb += 2) {
+        products(0);
+        stash(1, S1);
+        fetch(kb + 3, S1);
+        __syncthreads();
+        products(1);
+        stash(0, S0);
+        fetch(kb + 4, S0);
+        __syncthreads();
+    }
+    if (kb < blocks) products(0);
+
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+        const int m = m0 + (wm * TM + i) * 32 + li;
+        if (m >= M) continue;
+#pragma unroll
+        for (int j = 0; j < (GATED ? TN / 2 : TN); ++j) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int n = (GATED ? c0 + (wn * (TN / 2) + j) * 32 : n0 + (wn * TN + j) * 32) + 8 * q + 4 * h;
+                float y[4];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    if (GATED) {
+                        const float gate = acc[2 * j][i][4 * q + r], up = acc[2 * j + 1][i][4 * q + r];
+                        y[r] = (gate / (1.0f + expf(-gate))) * up;
+                    } else {
+                        y[r] = acc[j][i][4 * q + r];
+                    }
+                }
+                if (OUT_FLOAT) {
+                    float* o = (float*)out_raw + (size_t)m * N + n;
+                    if (n + 3 < N && (N & 3) == 0) *reinterpret_cast<float4*>(o) = float4{y[0], y[1], y[2], y[3]};
+                    else
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) if (n + r < N) o[r] = y[r];
+                } else {
+                    __bf16* o = (__bf16*)out_raw + (size_t)m * N + n;
+                    if (n + 3 < N && (N & 3) == 0) {
+                        typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4_t;
+                        *reinterpret_cast<bf16x4_t*>(o) = bf16x4_t{(__bf16)y[0], (__bf16)y[1], (__bf16)y[2], (__bf16)y[3]};
+                    } else
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) if (n + r < N) o[r] = (__bf16)y[r];
+                }
+            }
+        }
+    }
+}
+
+template <int WM, int WN, int TM, int TN, bool GATED>
+static int launch_wide(const void* a, const void* w, void* out, int M, int N, int K, int out_float,
+                       hipStream_t stream) {
+    using S = WideShape<WM, WN, TM, TN>;
+    const int tiles_m = (M + S::BM - 1) / S::BM;
+    const int tiles_n = GATED ? (N + S::BN / 2 - 1) / (S::BN / 2) : (N + S::BN - 1) / S::BN;
+    if ((long long)tiles_m * tiles_n > 0x7fffffffLL) return -2;
+    if ((unsigned long long)M * K >= (1ull << 31) || (unsigned long long)N * (GATED ? 2 : 1) * K >= (1ull << 31)) return -3;
+#define MLR_WIDE_LAUNCH(OF)                                                                                   \
+    {                                                                                                         \
+        auto* kernel = gemm_wide_kernel<WM, WN, TM, TN, OF, GATED>;                                           \
+        static const hipError_t allowed = hipFuncSetAttribute(                                                \
+            reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)S::lds_bytes); \
+        if (allowed != hipSuccess) return (int)allowed;                                                       \
+        kernel<<<dim3(tiles_m * tiles_n), S::THREADS, S::lds_bytes, stream>>>(                                \
+            (const __bf16*)a, (const __bf16*)w, out, M, N, K, tiles_m, tiles_n);                              \
+    }
+    if (out_float) MLR_WIDE_LAUNCH(true) else MLR_WIDE_LAUNCH(false)
+#undef MLR_WIDE_LAUNCH
+    return (int)hipGetLastError();
+}
+
+// The wide kernel's shapes, largest first: 256 x 256 (8 wavefronts), 128 x 256, 128 x 128 (two workgroups
+// a compute unit), 128 x 64 (rows x columns of the output; 64 x 64 in the gated case, whose last shape stages
+// 64 gate and 64 up rows).  The largest shape that still gives about a workgroup per compute unit wins:
+// measured at 2048 rows, 1.05 PFLOP/s on 24576 x 4096 with the first, 0.93-0.96 on 4096 x 4096 and
+// 4096 x 12288 with the second, 0.48-0.53 on 1024 x 2048 and 1024 x 3072 with the last (the vendor library:
+// 1.44, 1.18 and 0.56-0.64).
+#define WIDE_SHAPES 4
+template <bool GATED>
+static int launch_wide_shape(int shape, const void* a, const void* w, void* out, int M, int N, int K, int out_float,
+                             hipStream_t stream) {
+    switch (shape) {
+        case 0: return launch_wide<2, 4, 4, 2, GATED>(a, w, out, M, N, K, out_float, stream);
+        case 1: return launch_wide<2, 4, 2, 2, GATED>(a, w, out, M, N, K, out_float, stream);
+        case 2: return launch_wide<2, 2, 2, 2, GATED>(a, w, out, M, N, K, out_float, stream);
+        case 3:
+            if constexpr (GATED) return launch_wide<2, 2, 1, 2, true>(a, w, out, M, N, K, out_float, stream);
+            else return launch_wide<2, 2, 2, 1, false>(a, w, out, M, N, K, out_float, stream);
+        default: return -1;
+    }
+}
+
+static int wide_shape_for(int M, int N, bool gated) {
+    static const int rows[WIDE_SHAPES] = {256, 128, 128, 128}, cols[WIDE_SHAPES] = {256, 256, 128, 64};
+    static int units = 0;
+    if (units == 0) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        units = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+                    ? prop.multiProcessorCount : 256;
+    }
+    for (int s = 0; s < WIDE_SHAPES; ++s) {
+        const int bm = (gated && s == 3) ? 64 : rows[s], bn = gated ? (s == 3 ? 64 : cols[s] / 2) : cols[s];
+        const long long tiles = (long long)((M + bm - 1) / bm) * ((N + bn - 1) / bn);
+        if (tiles * 10 >= (long long)units * 7) return s;
+    }
+    return WIDE_SHAPES - 1;
+}
+
+// For tests and measurements: the wide kernel in a given shape (0 .. WIDE_SHAPES - 1; -1: the shape that
+// `mlr_gemm` would take), plain or gated.
+extern "C" int mlr_gemm_wide(const void* a, const void* w, void* out, int M, int N, int K, int out_float,
+                             int shape, int gated, hipStream_t stream) {
+    if (M <= 0 || N <= 0) return 0;
+    if (K <= 0 || K % WIDE_BK != 0 || (gated && out_float)) return -1;
+    if (shape < 0) shape = wide_shape_for(M, N, gated != 0);
+    if (gated) return launch_wide_shape<true>(shape, a, w, out, M, N, K, 0, stream);
+    return launch_wide_shape<false>(shape, a, w, out, M, N, K, out_float, stream);
+}
+
 template <int WM, int WN, int TM, int TN>
 static int launch(const void* a, const void* w, void* out, int M, int N, int K, int out_float,
                   hipStream_t stream) {
@@ -510,13 +770,15 @@ extern "C" int mlr_gemm(const void* a, const void* w, void* out, int M, int N, i
     if (M <= 64 && N >= 16384) return launch<2, 2, 2, 2>(a, w, out, M, N, K, out_float, stream);
     if (M <= 32) return launch_skinny<2, false>(a, w, out, M, N, K, out_float, stream);
     if (M <= 64) return launch_skinny<4, false>(a, w, out, M, N, K, out_float, stream);
+    if (K % WIDE_BK == 0 && (unsigned long long)M * K < (1ull << 31) && (unsigned long long)N * K < (1ull << 31))
+        return launch_wide_shape<false>(wide_shape_for(M, N, false), a, w, out, M, N, K, out_float, stream);
     if (M <= 128) return launch<2, 2, 2, 2>(a, w, out, M, N, K, out_float, stream);  // 64 x 64
     return launch<2, 2, 4, 4>(a, w, out, M, N, K, out_float, stream);                // 128 x 128
 }
 
-// out[M, N] = silu(a . w[0:N]^T) * (a . w[N:2N]^T) for M <= 64 (w is [2N, K]: gate rows, then up rows).
-// Returns 1 when M is too large for this kernel: the caller then runs the projection and the
-// activation separately.
+// out[M, N] = silu(a . w[0:N]^T) * (a . w[N:2N]^T) (w is [2N, K]: gate rows, then up rows): up to 64 rows on
+// the weight-streaming kernels, more on the wide kernel when K is a multiple of 64.  Returns 1 when no kernel
+// here takes the sizes: the caller then runs the projection and the activation separately.
 extern "C" int mlr_gemm_gated_silu(const void* a, const void* w, void* out, int M, int N, int K,
                                    hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
@@ -524,6 +786,8 @@ extern "C" int mlr_gemm_gated_silu(const void* a, const void* w, void* out, int 
     if (M <= 16) return launch_skinny<1, true>(a, w, out, M, N, K, 0, stream);
     if (M <= 32) return launch_skinny<2, true>(a, w, out, M, N, K, 0, stream);
     if (M <= 64) return launch_skinny<4, true>(a, w, out, M, N, K, 0, stream);
+    if (K % WIDE_BK == 0 && (unsigned long long)M * K < (1ull << 31) && 2ull * N * K < (1ull << 31))
+        return launch_wide_shape<true>(wide_shape_for(M, N, true), a, w, out, M, N, K, 0, stream);
     return 1;
 }
 

@@ -188,12 +188,20 @@ class Kernels:
 
     def gated_silu_fused(self, rows, k=None):
         """Whether `gemm_gated_silu` is the path for this many rows and inner size: the bfloat16 engine, where
-        `streams_weight` says so (elsewhere the library's product and a separate activation are faster)."""
+        `streams_weight` says so (elsewhere the library's product and a separate activation are faster), and
+        without the library any number of rows when the inner size is a multiple of 64."""
+        if self.dtype == torch.bfloat16 and not self.library_gemm and k is not None and k % 64 == 0 \
+                and rows * k < 2 ** 31:
+            return True
         return self.streams_weight(rows, k if k is not None else 1 << 30)
 
     def gemm_gated_silu(self, a, w, out):
-        """out[M, N] = silu(a . w[:N]^T) * (a . w[N:]^T), w = [gate; up] stacked, for few rows."""
-        _need(self.dtype == torch.bfloat16 and a.shape[0] <= 64, "gemm_gated_silu: bfloat16 and at most 64 rows")
+        """out[M, N] = silu(a . w[:N]^T) * (a . w[N:]^T), w = [gate; up] stacked: up to 64 rows, or any number
+        when the inner size is a multiple of 64 (the wide kernel's gated form)."""
+        _need(self.dtype == torch.bfloat16, "gemm_gated_silu: bfloat16 only")
+        _need(a.shape[0] <= 64 or (a.shape[1] % 64 == 0 and a.numel() < 2 ** 31 and w.numel() < 2 ** 31),
+              "gemm_gated_silu: more than 64 rows need an inner size that is a multiple of 64 (and matrices "
+              "below 2^31 elements)")
         _tensor(a, "a", self.dtype, ndim=2)
         _tensor(w, "w", self.dtype, ndim=2)
         m, k = a.shape

@@ -118,7 +118,8 @@ def test_silu_mul_and_residual(dtype):
 @pytest.mark.parametrize("mnk", [(7, 19, 33), (5, 37, 131), (1, 311, 80), (16, 64, 64), (17, 130, 100),
                                  (64, 200, 76), (65, 257, 256), (200, 300, 1024), (2, 2048, 1024),
                                  (33, 48, 520), (48, 1000, 264), (8, 6144, 1024), (129, 100, 40),
-                                 (5, 40, 192), (11, 72, 4160), (16, 33, 1024), (9, 130, 3072), (2, 24, 8192), (16, 40, 4096), (40, 96, 4096), (24, 56, 2048)])
+                                 (5, 40, 192), (11, 72, 4160), (16, 33, 1024), (9, 130, 3072), (2, 24, 8192), (16, 40, 4096), (40, 96, 4096), (24, 56, 2048),
+                                 (130, 70, 128), (300, 520, 192), (257, 1030, 64), (1000, 90, 320), (66, 4100, 1024)])
 def test_gemm(dtype, mnk):
     """Odd shapes as in the reference's GEMM test (tests/cuda_unit_tests.cu:207-209)."""
     from mini_llm_runtime_amd.kernels import Kernels
@@ -161,6 +162,74 @@ def test_gemm_rows_do_not_depend_on_the_batch(dtype):
         assert torch.equal(small, full[:64])
     else:
         torch.testing.assert_close(small.float(), full[:64].float(), atol=0.13, rtol=1e-2)   # one bfloat16 step at |x| ~ 16
+
+
+@pytest.mark.parametrize("shape", [0, 1, 2, 3])
+@pytest.mark.parametrize("gated", [False, True])
+@pytest.mark.parametrize("mnk", [(65, 70, 64), (300, 257, 192), (513, 1000, 128), (128, 256, 1024), (1, 5, 320)])
+def test_gemm_wide_every_shape(shape, gated, mnk):
+    """The many-row kernel in each of its workgroup shapes, plain and with the feed-forward's activation
+    in its epilogue, at sizes that fill no tile; and the same bits from every shape (an output element is
+    one chain of matrix-core sums over k, whatever tile it lies in)."""
+    from mini_llm_runtime_amd.kernels.ops import _c_int, _p, _stream
+    m, n, kk = mnk
+    lib = kernels(torch.bfloat16)._lib("gemm")
+    a = rnd((m, kk), torch.bfloat16, 60)
+    w = rnd((2 * n if gated else n, kk), torch.bfloat16, 61, 0.3)
+
+    def run(which, out_dtype):
+        out = torch.full((m, n), float("nan"), dtype=out_dtype, device="cuda")
+        rc = lib.mlr_gemm_wide(_p(a), _p(w), _p(out), _c_int(m), _c_int(n), _c_int(kk),
+                               _c_int(1 if out_dtype == torch.float32 else 0), _c_int(which), _c_int(1 if gated else 0),
+                               _stream())
+        assert rc == 0, rc
+        return out
+    out = run(shape, torch.bfloat16)
+    if gated:
+        g = a.double() @ w.double()[:n].T
+        u = a.double() @ w.double()[n:].T
+        want = g / (1 + torch.exp(-g)) * u
+    else:
+        want = a.double() @ w.double().T
+        torch.testing.assert_close(run(shape, torch.float32).double(), want, atol=1e-4 * math.sqrt(kk), rtol=1e-5)
+    torch.testing.assert_close(out.double(), want, atol=2e-2 * float(want.abs().max()), rtol=2e-2)
+    assert torch.equal(out, run(0, torch.bfloat16))
+    assert torch.equal(out, run(-1, torch.bfloat16))
+
+
+def test_gemm_wide_rows_do_not_depend_on_the_batch():
+    """More than 64 rows with an inner size that is a multiple of 64: the tile shape follows the number of
+    rows, a row's bits do not."""
+    from mini_llm_runtime_amd.kernels import Kernels
+    k = Kernels(torch.bfloat16, library_gemm=False)
+    a = rnd((700, 256), torch.bfloat16, 62)
+    w = rnd((1100, 256), torch.bfloat16, 63)
+
+    def run(lo, hi):
+        out = torch.empty((hi - lo, 1100), dtype=torch.bfloat16, device="cuda")
+        k.gemm(a[lo:hi].contiguous(), w, out)
+        return out
+    full = run(0, 700)
+    for lo, hi in [(0, 65), (100, 400), (630, 700), (1, 699)]:
+        assert torch.equal(run(lo, hi), full[lo:hi])
+
+
+def test_gemm_gated_silu_many_rows():
+    """Without the library the feed-forward's first projection keeps its fused activation at any number
+    of rows (inner size a multiple of 64)."""
+    from mini_llm_runtime_amd.kernels import Kernels
+    k = Kernels(torch.bfloat16, library_gemm=False)
+    assert k.gated_silu_fused(2048, 1024) and not k.gated_silu_fused(2048, 1000)
+    assert not kernels(torch.bfloat16).gated_silu_fused(2048, 1024)
+    m, n, kk = 333, 424, 384
+    a = rnd((m, kk), torch.bfloat16, 64)
+    w = rnd((2 * n, kk), torch.bfloat16, 65, 0.3)
+    out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    k.gemm_gated_silu(a, w, out)
+    g = a.double() @ w.double()[:n].T
+    u = a.double() @ w.double()[n:].T
+    want = g / (1 + torch.exp(-g)) * u
+    torch.testing.assert_close(out.double(), want, atol=2e-2 * float(want.abs().max()), rtol=2e-2)
 
 
 def plain_rope(x, pos, base):
