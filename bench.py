@@ -52,6 +52,8 @@ def main():
                     help="profiling aid: run just the decode steps or just the prefill; engine: the scheduler "
                          "over a burst of requests (3 x batch requests of 512 prompt and 128 output tokens, "
                          "batch slots), printed as one line of its own")
+    ap.add_argument("--library", type=int, default=1,
+                    help="0: every matrix product on the hand-written kernels, none in the vendor library")
     ap.add_argument("--prefill-graph", type=int, default=1,
                     help="1: the prefill step may be captured as a graph once its shape has come often enough")
     ap.add_argument("--prefill-reps", type=int, default=10, help="prefill steps; the fastest but the first counts")
@@ -101,7 +103,7 @@ def main():
         """Fill `batch` requests so that warmup + steps decode steps end at the context length; time `steps`."""
         runner = Runner(model, max_tokens=batch * (-(-args.context // 64) * 64), max_slots=batch,
                         max_length=args.context, max_batch_tokens=max(PREFILL_TOKENS, batch), page_size=args.page_size,
-                        target_workgroups=args.attn_workgroups)
+                        target_workgroups=args.attn_workgroups, library_gemm=bool(args.library))
         sampler = Sampler(runner.kernels, runner.device, max_rows=batch)
         fill = args.context - steps - warmup
         assert fill >= 1
@@ -139,7 +141,8 @@ def main():
     def prefill_run():
         runner = Runner(model, max_tokens=PREFILL_TOKENS, max_slots=1, max_length=PREFILL_TOKENS,
                         max_batch_tokens=PREFILL_TOKENS, page_size=args.page_size,
-                        graph_max_tokens=PREFILL_TOKENS if args.prefill_graph else 512)
+                        graph_max_tokens=PREFILL_TOKENS if args.prefill_graph else 512,
+                        library_gemm=bool(args.library))
         ids = torch.randint(0, c.vocab_size, (PREFILL_TOKENS,), generator=g).tolist()
         times = []
         for i in range(args.prefill_reps):

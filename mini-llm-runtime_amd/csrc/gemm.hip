@@ -598,18 +598,23 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_wide_kernel(const __bf16* _
         const __bf16* base = wide_lds + (size_t)buf * ROWS * WIDE_PITCH;
         const __bf16* wb = base + (wn * TN * 32 + li) * WIDE_PITCH + 8 * h;
         const __bf16* ab = base + (BN + wm * TM * 32 + li) * WIDE_PITCH + 8 * h;
+        // the operands of k step ks + 1 are asked for before the products of step ks
+        bf16x8 wf[2][TN], af[2][TM];
+        auto operands = [&](int ks, int set) {
+#pragma unroll
+            for (int j = 0; j < TN; ++j) wf[set][j] = *reinterpret_cast<const bf16x8*>(wb + j * 32 * WIDE_PITCH + 16 * ks);
+#pragma unroll
+            for (int i = 0; i < TM; ++i) af[set][i] = *reinterpret_cast<const bf16x8*>(ab + i * 32 * WIDE_PITCH + 16 * ks);
+        };
+        operands(0, 0);
 #pragma unroll
         for (int ks = 0; ks < WIDE_BK / 16; ++ks) {
-            bf16x8 wf[TN], af[TM];
-#pragma unroll
-            for (int j = 0; j < TN; ++j) wf[j] = *reinterpret_cast<const bf16x8*>(wb + j * 32 * WIDE_PITCH + 16 * ks);
-#pragma unroll
-            for (int i = 0; i < TM; ++i) af[i] = *reinterpret_cast<const bf16x8*>(ab + i * 32 * WIDE_PITCH + 16 * ks);
+            if (ks + 1 < WIDE_BK / 16) operands(ks + 1, (ks + 1) & 1);
 #pragma unroll
             for (int j = 0; j < TN; ++j)
 #pragma unroll
                 for (int i = 0; i < TM; ++i)
-                    acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[j], af[i], acc[j][i], 0, 0, 0);
+                    acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[ks & 1][j], af[ks & 1][i], acc[j][i], 0, 0, 0);
         }
     };
 

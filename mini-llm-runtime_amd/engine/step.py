@@ -31,13 +31,14 @@ class Entry:
 class Runner:
     def __init__(self, model, max_tokens, max_slots=4, max_length=None, max_batch_tokens=None,
                  page_size=16, split_keys=256, split_max_tokens=256, use_graphs=True, graph_max_batch=256,
-                 target_workgroups=512, graph_max_tokens=512, graph_after=4, max_graphs=64):
+                 target_workgroups=512, graph_max_tokens=512, graph_after=4, max_graphs=64, library_gemm=True):
         self.model = model
         self.dtype, self.device = model.dtype, model.device
         spec = model.spec
         self.max_length = min(max_length or spec.max_positions, spec.max_positions)
         self.max_batch_tokens = max_batch_tokens or self.max_length
-        self.kernels = Kernels(self.dtype)
+        # library_gemm=False: every product on the hand-written kernels (the vendor library takes none)
+        self.kernels = Kernels(self.dtype, library_gemm=library_gemm)
         self.kernels.prepare(model.libraries())
         self.cache = CacheManager(model.cache_entry_specs, self.dtype, self.device, page_size,
                                   max_tokens, max_slots, self.max_length)
