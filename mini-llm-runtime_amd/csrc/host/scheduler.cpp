@@ -4,6 +4,9 @@
 // then by arrival.  Policy mixed: every decoding request first gets one token, then prefilling
 // requests in order get min(budget left, prompt left, chunk) until the budget is spent.
 // Policy prefill_first: decodes run only when nothing is prefilling.
+// portion_step > 1 (ours, not the reference's): a portion that does not end its prompt is cut down to a
+// multiple of portion_step, so that the steps' shapes come again and the step function can replay them
+// as captured graphs; a portion shorter than portion_step stays as it is.
 #include <algorithm>
 #include <cstdint>
 #include <vector>
@@ -31,8 +34,9 @@ int64_t mlr_effective_priority(int priority, int64_t wait_ms, int aging_ms) {
 // policy: 0 mixed, 1 prefill_first.  Writes at most n slices; returns their number, or -1 on
 // bad arguments.
 int mlr_schedule_batch(const MlrScheduleItem* items, int n, int64_t batch_tokens, int64_t prefill_chunk,
-                       int policy, int aging_ms, MlrSlice* out) {
-    if (n < 0 || batch_tokens <= 0 || prefill_chunk <= 0 || aging_ms <= 0 || (policy != 0 && policy != 1))
+                       int policy, int aging_ms, int64_t portion_step, MlrSlice* out) {
+    if (n < 0 || batch_tokens <= 0 || prefill_chunk <= 0 || aging_ms <= 0 || (policy != 0 && policy != 1) ||
+        portion_step < 0)
         return -1;
     std::vector<MlrScheduleItem> prefill, decode;
     for (int i = 0; i < n; ++i) (items[i].prefill_remaining > 0 ? prefill : decode).push_back(items[i]);
@@ -53,8 +57,12 @@ int mlr_schedule_batch(const MlrScheduleItem* items, int n, int64_t batch_tokens
         }
     }
     for (const auto& item : prefill) {
-        const int64_t tokens = std::min({remaining, item.prefill_remaining, prefill_chunk});
+        int64_t tokens = std::min({remaining, item.prefill_remaining, prefill_chunk});
         if (tokens == 0) break;
+        if (portion_step > 1 && tokens < item.prefill_remaining) {
+            const int64_t whole = tokens - tokens % portion_step;
+            if (whole > 0) tokens = whole;                  // (a shorter portion stays: nothing may starve)
+        }
         out[count++] = {item.key, tokens, 1};
         remaining -= tokens;
     }

@@ -25,7 +25,7 @@ struct Plan {
     hipblasLtMatmulAlgo_t algo;
     size_t workspace = 0;
     bool timed = false;  // the algorithm was chosen by measurement
-    hipblasLtMatmulHeuristicResult_t candidates[16];
+    hipblasLtMatmulHeuristicResult_t candidates[8];
     int found = 0;
 };
 hipblasLtHandle_t g_handle = nullptr;
@@ -85,7 +85,7 @@ void choose_by_time(Plan& p, const void* a, const void* w, void* out, void* work
         // launches follow each other closely, as in a step: one untimed group, then the faster of two
         for (int group = 0; group < 3 && ok; ++group) {
             if (hipEventRecord(t0, stream) != hipSuccess) ok = false;
-            for (int run = 0; run < 8 && ok; ++run)
+            for (int run = 0; run < 4 && ok; ++run)
                 if (hipblasLtMatmul(g_handle, p.desc, &one, w, p.a, a, p.b, &zero, out, p.c, out, p.c, &c.algo,
                                     workspace, c.workspaceSize, stream) != HIPBLAS_STATUS_SUCCESS)
                     ok = false;
@@ -134,7 +134,7 @@ extern "C" int mlr_library_gemm(const void* a, const void* w, void* out, int M, 
     }
     Plan& p = it->second;
     // Row counts that come again (few rows: decoding batches are filled up to a few sizes; multiples of 64:
-    // prompt portions) are worth the 16 x 24 launches; a mixed step's odd row count may never return.
+    // prompt portions) are worth the 8 x 12 launches; a mixed step's odd row count may never return.
     if (!p.timed && g_tuning && (M <= 64 || M % 64 == 0)) {
         hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
         if (hipStreamIsCapturing(stream, &capturing) == hipSuccess && capturing == hipStreamCaptureStatusNone)

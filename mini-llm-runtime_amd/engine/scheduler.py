@@ -44,7 +44,7 @@ def _lib():
     lib = build.load("host")
     if not getattr(lib, "_mlr_sched_typed", False):
         lib.mlr_schedule_batch.argtypes = [ctypes.POINTER(_Item), ctypes.c_int, ctypes.c_int64, ctypes.c_int64,
-                                           ctypes.c_int, ctypes.c_int, ctypes.POINTER(_Slice)]
+                                           ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.POINTER(_Slice)]
         lib.mlr_effective_priority.argtypes = [ctypes.c_int, ctypes.c_int64, ctypes.c_int]
         lib.mlr_effective_priority.restype = ctypes.c_int64
         lib._mlr_sched_typed = True
@@ -55,9 +55,10 @@ def effective_priority(priority, wait_ms, aging_ms):
     return _lib().mlr_effective_priority(priority, int(wait_ms), aging_ms)
 
 
-def schedule_batch(items, batch_tokens, prefill_chunk, policy="mixed", aging_ms=250):
+def schedule_batch(items, batch_tokens, prefill_chunk, policy="mixed", aging_ms=250, portion_step=0):
     """items: (key, prefill_remaining, priority, wait_ms, order) each.  Returns the slices
-    [(key, tokens, is_prefill)] of the next batch."""
+    [(key, tokens, is_prefill)] of the next batch.  portion_step > 1: portions that do not end their
+    prompt are multiples of it (the reference has no such thing: 0 gives its decision)."""
     if policy not in POLICIES:
         raise ValueError(f"policy must be one of {sorted(POLICIES)}")
     n = len(items)
@@ -65,9 +66,10 @@ def schedule_batch(items, batch_tokens, prefill_chunk, policy="mixed", aging_ms=
     for i, (key, remaining, priority, wait_ms, order) in enumerate(items):
         arr[i] = _Item(key, remaining, priority, int(wait_ms), order)
     out = (_Slice * max(n, 1))()
-    count = _lib().mlr_schedule_batch(arr, n, batch_tokens, prefill_chunk, POLICIES[policy], aging_ms, out)
+    count = _lib().mlr_schedule_batch(arr, n, batch_tokens, prefill_chunk, POLICIES[policy], aging_ms,
+                                      portion_step, out)
     if count < 0:
-        raise ValueError("batch_tokens, prefill_chunk and aging_ms must be positive")
+        raise ValueError("batch_tokens, prefill_chunk and aging_ms must be positive, portion_step not negative")
     return [(out[i].key, out[i].tokens, bool(out[i].prefill)) for i in range(count)]
 
 
@@ -84,6 +86,9 @@ class EngineOptions:
     admission_reserve_ms: int = 2000
     policy: str = "mixed"
     queue_capacity: int = 65536
+    portion_step: int = 32            # ours: portions that do not end their prompt are multiples of this, so
+                                      # that step shapes come again and are replayed as graphs (0: the
+                                      # reference's exact portions)
 
     def validate(self):
         """src/config.cpp:8-36."""
@@ -99,6 +104,8 @@ class EngineOptions:
             raise ValueError("invalid aging interval")
         if self.policy not in POLICIES:
             raise ValueError(f"policy must be one of {sorted(POLICIES)}")
+        if self.portion_step < 0:
+            raise ValueError("portion_step must not be negative")
 
 
 @dataclass
@@ -278,7 +285,7 @@ class Engine:
         now = self.clock()
         items = [(i, len(r.prompt) - r.processed, r.priority, int((now - r.last_scheduled) * 1000), r.order)
                  for i, r in enumerate(self.active)]
-        slices = schedule_batch(items, o.batch_tokens, o.prefill_chunk, o.policy, o.aging_ms)
+        slices = schedule_batch(items, o.batch_tokens, o.prefill_chunk, o.policy, o.aging_ms, o.portion_step)
         if not slices:
             raise RuntimeError("scheduler made no progress")
         entries, sampled = [], []

@@ -80,18 +80,26 @@ class Runner:
         return tuple((len(e.tokens), tuple(int(w) for w in e.want)) for e in entries)
 
     def _decode_fill(self, entries):
-        """How many rows of the scratch request fill a batch of single tokens (each wanting its logits) up to
-        a size that comes again: every size up to 8, even sizes up to 16, multiples of 4 up to 64, of 8
-        beyond.  So that a server whose requests come and go captures a few dozen graphs, not one for every
-        number of live requests."""
-        n = len(entries)
+        """(rows of the scratch request, where they go) that fill the single tokens of a batch (each wanting
+        its logits) up to a number that comes again: every number up to 8, even ones up to 16, multiples of 4
+        up to 64, of 8 beyond.  So that a server whose requests come and go captures a few dozen graphs, not
+        one for every number of live requests.  A batch of single tokens only gets the rows at its end; a
+        batch whose single tokens come first and prompt portions after them (the scheduler's mixed batches)
+        gets them in front, so that the wanted logits stay one block of rows."""
         if self.cache.scratch_slot is None or not self.use_graphs:
-            return 0
-        if any(len(e.tokens) != 1 or list(e.want) != [0] for e in entries):
-            return 0
+            return 0, False
+        n = 0
+        while n < len(entries) and len(entries[n].tokens) == 1 and list(entries[n].want) == [0]:
+            n += 1
+        mixed = n < len(entries)
+        if n == 0 or (mixed and any(len(e.tokens) == 1 for e in entries[n:])):
+            return 0, False
         step = 1 if n <= 8 else 2 if n <= 16 else 4 if n <= 64 else 8
-        filled = -(-n // step) * step
-        return filled - n if filled <= min(self.graph_max_batch, self.max_batch_tokens) else 0
+        fill = -(-n // step) * step - n
+        total = sum(len(e.tokens) for e in entries) + fill
+        if n + fill > self.graph_max_batch or total > min(self.graph_max_tokens, self.max_batch_tokens):
+            return 0, False
+        return fill, mixed
 
     def _graph_wanted(self, entries, total, sig):
         """Steps are launch-bound unless they bring many tokens.  Steps of single tokens with logits for
@@ -122,7 +130,7 @@ class Runner:
                 return False
         return True
 
-    def _graph_step(self, entries, first, total, sig, fill=0):
+    def _graph_step(self, entries, first, total, sig, fill=0, fill_first=False):
         """The same kernels as any step, launched from a captured graph.  The graph's buffers are fixed:
         token ids, positions and slots live in a vector of their own per shape (the wanted rows and the
         token groups, which depend on the shape only, are written there once), key splits are laid out
@@ -148,17 +156,23 @@ class Runner:
             self._graphs[sig] = self._graphs.pop(sig)        # most recently used last
         meta = state["meta"]
         ids, pos, slot_of, segments = [], [], [], []
+
+        def scratch_rows():                               # rows of the scratch request: token 0 at position 0
+            for _ in range(fill):
+                segments.append((self.cache.scratch_slot, len(ids), 1, 0))
+                ids.append(0)
+                pos.append(0)
+                slot_of.append(self.cache.scratch_slot)
+        if fill_first:
+            scratch_rows()
         for e, p0 in zip(entries, first):
             n = len(e.tokens)
             segments.append((e.slot, len(ids), n, p0))
             ids.extend(int(t) for t in e.tokens)
             pos.extend(range(p0, p0 + n))
             slot_of.extend([e.slot] * n)
-        for _ in range(fill):                             # rows of the scratch request: token 0 at position 0
-            segments.append((self.cache.scratch_slot, len(ids), 1, 0))
-            ids.append(0)
-            pos.append(0)
-            slot_of.append(self.cache.scratch_slot)
+        if not fill_first:
+            scratch_rows()
         state["upload"].send(ids + pos + slot_of, meta)
         if state["graph"] is not None:
             state["graph"].replay()
@@ -230,14 +244,16 @@ class Runner:
         first = self.cache.commit_first(slots, counts)    # raises with nothing changed, else takes the pages
         try:
             sig = self._signature(entries) if self.use_graphs and total <= self.graph_max_tokens else None
-            fill = self._decode_fill(entries) if sig is not None else 0
+            fill, fill_first = self._decode_fill(entries) if sig is not None else (0, False)
             if fill:
-                sig = sig + ((1, (0,)),) * fill
+                sig = ((1, (0,)),) * fill + sig if fill_first else sig + ((1, (0,)),) * fill
             if sig is not None and self._graph_wanted(entries, total + fill, sig):
-                logits = self._graph_step(entries, first, total + fill, sig, fill)
+                logits = self._graph_step(entries, first, total + fill, sig, fill, fill_first)
                 self.cache.retire(slots)
                 self.steps += 1
-                return logits[:len(entries)] if fill else logits
+                if fill and logits is not None:           # the scratch rows' logits are dropped
+                    return logits[fill:] if fill_first else logits[:len(entries)]
+                return logits
             ids, pos, slot_of, rows = [], [], [], []
             segments = []
             for e, p0 in zip(entries, first):

@@ -159,6 +159,58 @@ def test_decode_batches_are_filled_up_to_a_size_that_comes_again(model_folders, 
     assert max_difference(outs[0], outs[1]) <= limit
 
 
+@pytest.mark.parametrize("dtype_name", DTYPES)
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_mixed_batches_fill_their_single_tokens_too(model_folders, plain_models, name, dtype_name):
+    """Eleven, then ten, then nine requests decode beside a portion of 16 tokens of a long prompt, as the
+    scheduler orders a mixed batch (single tokens first): the single tokens are filled up to twelve and to
+    ten with rows of the scratch request, in front, so two shapes are captured where three came.  Every
+    step's logits against the plain ones and against the same steps without graphs."""
+    from mini_llm_runtime_amd.engine import Entry, Runner
+    vocab = TINY[name]["vocab_size"]
+    n = 11
+    reqs = make_requests(vocab, [5 + (7 * i) % 19 + 12 for i in range(n)] + [16 * 13], seed=41)
+    want = plain_logits(plain_models[name], reqs)
+    model = load(model_folders, name, dtype_name)
+    long_id = f"r{n}"
+    outs = []
+    for use_graphs in (True, False):
+        r = Runner(model, max_tokens=n * 64 + 256, max_slots=n + 1, page_size=PAGE_SIZE[name], use_graphs=use_graphs,
+                   graph_after=1)
+        slots, at, got = {}, {}, {}
+        for rid, toks in reqs.items():
+            slots[rid] = r.open_request()
+            if rid == long_id:
+                at[rid] = 0
+                continue
+            at[rid] = len(toks) - 12
+            r.step([Entry(slots[rid], toks[:at[rid]], [])])
+        live = [rid for rid in reqs if rid != long_id]
+        for step in range(12):
+            if step in (4, 8):
+                r.close_request(slots.pop(live.pop()))
+            entries = [Entry(slots[rid], [reqs[rid][at[rid]]], [0]) for rid in live]
+            entries.append(Entry(slots[long_id], reqs[long_id][16 * step:16 * step + 16], [3, 15]))
+            logits = r.step(entries)
+            assert logits.shape[0] == len(live) + 2
+            rows = logits.double().cpu().numpy()
+            for rid, row in zip(live, rows):
+                got[(rid, at[rid])] = row
+                at[rid] += 1
+            got[(long_id, 16 * step + 3)], got[(long_id, 16 * step + 15)] = rows[len(live)], rows[len(live) + 1]
+        compare(got, {k: want[k] for k in got}, dtype_name)
+        if use_graphs:
+            shapes = sorted(len(sig) for sig, st in r._graphs.items() if st["graph"] is not None)
+            assert shapes == [11, 13] and r.graph_failures == 0        # ten and twelve single tokens + the portion
+        for rid in list(slots):
+            r.close_request(slots[rid])
+        r.cache.check()
+        assert r.cache.free_pages() == r.cache.num_pages
+        outs.append(got)
+    limit = 2e-5 if dtype_name == "float32" else 0.03 * max(float(np.abs(v).max()) for v in outs[0].values())
+    assert max_difference(outs[0], outs[1]) <= limit
+
+
 @pytest.mark.parametrize("mode", ["evict", "mismatch"])
 def test_graphs_that_are_dropped_or_do_not_hold(model_folders, plain_models, mode, monkeypatch):
     """With room for one captured shape, two alternating shapes push each other out again and again; and a

@@ -333,3 +333,19 @@ def test_shutdown_ends_queued_and_running_requests():
     assert not eng.has_work() and eng.free_credits == eng.total_pages and eng.runner.free_slots() == 2
     with pytest.raises(RuntimeError):
         eng.submit([1, 2, 3])
+
+
+def test_portions_that_do_not_end_a_prompt_are_multiples_of_the_step():
+    """Ours, not the reference's: with portion_step the shapes of steps come again.  The last portion of a
+    prompt and portions shorter than the step stay as they are, so nothing starves."""
+    items = [(0, 0, 0, 0, 0), (1, 0, 0, 0, 1), (2, 500, 0, 0, 2), (3, 500, 0, 0, 3)]
+    assert schedule_batch(items, 256, 128, portion_step=0) == [(0, 1, False), (1, 1, False), (2, 128, True), (3, 126, True)]
+    assert schedule_batch(items, 256, 128, portion_step=32) == [(0, 1, False), (1, 1, False), (2, 128, True), (3, 96, True)]
+    # the prompt's end is not cut
+    items = [(0, 0, 0, 0, 0), (2, 70, 0, 0, 2), (3, 45, 0, 0, 3)]
+    assert schedule_batch(items, 256, 128, portion_step=32) == [(0, 1, False), (2, 70, True), (3, 45, True)]
+    # less than a step left of the budget: the portion runs all the same
+    items = [(0, 0, 0, 0, 0), (2, 500, 0, 0, 2)]
+    assert schedule_batch(items, 8, 8, portion_step=32) == [(0, 1, False), (2, 7, True)]
+    with pytest.raises(ValueError):
+        schedule_batch(items, 8, 8, portion_step=-1)
