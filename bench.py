@@ -54,6 +54,8 @@ def main():
                          "batch slots), printed as one line of its own")
     ap.add_argument("--library", type=int, default=1,
                     help="0: every matrix product on the hand-written kernels, none in the vendor library")
+    ap.add_argument("--tune", type=int, default=1,
+                    help="0: the vendor library's first candidate for every shape, none timed")
     ap.add_argument("--prefill-graph", type=int, default=1,
                     help="1: the prefill step may be captured as a graph once its shape has come often enough")
     ap.add_argument("--prefill-reps", type=int, default=10, help="prefill steps; the fastest but the first counts")
@@ -73,6 +75,9 @@ def main():
     from mini_llm_runtime_amd.sampling import Sampler
 
     dtype = parse_dtype(args.dtype)
+    if not args.tune:
+        from mini_llm_runtime_amd.kernels import build
+        build.load("library_gemm").mlr_library_gemm_tuning(0)
     tag = "bf16" if dtype == torch.bfloat16 else "fp32"
     FULL_LAYERS, sizes = SIZES[args.size]
     if args.layers <= 0:

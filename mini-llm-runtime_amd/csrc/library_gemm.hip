@@ -67,7 +67,8 @@ int g_tuning = 1;
 
 // Runs every candidate on the caller's operands (each writes the same product into `out`) and keeps the
 // fastest.  A candidate that fails is passed over.
-void choose_by_time(Plan& p, const void* a, const void* w, void* out, void* workspace, hipStream_t stream) {
+void choose_by_time(Plan& p, const void* a, const void* w, void* out, void* workspace, size_t workspace_bytes,
+                    hipStream_t stream) {
     p.timed = true;
     if (p.found < 2) return;
     hipEvent_t t0 = nullptr, t1 = nullptr;
@@ -82,18 +83,23 @@ void choose_by_time(Plan& p, const void* a, const void* w, void* out, void* work
         const hipblasLtMatmulHeuristicResult_t& c = p.candidates[i];
         float fastest = 0.0f;
         bool ok = true;
-        // launches follow each other closely, as in a step: one untimed group, then the faster of two
-        for (int group = 0; group < 3 && ok; ++group) {
-            if (hipEventRecord(t0, stream) != hipSuccess) ok = false;
-            for (int run = 0; run < 4 && ok; ++run)
-                if (hipblasLtMatmul(g_handle, p.desc, &one, w, p.a, a, p.b, &zero, out, p.c, out, p.c, &c.algo,
-                                    workspace, c.workspaceSize, stream) != HIPBLAS_STATUS_SUCCESS)
-                    ok = false;
+        // One untimed run, then the fastest of three, each on cold caches (the workspace, which holds nothing
+        // between calls, is overwritten first: 128 MB push the operands out of the L2 and most of the
+        // last-level cache): in a model a weight is never in a cache when its product starts, and a
+        // candidate that wins on cached operands can lose by a tenth there.
+        for (int run = 0; run < 4 && ok; ++run) {
+            if (run > 0 && workspace_bytes > 0 &&
+                hipMemsetAsync(workspace, 0, workspace_bytes, stream) != hipSuccess)
+                ok = false;
+            if (ok && hipEventRecord(t0, stream) != hipSuccess) ok = false;
+            if (ok && hipblasLtMatmul(g_handle, p.desc, &one, w, p.a, a, p.b, &zero, out, p.c, out, p.c, &c.algo,
+                                      workspace, c.workspaceSize, stream) != HIPBLAS_STATUS_SUCCESS)
+                ok = false;
             float ms = 0.0f;
             if (ok && (hipEventRecord(t1, stream) != hipSuccess || hipEventSynchronize(t1) != hipSuccess ||
                        hipEventElapsedTime(&ms, t0, t1) != hipSuccess))
                 ok = false;
-            if (ok && group > 0 && (fastest == 0.0f || ms < fastest)) fastest = ms;
+            if (ok && run > 0 && (fastest == 0.0f || ms < fastest)) fastest = ms;
         }
         if (ok && (pick < 0 || fastest < best)) {
             best = fastest;
@@ -134,11 +140,11 @@ extern "C" int mlr_library_gemm(const void* a, const void* w, void* out, int M, 
     }
     Plan& p = it->second;
     // Row counts that come again (few rows: decoding batches are filled up to a few sizes; multiples of 64:
-    // prompt portions) are worth the 8 x 12 launches; a mixed step's odd row count may never return.
+    // prompt portions) are worth the 8 x 4 launches; a mixed step's odd row count may never return.
     if (!p.timed && g_tuning && (M <= 64 || M % 64 == 0)) {
         hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
         if (hipStreamIsCapturing(stream, &capturing) == hipSuccess && capturing == hipStreamCaptureStatusNone)
-            choose_by_time(p, a, w, out, workspace, stream);
+            choose_by_time(p, a, w, out, workspace, workspace_bytes, stream);
     }
     const float one = 1.0f, zero = 0.0f;
     const hipblasStatus_t st = hipblasLtMatmul(g_handle, p.desc, &one, w, p.a, a, p.b, &zero, out, p.c, out, p.c,
