@@ -270,7 +270,9 @@ class Kernels:
                _c_int(page_size), _c_int(1 if write_cache else 0), _stream()), "qk_norm_rope_kv")
 
     def attention_partial_numel(self, rows, q_heads, head_dim, max_splits):
-        return rows * q_heads * max_splits * (head_dim + 2)
+        """Floats of scratch memory for the partial results of split attention: per (row, head, split) the
+        unnormalised output, its maximum and its sum (the prompt-portion kernel keeps them 16 bytes apart)."""
+        return rows * q_heads * max_splits * (head_dim + 4)
 
     def paged_attention(self, q, k_pages, v_pages, block_table, slots, positions, out, q_heads,
                         kv_heads, head_dim, page_size, scale, window=None, split_keys=0, max_splits=1,
