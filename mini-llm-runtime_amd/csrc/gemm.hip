@@ -3,8 +3,11 @@
 //
 // Float engine: a plain tiled FMA kernel; every output element is one sequential sum over k,
 // so a row's result does not depend on the other rows of the batch.
-// Bfloat16 engine: MFMA (v_mfma_f32_16x16x32_bf16) tiles staged through LDS; the k order of
-// every output element is fixed as well (no split over k).
+// Bfloat16 engine, three families, each with a fixed k order for every output element (so a row's result
+// does not depend on the rows beside it): up to 64 rows the weight is streamed once straight into
+// v_mfma_f32_16x16x32_bf16 (`gemm_skinny_kernel`, optionally with the residual add and RMSNorm in front
+// or silu(gate) * up behind); more rows with k a multiple of 64 go to `gemm_wide_kernel` (32x32 tiles
+// out of double-buffered LDS blocks); any other k to the plain 16x16-tile kernel `gemm_bf16_kernel`.
 #include "common.h"
 #include <type_traits>
 
