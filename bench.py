@@ -54,6 +54,7 @@ def main():
                          "batch slots), printed as one line of its own")
     ap.add_argument("--library", type=int, default=1,
                     help="0: every matrix product on the hand-written kernels, none in the vendor library")
+    ap.add_argument("--split-keys", type=int, default=256, help="the smallest range of keys of one attention workgroup")
     ap.add_argument("--tune", type=int, default=1,
                     help="0: the vendor library's first candidate for every shape, none timed")
     ap.add_argument("--prefill-graph", type=int, default=1,
@@ -108,7 +109,8 @@ def main():
         """Fill `batch` requests so that warmup + steps decode steps end at the context length; time `steps`."""
         runner = Runner(model, max_tokens=batch * (-(-args.context // 64) * 64), max_slots=batch,
                         max_length=args.context, max_batch_tokens=max(PREFILL_TOKENS, batch), page_size=args.page_size,
-                        target_workgroups=args.attn_workgroups, library_gemm=bool(args.library))
+                        target_workgroups=args.attn_workgroups, library_gemm=bool(args.library),
+                        split_keys=args.split_keys)
         sampler = Sampler(runner.kernels, runner.device, max_rows=batch)
         fill = args.context - steps - warmup
         assert fill >= 1
