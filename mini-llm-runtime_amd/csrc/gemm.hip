@@ -644,41 +644,77 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_wide_kernel(const __bf16* _
     }
     if (kb < blocks) products(0);
 
+    constexpr int TNO = GATED ? TN / 2 : TN;              // 32-column tiles of output per wavefront
+    // this lane's results for tile (i, j), rows 8 q + 4 h .. + 3 of the instruction's C (output columns)
+    auto result = [&](int i, int j, int q, float* y) {
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
-        const int m = m0 + (wm * TM + i) * 32 + li;
-        if (m >= M) continue;
+        for (int r = 0; r < 4; ++r) {
+            if (GATED) {
+                const float gate = acc[2 * j][i][4 * q + r], up = acc[2 * j + 1][i][4 * q + r];
+                y[r] = (gate / (1.0f + expf(-gate))) * up;
+            } else {
+                y[r] = acc[j][i][4 * q + r];
+            }
+        }
+    };
+    const int wave_m0 = m0 + wm * TM * 32, wave_n0 = (GATED ? c0 : n0) + wn * TNO * 32;
+    if constexpr (!OUT_FLOAT) {
+        // bfloat16 results leave through LDS: a lane holds four columns of one row, which would be stores of
+        // 8 bytes to 64 different rows; a piece of LDS of the wavefront's own turns them into rows of 16-byte
+        // pieces, eight lanes a 128-byte line (measured on 2048 x 4096 x 1024: the stores took 8 of 28 us).
+        constexpr int COLS = TNO * 32, OPITCH = COLS + 8, ROWS_W = TM * 32;
+        static_assert((size_t)WM * WN * ROWS_W * OPITCH * sizeof(__bf16) <= S::lds_bytes, "the output tiles must fit the LDS");
+        __syncthreads();                                   // every wavefront has read its last operands
+        __bf16* mine = wide_lds + (size_t)wave * ROWS_W * OPITCH;
+        typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4_t;
 #pragma unroll
-        for (int j = 0; j < (GATED ? TN / 2 : TN); ++j) {
+        for (int i = 0; i < TM; ++i)
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int n = (GATED ? c0 + (wn * (TN / 2) + j) * 32 : n0 + (wn * TN + j) * 32) + 8 * q + 4 * h;
-                float y[4];
+            for (int j = 0; j < TNO; ++j)
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    if (GATED) {
-                        const float gate = acc[2 * j][i][4 * q + r], up = acc[2 * j + 1][i][4 * q + r];
-                        y[r] = (gate / (1.0f + expf(-gate))) * up;
-                    } else {
-                        y[r] = acc[j][i][4 * q + r];
-                    }
+                for (int q = 0; q < 4; ++q) {
+                    float y[4];
+                    result(i, j, q, y);
+                    *reinterpret_cast<bf16x4_t*>(mine + (i * 32 + li) * OPITCH + j * 32 + 8 * q + 4 * h) =
+                        bf16x4_t{(__bf16)y[0], (__bf16)y[1], (__bf16)y[2], (__bf16)y[3]};
                 }
-                if (OUT_FLOAT) {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        constexpr int PIECES = COLS / 8;                   // 16-byte pieces in a row of the wavefront's tile
+        const bool whole_n = (N & 7) == 0;
+#pragma unroll
+        for (int t0 = 0; t0 < ROWS_W * PIECES; t0 += 64) {
+            const int c = t0 + lane, row = c / PIECES, piece = c % PIECES;
+            const int m = wave_m0 + row, n = wave_n0 + 8 * piece;
+            if (m >= M || n >= N) continue;
+            const bf16x8 v = *reinterpret_cast<const bf16x8*>(mine + row * OPITCH + 8 * piece);
+            __bf16* o = (__bf16*)out_raw + (size_t)m * N + n;
+            if (whole_n && n + 8 <= N) {
+                *reinterpret_cast<bf16x8*>(o) = v;
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) if (n + e < N) o[e] = v[e];
+            }
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            const int m = wave_m0 + i * 32 + li;
+            if (m >= M) continue;
+#pragma unroll
+            for (int j = 0; j < TNO; ++j)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int n = wave_n0 + j * 32 + 8 * q + 4 * h;
+                    float y[4];
+                    result(i, j, q, y);
                     float* o = (float*)out_raw + (size_t)m * N + n;
                     if (n + 3 < N && (N & 3) == 0) *reinterpret_cast<float4*>(o) = float4{y[0], y[1], y[2], y[3]};
                     else
 #pragma unroll
                         for (int r = 0; r < 4; ++r) if (n + r < N) o[r] = y[r];
-                } else {
-                    __bf16* o = (__bf16*)out_raw + (size_t)m * N + n;
-                    if (n + 3 < N && (N & 3) == 0) {
-                        typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4_t;
-                        *reinterpret_cast<bf16x4_t*>(o) = bf16x4_t{(__bf16)y[0], (__bf16)y[1], (__bf16)y[2], (__bf16)y[3]};
-                    } else
-#pragma unroll
-                        for (int r = 0; r < 4; ++r) if (n + r < N) o[r] = (__bf16)y[r];
                 }
-            }
         }
     }
 }
