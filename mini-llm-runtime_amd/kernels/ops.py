@@ -190,9 +190,11 @@ class Kernels:
         """Whether `gemm_gated_silu` is the path for this many rows and inner size: the bfloat16 engine, where
         `streams_weight` says so (elsewhere the library's product and a separate activation are faster), and
         without the library any number of rows when the inner size is a multiple of 64."""
-        if self.dtype == torch.bfloat16 and not self.library_gemm and k is not None and k % 64 == 0 \
-                and rows * k < 2 ** 31:
-            return True
+        if self.dtype == torch.bfloat16 and rows > 64 and k is not None and k % 64 == 0 and rows * k < 2 ** 31:
+            # many rows: the wide kernel's gated form.  Beside the library it is the faster way while the inner
+            # size is short (measured against the library's product followed by the activation kernel, at 128
+            # to 2048 rows: 0.58-0.95 of their time at k = 1024, 0.84-1.07 at k = 2048, 1.01-1.40 beyond)
+            return not self.library_gemm or k <= 1024 or (k <= 2048 and rows <= 256)
         return self.streams_weight(rows, k if k is not None else 1 << 30)
 
     def gemm_gated_silu(self, a, w, out):
