@@ -82,3 +82,26 @@ def test_steps_without_wanted_logits_and_unfinished_requests(model_folders, plai
     got = replay(model_folders["A"], "float32", steps, 64, str(tmp_path / "o"), vocab)
     assert sorted(os.listdir(tmp_path / "o")) == ["9.f32"]
     np.testing.assert_allclose(got[("x", 29)], plain_models["A"].logits(toks, [29])[0], atol=2e-4, rtol=2e-4)
+
+
+def test_the_input_digest_knows_the_steps_boundaries(model_folders, tmp_path):
+    """The digest on standard error is the same for the same steps and differs when the same tokens are cut
+    differently (the reference digests its replayed batches with their boundaries,
+    tests/cuda_validation_support.h:81-91)."""
+    vocab = TINY["A"]["vocab_size"]
+    toks = make_requests(vocab, [24], seed=2)["r0"]
+
+    def digest(cuts, label):
+        lines, at = [], 0
+        for i, n in enumerate(cuts):
+            lines.append(json.dumps(dict(step=i, entries=[dict(id="x", tokens=toks[at:at + n], want=[n - 1])], end=[])))
+            at += n
+        cmd = [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", model_folders["A"], "--dtype", "float32",
+               "--out", str(tmp_path / label), "--max-tokens", "64"]
+        done = subprocess.run(cmd, input="\n".join(lines) + "\n", capture_output=True, text=True, timeout=120)
+        assert done.returncode == 0, done.stderr
+        found = [l.split()[-1] for l in done.stderr.splitlines() if l.startswith("[trace_run] input digest")]
+        assert len(found) == 1 and len(found[0]) == 64
+        return found[0]
+    a, b, c = digest([24], "a"), digest([24], "b"), digest([20, 4], "c")
+    assert a == b and a != c
