@@ -180,7 +180,7 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(AttnArgs a) {
 #pragma unroll
             for (int i = 0; i < MAX_DIM_REGS; ++i) {
                 const int d = lane + 64 * i;
-                if (d < D) dst[d] = from_float<elem_t>(den > 0.f ? acc[hh][i] / den : 0.f);
+                if (d < D) dst[d] = from_float<elem_t>(den != 0.f ? acc[hh][i] / den : 0.f);
             }
         }
     }
@@ -231,7 +231,7 @@ __global__ __launch_bounds__(64) void attention_combine_kernel(AttnArgs a) {
 #pragma unroll
     for (int i = 0; i < MAX_DIM_REGS; ++i) {
         const int d = threadIdx.x + 64 * i;
-        if (d < D) a.out[((size_t)m * a.q_heads + head) * D + d] = from_float<elem_t>(den > 0.f ? num[i] / den : 0.f);
+        if (d < D) a.out[((size_t)m * a.q_heads + head) * D + d] = from_float<elem_t>(den != 0.f ? num[i] / den : 0.f);
     }
 }
 
@@ -448,7 +448,10 @@ __global__ __launch_bounds__(256, (NCH <= 4 ? 2 : 1)) void attention_mfma_kernel
     for (int i = 0; i < 2 * NCH; ++i) o[i] = floatx4{0.f, 0.f, 0.f, 0.f};
 
     // this lane's fixed offsets into a key page (row col, channels 8b ..) and a value page (row col, keys 4b ..)
-    const int k_lane = col * D + 8 * b, v_lane = col * P + 4 * b;
+    // (the channel offset 8 b joins the key row only where it lies inside the head: with head_dim 16 the
+    // lane blocks b = 2, 3 have no channels, and col * D + 8 b would reach into the next key's row and, in
+    // the last row of the last page, past the end of the cache)
+    const int k_lane = col * D, v_lane = col * P + 4 * b;
     const bool d_whole = (D & 31) == 0;
     // No branch around a load: a load behind a branch makes the compiler wait for every load in flight.
     // A missing page reads page 0 instead, channels beyond head_dim read channel block 0; both are
@@ -467,7 +470,7 @@ __global__ __launch_bounds__(256, (NCH <= 4 ? 2 : 1)) void attention_mfma_kernel
             const __bf16* vptr = vp_base + pk * D * P + key0 % P + v_lane;
 #pragma unroll
             for (int c = 0; c < NCH; ++c)
-                T.k[j][c] = *reinterpret_cast<const bf16x8*>(kptr + (32 * c + 8 * b < D ? 32 * c : 0));
+                T.k[j][c] = *reinterpret_cast<const bf16x8*>(kptr + (32 * c + 8 * b < D ? 32 * c + 8 * b : 0));
 #pragma unroll
             for (int db = 0; db < 2 * NCH; ++db)
                 T.v[db][j] = *reinterpret_cast<const bf16x4*>(vptr + (size_t)(16 * db < D ? 16 * db : 0) * P);
@@ -588,20 +591,18 @@ __global__ __launch_bounds__(256, (NCH <= 4 ? 2 : 1)) void attention_mfma_kernel
     if (wave == 0) {
         float m_tot = m_run;
         for (int w = 0; w < 3; ++w) m_tot = fmaxf(m_tot, lds[(size_t)w * stride + 16 * D + col]);
-        float l_tot = 0.f;
-        float own = 0.f;
-        if (m_tot > -INFINITY) {
-            own = m_run > -INFINITY ? __builtin_amdgcn_exp2f(m_run - m_tot) : 0.f;
-            l_tot = l_run * own;
-        }
+        // (a wavefront that saw no key has sum 0 and is passed over; one whose keys were all NaN -- a page
+        // that nobody wrote -- has maximum -inf too, but a NaN sum, and must not be: 0 x NaN stays NaN)
+        const float own = m_run > -INFINITY ? __builtin_amdgcn_exp2f(m_run - m_tot) : 0.f;
+        float l_tot = l_run * own;
 #pragma unroll
         for (int db = 0; db < 2 * NCH; ++db) o[db] *= own;
         for (int w = 0; w < 3; ++w) {
             const float* src = lds + (size_t)w * stride;
-            const float mw = src[16 * D + col];
-            if (!(mw > -INFINITY)) continue;
-            const float f = __builtin_amdgcn_exp2f(mw - m_tot);
-            l_tot += src[16 * D + 16 + col] * f;
+            const float mw = src[16 * D + col], lw = src[16 * D + 16 + col];
+            if (lw == 0.f) continue;
+            const float f = mw > -INFINITY ? __builtin_amdgcn_exp2f(mw - m_tot) : 0.f;
+            l_tot += lw * f;
 #pragma unroll
             for (int db = 0; db < 2 * NCH; ++db) {
                 if (16 * db >= D) break;
@@ -629,7 +630,7 @@ __global__ __launch_bounds__(256, (NCH <= 4 ? 2 : 1)) void attention_mfma_kernel
                     if (16 * db >= D) break;
                     bf16x4 w4;
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) w4[r] = (__bf16)(l_tot > 0.f ? o[db][r] / l_tot : 0.f);
+                    for (int r = 0; r < 4; ++r) w4[r] = (__bf16)(l_tot != 0.f ? o[db][r] / l_tot : 0.f);
                     *reinterpret_cast<bf16x4*>(dst + 16 * db + 4 * b) = w4;
                 }
             }
@@ -877,7 +878,7 @@ __device__ __forceinline__ void prefill_group(const AttnArgs& a, const int32_t* 
         if (16 * db >= D) break;
         bf16x4 w4;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) w4[r] = (__bf16)(l_run > 0.f ? o[db][r] / l_run : 0.f);
+        for (int r = 0; r < 4; ++r) w4[r] = (__bf16)(l_run != 0.f ? o[db][r] / l_run : 0.f);
         *reinterpret_cast<bf16x4*>(dst + 16 * db + 4 * b) = w4;
     }
 }
@@ -946,7 +947,7 @@ __global__ __launch_bounds__(64) void attention_combine_groups_kernel(AttnArgs a
 #pragma unroll
         for (int i = 0; i < MAX_DIM_REGS; ++i) {
             const int d = threadIdx.x + 64 * i;
-            if (d < D) a.out[((size_t)m * a.q_heads + head) * D + d] = from_float<elem_t>(den > 0.f ? num[i] / den : 0.f);
+            if (d < D) a.out[((size_t)m * a.q_heads + head) * D + d] = from_float<elem_t>(den != 0.f ? num[i] / den : 0.f);
         }
     }
 }

@@ -385,7 +385,7 @@ __device__ __forceinline__ void tile_group(const TileArgs& a, int grp, int kvh, 
             }
             return;
         }
-        const float inv = l > 0.f ? 1.f / l : 0.f;
+        const float inv = l != 0.f ? 1.f / l : 0.f;      // (a NaN sum must show, not read as "no key")
         __bf16* dst = a.out + ((size_t)(row0 + tok) * a.q_heads + kvh * g + hh) * D;
 #pragma unroll
         for (int db = 0; db < DB; ++db)
@@ -432,7 +432,7 @@ __global__ __launch_bounds__(256) void tiles_combine_kernel(TileArgs a) {
         n0 += w * p[d0];
         n1 += w * p[d1];
     }
-    const float inv = den > 0.f ? 1.f / den : 0.f;
+    const float inv = den != 0.f ? 1.f / den : 0.f;
     __bf16* dst = a.out + ((size_t)m * a.q_heads + head) * D;
     if (lane < D) dst[lane] = (__bf16)(n0 * inv);
     if (lane + 64 < D) dst[lane + 64] = (__bf16)(n1 * inv);
