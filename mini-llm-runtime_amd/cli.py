@@ -1,8 +1,16 @@
 """`mini-llm`: generate from token ids on one MI355X.  Options keep the names and meanings of the
-reference's CLIs (apps/mini_main.cpp:19-83, apps/cuda_main.cpp:18-54) where it has them: the
-prompt runs in portions of --chunk tokens with logits asked for at its last token only, then one
-token per step; the last generated token is never fed back, so the cache must hold
-prompt + tokens - 1 positions.  There is no tokenizer here: the prompt is given as ids.
+reference's CLIs (apps/mini_main.cpp:19-83, apps/cuda_main.cpp:18-54) where it has them.  There is no
+tokenizer here: prompts are given as ids.
+
+Two ways to run:
+
+  * `--prompt-ids 1,2,3`: one sequence straight on the step function, as the reference's CLIs run theirs:
+    the prompt in portions of --chunk tokens with logits asked for at its last token only, then one token
+    per step; the last generated token is never fed back, so the cache must hold prompt + tokens - 1
+    positions.
+  * `--prompts-file FILE` (one comma-separated prompt a line): every prompt becomes a request of the
+    scheduler (`Engine`): admission, portions under the token budget, continuous batching over
+    --sequences slots, --policy mixed or prefill_first.
 """
 from __future__ import annotations
 
@@ -12,25 +20,42 @@ import sys
 import tempfile
 import time
 
-USAGE = """mini-llm (--model DIR | --random-weights CONFIG.json [--seed 0]) --prompt-ids 1,2,3
+from .options import Option, OptionError, parse
+
+USAGE = """mini-llm (--model DIR | --random-weights CONFIG.json [--seed 0]) (--prompt-ids 1,2,3 | --prompts-file FILE)
          [--tokens 32] [--context 2048] [--batch 128] [--chunk 128] [--sequences 4]
          [--dtype bfloat16|float32] [--temperature 0] [--sample-seed 0] [--page-size 16]
-         [--device 0] [--device-budget-bytes 0] [--ignore-eos] [--device-time] [--output NEW_REPORT.json]
+         [--policy mixed|prefill_first] [--device 0] [--device-budget-bytes 0] [--ignore-eos]
+         [--device-time] [--profile] [--check-finite] [--output NEW_REPORT.json]
          [--cuda-precision f32-pedantic] [--kv-layout paged]
 mini-llm --model DIR --inspect
 """
+
+TABLE = [
+    Option("--help", "switch"), Option("--inspect", "switch"), Option("--ignore-eos", "switch"),
+    Option("--device-time", "switch"), Option("--profile", "switch"), Option("--check-finite", "switch"),
+    Option("--model"), Option("--random-weights"), Option("--output"), Option("--prompts-file"),
+    Option("--dtype", default="bfloat16"), Option("--policy", default="mixed"),
+    Option("--cuda-precision"), Option("--kv-layout", default="paged"),
+    Option("--prompt-ids", "ints", default=[]),
+    Option("--seed", "int", 0, 0, 2 ** 63 - 1), Option("--sample-seed", "int", 0, 0, 2 ** 63 - 1),
+    Option("--tokens", "int", 32, 1, 4096), Option("--context", "int", 2048, 1, 2 ** 31 - 1),
+    Option("--batch", "int", 128, 1, 2 ** 20), Option("--chunk", "int", None, 1, 2 ** 20),
+    Option("--sequences", "int", 4, 1, 4096), Option("--page-size", "int", 16, 1, 1024),
+    Option("--device", "int", 0, 0, 2 ** 31 - 1), Option("--device-budget-bytes", "int", 0, 0, 2 ** 63 - 1),
+    Option("--temperature", "float", 0.0, 0.0, 1e6),
+]
 
 
 def inspect(opts):
     """What the model folder holds, without a GPU: architecture, configuration, files, tensors, and whether
     the tensors are the ones the architecture expects (apps/mini_main.cpp:54-69 prints the same of its file)."""
     from .config import load_config
-    from .options import OptionError
     from .parts.model import expected_tensors
     from .weights.loader import WeightError, check_names, open_model_folder
-    if not opts.has("--model"):
+    if not opts.given("--model"):
         raise OptionError("--inspect needs --model")
-    folder = opts.get("--model")
+    folder = opts["--model"]
     config = load_config(folder)
     names, files = open_model_folder(folder)
     found = {name: f.entries[name] for name, f in names.items()}
@@ -51,137 +76,192 @@ def inspect(opts):
     return 0
 
 
+def read_prompts(path, vocab):
+    prompts = []
+    with open(path) as f:
+        for number, line in enumerate(f, 1):
+            line = line.strip()
+            if not line or line.startswith("#"):
+                continue
+            try:
+                ids = [int(piece) for piece in line.split(",")]
+            except ValueError:
+                raise OptionError(f"--prompts-file line {number}: not a comma-separated list of integers") from None
+            if any(t < 0 or t >= vocab for t in ids):
+                raise OptionError(f"--prompts-file line {number}: a token id lies outside the vocabulary")
+            prompts.append(ids)
+    if not prompts:
+        raise OptionError("--prompts-file names no prompt")
+    return prompts
+
+
+def one_sequence(opts, model, runner, sampler, prompt, count, chunk):
+    """The reference CLI's loop (apps/cuda_main.cpp:91-119): portions, then one token per step."""
+    import torch
+    from .engine import Entry
+    from .sampling import RequestRng
+    temperature = opts["--temperature"]
+    rng = RequestRng(opts["--sample-seed"])
+    timing = opts["--device-time"]
+    forwards = []
+
+    def run(entry, phase):
+        t0 = time.perf_counter()
+        if timing:
+            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record()
+        logits = runner.step([entry])
+        token = None
+        if logits is not None:
+            token = sampler.sample(logits, [temperature], [rng.uniform() if temperature > 0 else 0.0])[0]
+        else:
+            torch.cuda.synchronize()
+        if timing:
+            end.record()
+            end.synchronize()
+        forwards.append({"phase": phase, "input_tokens": len(entry.tokens),
+                         "logits_rows": 0 if logits is None else 1,
+                         "host_forward_to_token_ns": int((time.perf_counter() - t0) * 1e9),
+                         "device_elapsed_ms": start.elapsed_time(end) if timing else None})
+        return token
+
+    slot = runner.open_request()
+    started = time.perf_counter()
+    token = None
+    for begin in range(0, len(prompt), chunk):
+        part = prompt[begin:begin + chunk]
+        last = begin + len(part) == len(prompt)
+        token = run(Entry(slot, part, [len(part) - 1] if last else []), "prefill")
+    prefill_s = time.perf_counter() - started
+    generated = []
+    eos = set(model.spec.eos_token_ids)
+    for i in range(count):
+        generated.append(token)
+        stop = token in eos and not opts["--ignore-eos"]
+        if stop or i + 1 == count:
+            break
+        token = run(Entry(slot, [token], [0]), "decode")
+    elapsed = time.perf_counter() - started
+    pages_before = runner.cache.num_pages - runner.cache.free_pages()
+    runner.close_request(slot)
+    return {"input_token_ids": prompt, "token_ids": generated, "prompt_tokens": len(prompt),
+            "completion_tokens": len(generated), "ttft_ms": prefill_s * 1e3, "elapsed_s": elapsed,
+            "output_tokens_per_second": len(generated) / elapsed if elapsed > 0 else None,
+            "used_kv_pages_before_release": pages_before,
+            "used_kv_pages_after_release": runner.cache.num_pages - runner.cache.free_pages(),
+            "forwards": forwards}
+
+
+def many_requests(opts, engine, prompts, count):
+    """Every prompt a request of the scheduler; the report lists them in the order of the file."""
+    started = time.perf_counter()
+    ids = [engine.submit(p, max_tokens=count, temperature=opts["--temperature"], seed=opts["--sample-seed"] + i,
+                         ignore_eos=opts["--ignore-eos"]) for i, p in enumerate(prompts)]
+    first = {}
+    while engine.has_work():
+        for rid, token, _ in engine.step():
+            if token is not None and rid not in first:
+                first[rid] = time.perf_counter() - started
+    elapsed = time.perf_counter() - started
+    requests = [{"input_token_ids": p, "token_ids": list(engine.finished[rid].generated),
+                 "finish_reason": engine.finished[rid].finish_reason, "ttft_ms": first.get(rid, 0.0) * 1e3}
+                for rid, p in zip(ids, prompts)]
+    generated = sum(len(r["token_ids"]) for r in requests)
+    return {"requests": requests, "prompt_tokens": sum(len(p) for p in prompts), "completion_tokens": generated,
+            "elapsed_s": elapsed, "output_tokens_per_second": generated / elapsed if elapsed > 0 else None,
+            "policy": engine.options.policy, "scheduler": dict(engine.stats),
+            "used_kv_pages_after_release": engine.runner.cache.num_pages - engine.runner.cache.free_pages()}
+
+
 def main(argv=None):
-    from .options import OptionError, Options
     argv = sys.argv[1:] if argv is None else argv
     try:
-        opts = Options(argv, {"--model", "--random-weights", "--seed", "--prompt-ids", "--tokens", "--context",
-                              "--batch", "--chunk", "--sequences", "--dtype", "--temperature", "--sample-seed",
-                              "--page-size", "--device", "--output", "--device-budget-bytes", "--cuda-precision",
-                              "--kv-layout"},
-                       {"--help", "--ignore-eos", "--device-time", "--inspect"})
-        if opts.has("--help") or not (opts.has("--model") or opts.has("--random-weights")):
+        opts = parse(argv, TABLE)
+        if opts["--help"] or not (opts.given("--model") or opts.given("--random-weights")):
             sys.stdout.write(USAGE)
-            return 0 if opts.has("--help") else 1
-        if opts.has("--model") and opts.has("--random-weights"):
+            return 0 if opts["--help"] else 1
+        if opts.given("--model") and opts.given("--random-weights"):
             raise OptionError("give --model or --random-weights, not both")
-        if opts.has("--inspect"):
+        if opts["--inspect"]:
             return inspect(opts)
-        output = opts.get("--output")
-        if opts.has("--output") and (not output or os.path.exists(output)):
+        output = opts["--output"]
+        if opts.given("--output") and (not output or os.path.exists(output)):
             raise OptionError("--output must be a new file")
-        context = opts.integer("--context", 2048, 1, 2 ** 31 - 1)
-        batch = opts.integer("--batch", 128, 1, 2 ** 20)
-        chunk = opts.integer("--chunk", batch, 1, batch)
-        sequences = opts.integer("--sequences", 4, 1, 4096)
-        count = opts.integer("--tokens", 32, 1, 4096)
-        page = opts.integer("--page-size", 16, 1, 1024)
-        device = opts.integer("--device", 0, 0, 2 ** 31 - 1)
-        temperature = opts.number("--temperature", 0.0, 0.0, 1e6)
-        sample_seed = opts.integer("--sample-seed", 0, 0, 2 ** 63 - 1)
-        prompt = opts.integers("--prompt-ids")
-        budget = opts.integer("--device-budget-bytes", 0, 0, 2 ** 63 - 1)
+        if opts.given("--prompt-ids") == opts.given("--prompts-file"):
+            raise OptionError("give --prompt-ids or --prompts-file (one of them)")
+        context, batch, sequences = opts["--context"], opts["--batch"], opts["--sequences"]
+        chunk = opts["--chunk"] if opts.given("--chunk") else batch
+        if chunk > batch:
+            raise OptionError(f"--chunk {chunk}: not an integer in 1..{batch} (--batch)")
+        count, page, budget = opts["--tokens"], opts["--page-size"], opts["--device-budget-bytes"]
         # the reference's names for what is a choice of one here (apps/cuda_main.cpp:18-47): its 32-bit mode
         # is --dtype float32; its FP16-matrix mode and its contiguous cache layout are not built
-        if opts.get("--kv-layout", "paged") != "paged":
+        if opts["--kv-layout"] != "paged":
             raise OptionError("--kv-layout: only the paged cache is built")
-        if opts.has("--cuda-precision"):
-            if opts.get("--cuda-precision") != "f32-pedantic":
+        if opts.given("--cuda-precision"):
+            if opts["--cuda-precision"] != "f32-pedantic":
                 raise OptionError("--cuda-precision: only f32-pedantic (= --dtype float32) is built; "
                                   "the reduced-precision engine is --dtype bfloat16")
-            if opts.has("--dtype") and opts.get("--dtype") not in ("float32", "fp32"):
+            if opts.given("--dtype") and opts["--dtype"] not in ("float32", "fp32"):
                 raise OptionError("--cuda-precision f32-pedantic contradicts --dtype")
+        if opts["--policy"] not in ("mixed", "prefill_first"):
+            raise OptionError("--policy: mixed or prefill_first")
 
         import torch
         from .api import parse_dtype
         from .config import config_from_dict
-        from .engine import Entry, Runner
+        from .engine import Engine, EngineOptions, MemoryBudgetError, Runner
         from .parts import DecoderModel
-        from .sampling import RequestRng, Sampler
+        from .sampling import Sampler
         from .weights import write_random_model
-        dtype = parse_dtype("float32" if opts.has("--cuda-precision") else opts.get("--dtype", "bfloat16"))
+        dtype = parse_dtype("float32" if opts.given("--cuda-precision") else opts["--dtype"])
         scratch = None
-        if opts.has("--random-weights"):
-            with open(opts.get("--random-weights")) as f:
+        if opts.given("--random-weights"):
+            with open(opts["--random-weights"]) as f:
                 config = config_from_dict(json.load(f))
             scratch = tempfile.TemporaryDirectory(prefix="mini-llm-random-")
-            folder = write_random_model(scratch.name, config, opts.integer("--seed", 0, 0, 2 ** 63 - 1))
+            folder = write_random_model(scratch.name, config, opts["--seed"])
         else:
-            folder = opts.get("--model")
-        model = DecoderModel.load(folder, dtype, f"cuda:{device}")
+            folder = opts["--model"]
+        try:
+            model = DecoderModel.load(folder, dtype, f"cuda:{opts['--device']}", device_budget_bytes=budget)
+        except MemoryBudgetError as error:
+            raise OptionError(str(error)) from None
         vocab = model.spec.vocab_size
-        if not prompt or any(t < 0 or t >= vocab for t in prompt):
-            raise OptionError("--prompt-ids must name at least one token id inside the vocabulary")
         limit = min(context, model.spec.max_positions)
-        if len(prompt) > limit or count - 1 > limit - len(prompt):
-            raise OptionError("prompt and the output tokens written to the cache exceed the context")
-        pages = sequences * ((limit + page - 1) // page)
-        # the budget gate, before the cache is allocated (src/minillm/cuda/storage.cpp:168-175)
-        element = 4 if dtype == torch.float32 else 2
-        cache_bytes = sum(2 * spec.kv_heads * spec.head_dim * element for spec in model.cache_entry_specs
-                          if hasattr(spec, "kv_heads")) * (pages + 1) * page
-        weight_bytes = model.weight_bytes()
-        if budget and weight_bytes + cache_bytes > budget:
-            raise OptionError(f"weights ({weight_bytes} bytes) and cache ({cache_bytes} bytes) exceed "
-                              f"--device-budget-bytes {budget}")
-        runner = Runner(model, max_tokens=pages * page, max_slots=sequences, max_length=limit,
-                        max_batch_tokens=batch, page_size=page)
-        sampler = Sampler(runner.kernels, runner.device, max_rows=1)
-        rng = RequestRng(sample_seed)
-        timing = opts.has("--device-time")
-        forwards = []
-
-        def run(entry, phase):
-            t0 = time.perf_counter()
-            if timing:
-                start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                start.record()
-            logits = runner.step([entry])
-            token = None
-            if logits is not None:
-                token = sampler.sample(logits, [temperature], [rng.uniform() if temperature > 0 else 0.0])[0]
+        pool = sequences * ((limit + page - 1) // page) * page
+        common = {"backend": "mini-llm-runtime_amd", "dtype": str(dtype).replace("torch.", "")}
+        try:
+            if opts.given("--prompts-file"):
+                prompts = read_prompts(opts["--prompts-file"], vocab)
+                for p in prompts:
+                    if len(p) + count > limit:
+                        raise OptionError("a prompt and its output tokens exceed the context")
+                engine = Engine(model, EngineOptions(
+                    context_tokens=pool, max_model_len=limit, max_active=sequences, batch_tokens=max(batch, sequences),
+                    prefill_chunk=min(chunk, max(batch, sequences)), block_size=page, policy=opts["--policy"]),
+                    device_budget_bytes=budget, check_finite=opts["--check-finite"], profile=opts["--profile"])
+                runner = engine.runner
+                report = many_requests(opts, engine, prompts, count)
             else:
-                torch.cuda.synchronize()
-            if timing:
-                end.record()
-                end.synchronize()
-            forwards.append({"phase": phase, "input_tokens": len(entry.tokens),
-                             "logits_rows": 0 if logits is None else 1,
-                             "host_forward_to_token_ns": int((time.perf_counter() - t0) * 1e9),
-                             "device_elapsed_ms": start.elapsed_time(end) if timing else None})
-            return token
-
-        slot = runner.open_request()
-        started = time.perf_counter()
-        token = None
-        for begin in range(0, len(prompt), chunk):
-            part = prompt[begin:begin + chunk]
-            last = begin + len(part) == len(prompt)
-            token = run(Entry(slot, part, [len(part) - 1] if last else []), "prefill")
-        prefill_s = time.perf_counter() - started
-        generated = []
-        eos = set(model.spec.eos_token_ids)
-        for i in range(count):
-            generated.append(token)
-            stop = token in eos and not opts.has("--ignore-eos")
-            if stop or i + 1 == count:
-                break
-            token = run(Entry(slot, [token], [0]), "decode")
-        elapsed = time.perf_counter() - started
-        pages_before = runner.cache.num_pages - runner.cache.free_pages()
-        runner.close_request(slot)
-        report = {
-            "backend": "mini-llm-runtime_amd", "dtype": str(dtype).replace("torch.", ""),
-            "input_token_ids": prompt, "token_ids": generated, "prompt_tokens": len(prompt),
-            "completion_tokens": len(generated), "ttft_ms": prefill_s * 1e3, "elapsed_s": elapsed,
-            "output_tokens_per_second": len(generated) / elapsed if elapsed > 0 else None,
-            "limits": {"max_sequences": sequences, "max_model_len": limit, "batch_tokens": batch,
-                       "page_size": page},
-            "device_bytes": {"weights": weight_bytes, "cache": runner.cache.kv_bytes(), "budget": budget},
-            "used_kv_pages_before_release": pages_before,
-            "used_kv_pages_after_release": runner.cache.num_pages - runner.cache.free_pages(),
-            "forwards": forwards,
-        }
+                prompt = opts["--prompt-ids"]
+                if not prompt or any(t < 0 or t >= vocab for t in prompt):
+                    raise OptionError("--prompt-ids must name at least one token id inside the vocabulary")
+                if len(prompt) > limit or count - 1 > limit - len(prompt):
+                    raise OptionError("prompt and the output tokens written to the cache exceed the context")
+                runner = Runner(model, max_tokens=pool, max_slots=sequences, max_length=limit, max_batch_tokens=batch,
+                                page_size=page, device_budget_bytes=budget, check_finite=opts["--check-finite"],
+                                profile=opts["--profile"])
+                sampler = Sampler(runner.kernels, runner.device, max_rows=1)
+                report = one_sequence(opts, model, runner, sampler, prompt, count, chunk)
+        except MemoryBudgetError as error:
+            raise OptionError(str(error)) from None
+        report = {**common, **report,
+                  "limits": {"max_sequences": sequences, "max_model_len": limit, "batch_tokens": batch, "page_size": page},
+                  "device_bytes": {"weights": model.weight_bytes(), "cache": runner.cache.kv_bytes(), "budget": budget,
+                                   "plan": runner.memory_plan.as_dict()}}
+        if opts["--profile"]:
+            report["profile"] = runner.profile_report()
         text = json.dumps(report, indent=2)
         if output:
             with open(output, "x") as f:

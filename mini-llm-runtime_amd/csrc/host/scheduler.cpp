@@ -1,14 +1,22 @@
-// The batch-forming decision as a pure function, after the reference's `schedule_batch`
-// (src/scheduler.cpp:11-49): requests that still have prompt tokens to run are "prefill",
-// the others "decode".  Both lists are ordered by aged priority (priority + wait / aging),
-// then by arrival.  Policy mixed: every decoding request first gets one token, then prefilling
-// requests in order get min(budget left, prompt left, chunk) until the budget is spent.
-// Policy prefill_first: decodes run only when nothing is prefilling.
-// portion_step > 1 (ours, not the reference's): a portion that does not end its prompt is cut down to a
-// multiple of portion_step, so that the steps' shapes come again and the step function can replay them
-// as captured graphs; a portion shorter than portion_step stays as it is.
+// Which request brings how many tokens to the next step: a pure function of the running requests.
+//
+// The decision is the reference's (src/scheduler.cpp:11-49, vectors in tests/core_tests.cpp:123-146):
+// a request that still has prompt tokens to run is a prompt, the others decode; rank = aged priority
+// (priority + whole aging intervals waited), higher first, earlier arrival first among equals.  Policy
+// 0 (mixed): every decoding request gets one token, in rank order, while the budget lasts; what is
+// left goes to prompts in rank order, each min(budget left, prompt left, chunk).  Policy 1
+// (prefill_first): as long as any prompt runs, decoding requests get nothing.
+//
+// How it is done here: every request gets one rank in one sorted index array, which is swept twice
+// (single tokens, then portions), so that the slices come out in the order the step function wants
+// them: single tokens in front, portions behind.
+//
+// portion_step > 1 is this engine's own: a portion that does not end its prompt is cut down to a
+// multiple of portion_step, so that step shapes come again and can be replayed as captured graphs; a
+// portion shorter than portion_step stays as it is, so that nothing starves.
 #include <algorithm>
 #include <cstdint>
+#include <numeric>
 #include <vector>
 
 extern "C" {
@@ -28,45 +36,52 @@ struct MlrSlice {
 };
 
 int64_t mlr_effective_priority(int priority, int64_t wait_ms, int aging_ms) {
-    return priority + std::max<int64_t>(0, wait_ms) / aging_ms;
+    const int64_t waited = wait_ms > 0 ? wait_ms : 0;
+    return (int64_t)priority + waited / aging_ms;
 }
 
-// policy: 0 mixed, 1 prefill_first.  Writes at most n slices; returns their number, or -1 on
-// bad arguments.
+// Writes at most n slices; returns their number, or -1 on bad arguments.
 int mlr_schedule_batch(const MlrScheduleItem* items, int n, int64_t batch_tokens, int64_t prefill_chunk,
                        int policy, int aging_ms, int64_t portion_step, MlrSlice* out) {
-    if (n < 0 || batch_tokens <= 0 || prefill_chunk <= 0 || aging_ms <= 0 || (policy != 0 && policy != 1) ||
-        portion_step < 0)
-        return -1;
-    std::vector<MlrScheduleItem> prefill, decode;
-    for (int i = 0; i < n; ++i) (items[i].prefill_remaining > 0 ? prefill : decode).push_back(items[i]);
-    const auto before = [&](const MlrScheduleItem& l, const MlrScheduleItem& r) {
-        const auto lp = mlr_effective_priority(l.priority, l.wait_ms, aging_ms);
-        const auto rp = mlr_effective_priority(r.priority, r.wait_ms, aging_ms);
-        return lp != rp ? lp > rp : l.order < r.order;
-    };
-    std::stable_sort(prefill.begin(), prefill.end(), before);
-    std::stable_sort(decode.begin(), decode.end(), before);
-    int count = 0;
-    int64_t remaining = batch_tokens;
-    if (policy == 0 || prefill.empty()) {
-        for (const auto& item : decode) {
-            if (remaining == 0) break;
-            out[count++] = {item.key, 1, 0};
-            --remaining;
+    const bool arguments_ok = n >= 0 && batch_tokens > 0 && prefill_chunk > 0 && aging_ms > 0 &&
+                              (policy == 0 || policy == 1) && portion_step >= 0;
+    if (!arguments_ok) return -1;
+
+    std::vector<int64_t> rank(n);
+    bool prompts_run = false;
+    for (int i = 0; i < n; ++i) {
+        rank[i] = mlr_effective_priority(items[i].priority, items[i].wait_ms, aging_ms);
+        prompts_run = prompts_run || items[i].prefill_remaining > 0;
+    }
+    std::vector<int> by_rank(n);
+    std::iota(by_rank.begin(), by_rank.end(), 0);
+    std::sort(by_rank.begin(), by_rank.end(), [&](int a, int b) {
+        if (rank[a] != rank[b]) return rank[a] > rank[b];
+        if (items[a].order != items[b].order) return items[a].order < items[b].order;
+        return a < b;
+    });
+
+    int written = 0;
+    int64_t budget = batch_tokens;
+    const bool decoding_runs = policy == 0 || !prompts_run;
+    if (decoding_runs) {
+        for (int i : by_rank) {
+            if (budget == 0) break;
+            if (items[i].prefill_remaining > 0) continue;
+            out[written++] = MlrSlice{items[i].key, 1, 0};
+            budget -= 1;
         }
     }
-    for (const auto& item : prefill) {
-        int64_t tokens = std::min({remaining, item.prefill_remaining, prefill_chunk});
-        if (tokens == 0) break;
-        if (portion_step > 1 && tokens < item.prefill_remaining) {
-            const int64_t whole = tokens - tokens % portion_step;
-            if (whole > 0) tokens = whole;                  // (a shorter portion stays: nothing may starve)
-        }
-        out[count++] = {item.key, tokens, 1};
-        remaining -= tokens;
+    for (int i : by_rank) {
+        const int64_t left = items[i].prefill_remaining;
+        if (left <= 0) continue;
+        if (budget == 0) break;
+        int64_t take = std::min(std::min(budget, prefill_chunk), left);
+        if (portion_step > 1 && take < left && take >= portion_step) take -= take % portion_step;
+        out[written++] = MlrSlice{items[i].key, take, 1};
+        budget -= take;
     }
-    return count;
+    return written;
 }
 
 }  // extern "C"

@@ -1,68 +1,95 @@
-"""Command-line options in the reference's manner (apps/options.h:12-62): names match exactly,
-an option is either a flag or takes one value, an unknown or repeated option is an error, and
-numbers are checked against a range."""
+"""Command-line options, declared once per program as a table and parsed in one pass.
+
+The rules are the reference's (apps/options.h:12-62): a name matches exactly or not at all, an
+option is a switch or takes exactly one value, naming an option twice or naming one the program
+does not have is an error, and a number must lie in its declared range.  Here a program states
+name, kind, default and range in one place (`Option`), and `parse` returns every value already
+converted and checked, so no call site converts or range-checks again.
+"""
 from __future__ import annotations
 
 import math
+import re
+from dataclasses import dataclass
+from typing import Optional, Sequence
+
+_INTEGER = re.compile(r"-?[0-9]+")
 
 
 class OptionError(ValueError):
     pass
 
 
-class Options:
-    def __init__(self, argv, values, flags=("--help",)):
-        self._args = {}
-        values, flags = set(values), set(flags)
-        i = 0
-        while i < len(argv):
-            name = argv[i]
-            if name in self._args:
-                raise OptionError(f"duplicate option: {name}")
-            if name in flags:
-                self._args[name] = "true"
-            elif name in values and i + 1 < len(argv):
-                i += 1
-                self._args[name] = argv[i]
-            else:
-                raise OptionError(f"unknown option or missing value: {name}")
-            i += 1
+@dataclass(frozen=True)
+class Option:
+    name: str                       # as typed, e.g. "--tokens"
+    kind: str = "text"              # "switch", "text", "int", "float" or "ints" (comma-separated integers)
+    default: object = None
+    low: Optional[float] = None     # inclusive range of an "int" or "float"
+    high: Optional[float] = None
 
-    def has(self, key):
-        return key in self._args
+    def convert(self, text):
+        if self.kind == "text":
+            return text
+        if self.kind == "int":
+            if _INTEGER.fullmatch(text):
+                value = int(text)
+                if (self.low is None or value >= self.low) and (self.high is None or value <= self.high):
+                    return value
+            raise OptionError(f"{self.name} {text!r}: not an integer in {self._range()}")
+        if self.kind == "float":
+            try:
+                value = float(text)
+            except ValueError:
+                value = math.nan
+            if math.isfinite(value) and (self.low is None or value >= self.low) and \
+                    (self.high is None or value <= self.high):
+                return value
+            raise OptionError(f"{self.name} {text!r}: not a number in {self._range()}")
+        if self.kind == "ints":
+            pieces = text.split(",") if text else []
+            if all(_INTEGER.fullmatch(piece) for piece in pieces):
+                return [int(piece) for piece in pieces]
+            raise OptionError(f"{self.name} {text!r}: not a comma-separated list of integers")
+        raise OptionError(f"{self.name}: option kind {self.kind!r} is not known")
 
-    def get(self, key, fallback=""):
-        return self._args.get(key, fallback)
+    def _range(self):
+        low = "-inf" if self.low is None else f"{self.low:g}"
+        high = "inf" if self.high is None else f"{self.high:g}"
+        return f"{low}..{high}"
 
-    def integer(self, key, fallback, minimum, maximum):
-        if not self.has(key):
-            return fallback
-        text = self.get(key)
-        try:
-            if text != text.strip() or text.startswith("+"):
-                raise ValueError
-            value = int(text, 10)
-        except ValueError:
-            raise OptionError(f"out-of-range integer: {key}") from None
-        if value < minimum or value > maximum:
-            raise OptionError(f"out-of-range integer: {key}")
-        return value
 
-    def number(self, key, fallback, minimum, maximum):
-        if not self.has(key):
-            return fallback
-        try:
-            value = float(self.get(key))
-        except ValueError:
-            raise OptionError(f"out-of-range number: {key}") from None
-        if not math.isfinite(value) or value < minimum or value > maximum:
-            raise OptionError(f"out-of-range number: {key}")
-        return value
+class Parsed:
+    """The values of a command line: `parsed["--tokens"]` (the default where the option was not typed),
+    `parsed.given("--tokens")` (whether it was typed)."""
 
-    def integers(self, key):
-        """A comma-separated list of integers (token ids)."""
-        text = self.get(key)
-        try:
-            return [int(part, 10) for part in text.split(",")] if text else []
-        except ValueError:
-            raise OptionError(f"not a list of integers: {key}") from None
+    def __init__(self, values, typed):
+        self._values, self._typed = values, typed
+
+    def __getitem__(self, name):
+        return self._values[name]
+
+    def given(self, name):
+        return name in self._typed
+
+
+def parse(argv: Sequence[str], table: Sequence[Option]) -> Parsed:
+    by_name = {option.name: option for option in table}
+    values = {option.name: (False if option.kind == "switch" else option.default) for option in table}
+    typed = set()
+    words = iter(argv)
+    for word in words:
+        option = by_name.get(word)
+        if option is None:
+            raise OptionError(f"{word}: not an option of this program")
+        if word in typed:
+            raise OptionError(f"{word}: given twice")
+        typed.add(word)
+        if option.kind == "switch":
+            values[word] = True
+            continue
+        text = next(words, None)
+        if text is None:
+            raise OptionError(f"{word}: a value must follow")
+        values[word] = option.convert(text)
+    return Parsed(values, typed)

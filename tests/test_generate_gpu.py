@@ -51,6 +51,34 @@ def test_greedy_generation_through_the_python_entry_point(model_folders, plain_m
         assert one == outs[0] == plain_models[name].greedy(prompts[0], 8)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_prefill_first_through_the_engine(model_folders, plain_models, dtype):
+    """Policy prefill_first on the GPU, requests arriving while others decode: decoding requests are left out
+    of the steps that run prompts and resume from an untouched cache; every request gets the plain greedy
+    tokens; pages and slots come back."""
+    import torch
+    from mini_llm_runtime_amd.engine import Engine, EngineOptions
+    from mini_llm_runtime_amd.parts import DecoderModel
+    name = "B"
+    model = DecoderModel.load(model_folders[name], torch.float32 if dtype == "float32" else torch.bfloat16)
+    eng = Engine(model, EngineOptions(context_tokens=512, max_model_len=128, max_active=4, batch_tokens=16,
+                                      prefill_chunk=8, block_size=PAGE_SIZE[name], policy="prefill_first"))
+    prompts = prompts_for(name, (9, 30, 17, 5, 22))
+    ids = [eng.submit(prompts[0], max_tokens=10)]
+    for _ in range(4):
+        eng.step()                                           # the first request decodes already
+    ids += [eng.submit(p, max_tokens=7) for p in prompts[1:3]]
+    for _ in range(3):
+        eng.step()
+    ids += [eng.submit(p, max_tokens=7) for p in prompts[3:]]
+    done = eng.run_until_done()
+    for rid, prompt in zip(ids, prompts):
+        check_greedy(plain_models[name], prompt, done[rid], dtype)
+    assert eng.stats["mixed_batches"] == 0 and eng.stats["batches"] > 10
+    assert eng.runner.cache.free_pages() == eng.total_pages and eng.runner.free_slots() == 4
+    eng.runner.cache.check()
+
+
 def test_many_requests_on_a_pool_that_holds_three(model_folders, plain_models):
     """Thirty requests of every length on a cache of 192 tokens: most of them wait for pages, pages and slots
     are used again and again, portions of prompts run beside decoding requests; every request still gets
@@ -173,10 +201,10 @@ def test_command_line(model_folders, plain_models, tmp_path):
     assert rc["device_bytes"]["cache"] == 2 * 2 * 2 * 16 * 4 * (4 + 1) * 16      # 2 layers x (k, v) x 2 heads x 16 x float x 5 pages x 16
     # errors: one line on stderr, exit code 1
     for args, text in [(["--model", model_folders["A"], "--prompt-ids", ids, "--output", report_path], "new file"),
-                       (["--model", model_folders["A"], "--prompt-ids", "1,2", "--tokens", "0"], "out-of-range"),
+                       (["--model", model_folders["A"], "--prompt-ids", "1,2", "--tokens", "0"], "not an integer in 1..4096"),
                        (["--model", model_folders["A"], "--prompt-ids", "999"], "vocabulary"),
                        (["--model", model_folders["A"], "--prompt-ids", ids, "--context", "15", "--tokens", "4"], "exceed"),
-                       (["--model", model_folders["A"], "--bogus"], "unknown option"),
+                       (["--model", model_folders["A"], "--bogus"], "not an option"),
                        (["--model", model_folders["A"], "--prompt-ids", ids, "--kv-layout", "contiguous"], "paged"),
                        (["--model", model_folders["A"], "--prompt-ids", ids, "--cuda-precision", "f16-matrix-f32acc"],
                         "f32-pedantic"),
@@ -185,3 +213,34 @@ def test_command_line(model_folders, plain_models, tmp_path):
         bad = run_cli(args)
         assert bad.returncode == 1 and text in bad.stderr, (args, bad.stderr)
     assert run_cli(["--help"]).returncode == 0 and run_cli([]).returncode == 1
+
+
+def test_command_line_through_the_scheduler(model_folders, plain_models, tmp_path):
+    """--prompts-file: every line a request of the scheduler (continuous batching over --sequences slots)."""
+    prompts = prompts_for("A", (7, 13, 5, 1, 30, 9))
+    path = str(tmp_path / "prompts.txt")
+    with open(path, "w") as f:
+        f.write("# one prompt a line\n" + "\n".join(",".join(str(t) for t in p) for p in prompts) + "\n")
+    for policy in ("mixed", "prefill_first"):
+        done = run_cli(["--model", model_folders["A"], "--prompts-file", path, "--tokens", "6", "--dtype", "float32",
+                        "--context", "64", "--sequences", "3", "--batch", "16", "--chunk", "8", "--policy", policy,
+                        "--check-finite"])
+        assert done.returncode == 0, done.stderr
+        report = json.loads(done.stdout)
+        assert [r["input_token_ids"] for r in report["requests"]] == prompts
+        for r, p in zip(report["requests"], prompts):
+            assert r["token_ids"] == plain_models["A"].greedy(p, 6) and r["finish_reason"] == "length"
+        assert report["policy"] == policy and report["completion_tokens"] == 36
+        assert (report["scheduler"]["mixed_batches"] > 0) == (policy == "mixed")
+        assert report["scheduler"]["max_batch_sequences"] <= 3 and report["used_kv_pages_after_release"] == 0
+        plan = report["device_bytes"]["plan"]
+        assert plan["kv_pages"] == report["device_bytes"]["cache"] and plan["total"] > plan["weights"] > 0
+    for args, text in [(["--model", model_folders["A"], "--prompts-file", path, "--prompt-ids", "1"], "one of them"),
+                       (["--model", model_folders["A"], "--prompts-file", path, "--policy", "fastest"], "--policy"),
+                       (["--model", model_folders["A"], "--prompts-file", str(tmp_path / "none.txt")], "none.txt"),
+                       (["--model", model_folders["A"], "--prompts-file", path, "--context", "32", "--tokens", "8"],
+                        "exceed"),
+                       (["--model", model_folders["A"], "--prompts-file", path, "--device-budget-bytes", "1000"],
+                        "exceed")]:
+        bad = run_cli(args)
+        assert bad.returncode == 1 and text in bad.stderr, (args, bad.stderr)

@@ -6,7 +6,7 @@ import pytest
 
 from mini_llm_runtime_amd.cache import CacheFull, PageBook
 from mini_llm_runtime_amd.engine import Engine, EngineOptions, effective_priority, schedule_batch
-from mini_llm_runtime_amd.options import OptionError, Options
+from mini_llm_runtime_amd.options import Option, OptionError, parse
 
 
 def test_mixed_budget_and_decode_protection():
@@ -136,6 +136,29 @@ def test_batched_equals_serial():
     assert eng.runner.book.free_slots() == 4
 
 
+def test_prefill_first_leaves_decoding_requests_out_while_prompts_run():
+    """Policy prefill_first through the engine: a request that is decoding gets no token in a step that runs
+    a prompt, goes on later with an untouched history, and serial == batched; everything comes back."""
+    eng, _ = engine(policy="prefill_first", batch_tokens=8, prefill_chunk=8)
+    a = eng.submit([1, 2, 3], max_tokens=7)
+    eng.step()
+    eng.step()                                       # a has its first two tokens
+    b = eng.submit(list(range(40, 60)), max_tokens=3)
+    eng.step()
+    assert eng.runner.batches[-1] == [(1, 8, [])]    # the prompt alone: a sits out
+    c = eng.submit(list(range(70, 79)), max_tokens=2)
+    out = eng.run_until_done()
+    prompts = {a: [1, 2, 3], b: list(range(40, 60)), c: list(range(70, 79))}
+    for rid, n in ((a, 7), (b, 3), (c, 2)):
+        assert out[rid] == serial(prompts[rid], n)
+    for batch in eng.runner.batches:                 # never a decoded token beside a prompt portion
+        kinds = {"decode" if (n == 1 and want == [0]) else "prompt" for _, n, want in batch}
+        assert kinds != {"decode", "prompt"} or all(n == 1 for _, n, _ in batch)
+    assert eng.stats["mixed_batches"] == 0
+    assert eng.free_credits == eng.total_pages and eng.runner.book.free_pages() == eng.total_pages
+    assert eng.runner.book.free_slots() == 4
+
+
 def test_prompt_portions_and_wanted_places():
     eng, _ = engine(batch_tokens=8, prefill_chunk=5)
     eng.submit(list(range(12)), max_tokens=3)
@@ -260,23 +283,30 @@ def test_a_failed_step_stops_the_engine():
 
 # ------------------------------------------------------------------------------- command-line options
 def test_option_parser():
-    """apps/options.h:12-62: exact names, value or flag, duplicates and unknowns are errors."""
-    o = Options(["--model", "m", "--tokens", "8", "--ignore-eos", "--temperature", "0.5", "--prompt-ids", "1,2,3"],
-                {"--model", "--tokens", "--temperature", "--prompt-ids"}, {"--help", "--ignore-eos"})
-    assert o.get("--model") == "m" and o.has("--ignore-eos") and not o.has("--help")
-    assert o.integer("--tokens", 32, 1, 4096) == 8 and o.integer("--chunk", 7, 1, 10) == 7
-    assert o.number("--temperature", 0.0, 0.0, 10.0) == 0.5 and o.integers("--prompt-ids") == [1, 2, 3]
-    for argv in [["--model", "a", "--model", "b"], ["--bogus"], ["--model"], ["--tokens", "8", "extra"]]:
+    """The reference's rules (apps/options.h:12-62): exact names, a switch or one value, an option named twice
+    or unknown is an error, numbers lie in their declared range."""
+    table = [Option("--help", "switch"), Option("--ignore-eos", "switch"), Option("--model"),
+             Option("--tokens", "int", 32, 1, 4096), Option("--chunk", "int", 7, 1, 10),
+             Option("--temperature", "float", 0.0, 0.0, 10.0), Option("--prompt-ids", "ints", [])]
+    o = parse(["--model", "m", "--tokens", "8", "--ignore-eos", "--temperature", "0.5", "--prompt-ids", "1,2,3"], table)
+    assert o["--model"] == "m" and o["--ignore-eos"] is True and o["--help"] is False
+    assert o.given("--tokens") and not o.given("--chunk") and not o.given("--help")
+    assert o["--tokens"] == 8 and o["--chunk"] == 7 and o["--temperature"] == 0.5 and o["--prompt-ids"] == [1, 2, 3]
+    assert parse([], table)["--tokens"] == 32 and parse(["--prompt-ids", ""], table)["--prompt-ids"] == []
+    assert parse(["--model", "--help"], table)["--model"] == "--help"        # a value is whatever follows
+    for argv in [["--model", "a", "--model", "b"], ["--bogus"], ["--model"], ["--tokens", "8", "extra"],
+                 ["--help", "--help"], ["--tok", "8"], ["-model", "a"]]:
         with pytest.raises(OptionError):
-            Options(argv, {"--model", "--tokens"}, {"--help"})
-    for text in ["0", "5000", "8x", "", " 8", "+8", "1e3"]:
+            parse(argv, table)
+    for text in ["0", "5000", "8x", "", " 8", "+8", "1e3", "8.0", "0x10"]:
         with pytest.raises(OptionError):
-            Options(["--tokens", text], {"--tokens"}).integer("--tokens", 32, 1, 4096)
-    for text in ["nan", "inf", "-1", "x"]:
+            parse(["--tokens", text], table)
+    for text in ["nan", "inf", "-1", "x", "10.5", ""]:
         with pytest.raises(OptionError):
-            Options(["--t", text], {"--t"}).number("--t", 0.0, 0.0, 10.0)
-    with pytest.raises(OptionError):
-        Options(["--p", "1,a"], {"--p"}).integers("--p")
+            parse(["--temperature", text], table)
+    for text in ["1,a", "1,,2", "1, 2", ","]:
+        with pytest.raises(OptionError):
+            parse(["--prompt-ids", text], table)
 
 
 def test_cancelled_requests_end_at_the_next_step_and_give_everything_back():
