@@ -211,6 +211,29 @@ class PageBook:
 class CacheManager:
     """Device memory for every cache entry of a model plus the bookkeeping above."""
 
+    @staticmethod
+    def plan(entry_specs, dtype, page_size, max_tokens, max_slots, max_length):
+        """(bytes of pages, of block tables, of state slabs) that a manager with these sizes allocates:
+        per group of equal `KvSpec`s keys and values [entries, pages + 1, kv_heads, page_size, head_dim]
+        and a table [max_slots + 1, ceil(max_length / page_size)] of int32; per `StateSpec` a slab
+        [max_slots, *shape]."""
+        element = torch.empty((), dtype=dtype).element_size()
+        pages = (max_tokens + page_size - 1) // page_size + 1
+        blocks = (max_length + page_size - 1) // page_size
+        groups = {}
+        state = 0
+        for spec in entry_specs:
+            if isinstance(spec, KvSpec):
+                groups[spec] = groups.get(spec, 0) + 1
+            elif isinstance(spec, StateSpec):
+                count = max_slots
+                for extent in spec.shape:
+                    count *= int(extent)
+                state += count * torch.empty((), dtype=spec.dtype).element_size()
+        kv = sum(2 * n * pages * spec.kv_heads * page_size * spec.head_dim * element for spec, n in groups.items())
+        tables = len(groups) * (max_slots + 1) * blocks * 4
+        return kv, tables, state
+
     def __init__(self, entry_specs, dtype, device, page_size, max_tokens, max_slots, max_length):
         if page_size <= 0 or max_tokens <= 0:
             raise CacheError("page_size and max_tokens must be positive")
@@ -263,6 +286,12 @@ class CacheManager:
 
     def kv_bytes(self):
         return sum(t.numel() * t.element_size() for t in self._k + self._v)
+
+    def table_bytes(self):
+        return sum(t.numel() * t.element_size() for t in self._tables)
+
+    def state_bytes(self):
+        return sum(t.numel() * t.element_size() for t in self._states.values())
 
     # -- requests --------------------------------------------------------------------------------
     def acquire_slot(self):

@@ -207,6 +207,38 @@ __global__ void silu_mul_kernel(const elem_t* __restrict__ gate_up, elem_t* __re
     }
 }
 
+// The check of the hidden state (a debug mode; the reference runs the like after every layer and poisons
+// its runtime, src/minillm/cuda/layer.cpp:71, src/minillm/cuda/ops.cu:29-43).  status[0] collects bits
+// (1: a NaN, 2: an infinity), status[1] the smallest (layer << 20 | row) at which one was seen.
+__global__ void status_reset_kernel(int32_t* __restrict__ status) {
+    if (threadIdx.x == 0) {
+        status[0] = 0;
+        status[1] = 0x7fffffff;
+    }
+}
+
+// One workgroup per row of x = h + delta (delta may be null): which kinds of non-finite values it holds.
+__global__ void finite_check_kernel(const float* __restrict__ h, const elem_t* __restrict__ delta, int width, int layer,
+                                    int32_t* __restrict__ status) {
+    const int r = blockIdx.x;
+    const float* hrow = h + (size_t)r * width;
+    const elem_t* drow = delta ? delta + (size_t)r * width : nullptr;
+    int bits = 0;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) {
+        const float x = hrow[i] + (drow ? to_float(drow[i]) : 0.f);
+        const uint32_t u = __float_as_uint(x) & 0x7fffffffu;
+        if (u > 0x7f800000u) bits |= 1;
+        else if (u == 0x7f800000u) bits |= 2;
+    }
+    if (__any(bits != 0)) {                     // (rare: one atomic per wavefront that saw something)
+        for (int off = 32; off > 0; off >>= 1) bits |= __shfl_xor(bits, off, MLR_WAVE);
+        if ((threadIdx.x & 63) == 0) {
+            atomicOr(&status[0], bits);
+            atomicMin(&status[1], (layer << 20) | (r < (1 << 20) ? r : (1 << 20) - 1));
+        }
+    }
+}
+
 static int grid_for(size_t count, int block) {
     size_t g = (count + block - 1) / block;
     return (int)(g > 65535 ? 65535 : (g == 0 ? 1 : g));
@@ -237,6 +269,19 @@ int mlr_add_rmsnorm(float* h, const void* delta, const float* weight, void* out,
     }
     add_rmsnorm_kernel<<<n_out, 256, 0, stream>>>(h, (const elem_t*)delta, weight, (elem_t*)out, rows,
                                                   width, eps, write_h);
+    return (int)hipGetLastError();
+}
+
+int mlr_status_reset(int32_t* status, hipStream_t stream) {
+    status_reset_kernel<<<1, 64, 0, stream>>>(status);
+    return (int)hipGetLastError();
+}
+
+int mlr_finite_check(const float* h, const void* delta, int rows, int width, int layer, int32_t* status,
+                     hipStream_t stream) {
+    if (rows <= 0) return 0;
+    if (layer < 0 || layer >= 2047) return -1;
+    finite_check_kernel<<<rows, 256, 0, stream>>>(h, (const elem_t*)delta, width, layer, status);
     return (int)hipGetLastError();
 }
 

@@ -1,6 +1,8 @@
 from .context import StepContext, Uploader, Workspace
+from .memory import MemoryBudgetError, MemoryPlan, device_budget
 from .scheduler import Engine, EngineOptions, Request, effective_priority, schedule_batch
-from .step import Entry, Runner, StepError
+from .step import Entry, NonFiniteHidden, Runner, StepError
 
 __all__ = ["StepContext", "Workspace", "Engine", "EngineOptions", "Request", "effective_priority",
-           "schedule_batch", "Entry", "Runner", "StepError"]
+           "schedule_batch", "Entry", "Runner", "StepError", "NonFiniteHidden", "MemoryBudgetError", "MemoryPlan",
+           "device_budget"]

@@ -5,13 +5,36 @@ import torch
 
 
 class Workspace:
-    """Named scratch buffers that live as long as the runner: a buffer is allocated when a name
-    is first asked for and grows only when a larger size is asked, so steady steps allocate
-    nothing."""
+    """Named scratch buffers that live as long as the runner.  `reserve` carves every buffer that the
+    parts have named for the largest step out of ONE allocation; a name that was not planned (a part
+    without a plan), or a size beyond its plan, is allocated when it is first asked for and grows only
+    when a larger size is asked, so steady steps allocate nothing either way."""
 
     def __init__(self, device):
         self.device = torch.device(device)
         self._buffers = {}
+        self._arena = None
+        self.planned_bytes = 0
+        self._unplanned = {}          # (name, dtype) -> bytes allocated outside the plan
+
+    @staticmethod
+    def plan_bytes(plan):
+        """plan: {(name, dtype): elements}.  Bytes of the one allocation that holds them (256-byte places)."""
+        return sum(-(-count * torch.empty((), dtype=dtype).element_size() // 256) * 256
+                   for (_, dtype), count in plan.items())
+
+    def reserve(self, plan):
+        total = self.plan_bytes(plan)
+        self._arena = torch.empty(max(total, 1), dtype=torch.uint8, device=self.device)
+        self.planned_bytes = total
+        at = 0
+        for (name, dtype), count in plan.items():
+            size = count * torch.empty((), dtype=dtype).element_size()
+            self._buffers[(name, dtype)] = self._arena[at:at + size].view(dtype)
+            at += -(-size // 256) * 256
+
+    def unplanned_bytes(self):
+        return sum(self._unplanned.values())
 
     def get(self, name, shape, dtype):
         count = 1
@@ -22,23 +45,11 @@ class Workspace:
         if buf is None or buf.numel() < count:
             buf = torch.empty(max(count, 1), dtype=dtype, device=self.device)
             self._buffers[key] = buf
-        return buf[:count].view(shape)
-
-    def get_zeroed(self, name, shape, dtype):
-        """As `get`, for buffers whose users leave them zero after use (counters): the memory is zeroed
-        when it is allocated, never afterwards."""
-        count = 1
-        for extent in shape:
-            count *= int(extent)
-        key = (name, dtype)
-        buf = self._buffers.get(key)
-        if buf is None or buf.numel() < count:
-            buf = torch.zeros(max(count, 1), dtype=dtype, device=self.device)
-            self._buffers[key] = buf
+            self._unplanned[key] = buf.numel() * buf.element_size()
         return buf[:count].view(shape)
 
     def bytes(self):
-        return sum(b.numel() * b.element_size() for b in self._buffers.values())
+        return self.planned_bytes + self.unplanned_bytes()
 
     def buffers(self):
         """The buffers as they are now.  A captured graph holds on to this list: it keeps using the
@@ -92,6 +103,7 @@ class StepContext:
         self._groups = {}
         self._group_upload = None
         self.fixed_groups = None      # a captured step's groups: {key: token_groups' result}, in tensors of their own
+        self.status = None            # device int32 [2] when the hidden state is to be checked after every layer
 
     def begin_step(self):
         self._groups = {}
@@ -138,17 +150,19 @@ class StepContext:
         self._groups[key] = hit
         return hit
 
-    def attention_split(self, rows, batch_rows, kv_heads, q_heads, head_dim):
+    def attention_split(self, rows, batch_rows, kv_heads, q_heads, head_dim, longest=None):
         """(split_keys, max_splits, partial buffer).  A batch of many tokens fills the GPU with one
         workgroup per (token group, kv head); a small batch over long contexts does not, so there the
         keys of a token are split over several workgroups, in ranges [s * split_keys, (s + 1) *
         split_keys) of absolute key positions, and merged in ascending order.  split_keys is the
         largest of base, 2 base, 4 base, ... that still gives `target_workgroups`; what a token's
         result is does not depend on the choice beyond rounding.  `rows` tokens take part; the partial
-        results are indexed by batch row, of which there are `batch_rows`."""
-        if rows > self.split_max_tokens:
+        results are indexed by batch row, of which there are `batch_rows`.  `longest`: the most keys a
+        workgroup of the kernel can walk without a split; a longer context is split whatever the batch."""
+        forced = longest is not None and self.max_context > longest
+        if rows > self.split_max_tokens and not forced:
             return 0, 1, None
-        return self._split(max(1, rows * kv_heads), self.target_workgroups, batch_rows, q_heads, head_dim)
+        return self._split(max(1, rows * kv_heads), self.target_workgroups, batch_rows, q_heads, head_dim, longest)
 
     def group_split(self, groups, batch_rows, kv_heads, q_heads, head_dim, longest=None):
         """As `attention_split` for `groups` groups of many tokens each (prompt portions), which give

@@ -134,14 +134,21 @@ class Request:
 class Engine:
     """Continuous batching over one `Runner`.  Single-threaded: the caller drives `step()`."""
 
-    def __init__(self, model, options: EngineOptions = None, clock=time.monotonic, runner=None, sampler=None):
+    def __init__(self, model, options: EngineOptions = None, clock=time.monotonic, runner=None, sampler=None,
+                 device_budget_bytes=None, check_finite=False, profile=False):
+        """`device_budget_bytes`, `check_finite`, `profile`: handed to the `Runner` that is built here (see
+        there): the budget gate before the cache is allocated, the check of the hidden state after every
+        layer, time per kernel class."""
         self.options = options or EngineOptions()
         self.options.validate()
         o = self.options
         self.model = model
+        # (a step of the scheduler asks for at most one row of logits per request)
         self.runner = runner or Runner(model, max_tokens=o.context_tokens, max_slots=o.max_active,
                                        max_length=min(o.max_model_len, model.spec.max_positions),
-                                       max_batch_tokens=o.batch_tokens, page_size=o.block_size)
+                                       max_batch_tokens=o.batch_tokens, page_size=o.block_size,
+                                       max_logits_rows=o.max_active, device_budget_bytes=device_budget_bytes,
+                                       check_finite=check_finite, profile=profile)
         self.sampler = sampler or Sampler(self.runner.kernels, self.runner.device, max_rows=o.max_active)
         self.clock = clock
         self.total_pages = o.context_tokens // o.block_size

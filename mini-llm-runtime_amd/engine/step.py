@@ -14,11 +14,18 @@ import torch
 
 from ..cache.manager import CacheManager
 from ..kernels import Kernels
+from ..kernels.ops import LIBRARY_GEMM_WORKSPACE
+from ..kernels.profile import Profiler
 from .context import StepContext, Uploader, Workspace
+from .memory import MemoryPlan
 
 
 class StepError(ValueError):
     """The batch was refused before anything was changed."""
+
+
+class NonFiniteHidden(RuntimeError):
+    """The hidden state held a NaN or an infinity after some layer (check_finite); the runner is poisoned."""
 
 
 @dataclass
@@ -31,7 +38,16 @@ class Entry:
 class Runner:
     def __init__(self, model, max_tokens, max_slots=4, max_length=None, max_batch_tokens=None,
                  page_size=16, split_keys=256, split_max_tokens=256, use_graphs=True, graph_max_batch=256,
-                 target_workgroups=512, graph_max_tokens=512, graph_after=4, max_graphs=64, library_gemm=True):
+                 target_workgroups=512, graph_max_tokens=512, graph_after=4, max_graphs=64, library_gemm=True,
+                 max_logits_rows=None, device_budget_bytes=None, check_finite=False, profile=False):
+        """`max_tokens`: tokens the page pool holds; `max_length`: longest request; `max_batch_tokens`: most
+        tokens of one step; `max_logits_rows`: most wanted places of one step (default: every token).
+        `device_budget_bytes`: None for no gate, else the device memory that the runner will hold is planned and
+        compared with min(this cap (0: none), 80 % of the free memory, free - 512 MiB) before the cache is
+        allocated (`MemoryBudgetError`).  `check_finite`: after every layer one small kernel looks at the
+        hidden state; a NaN or an infinity ends the step with `NonFiniteHidden` naming the first layer and
+        row, and poisons the runner (one more synchronisation a step: a debug mode).  `profile`: events
+        around every launch, summed per kernel class (`profile_report`); steps then run eagerly."""
         self.model = model
         self.dtype, self.device = model.dtype, model.device
         spec = model.spec
@@ -40,12 +56,40 @@ class Runner:
         # library_gemm=False: every product on the hand-written kernels (the vendor library takes none)
         self.kernels = Kernels(self.dtype, library_gemm=library_gemm)
         self.kernels.prepare(model.libraries())
+        for block in model.blocks:                        # sizes that no step could serve are refused now
+            for part in block.parts().values():
+                if hasattr(part, "check_limits"):
+                    part.check_limits(self.kernels, self.max_length, page_size, split_keys)
+        self.max_logits_rows = min(max_logits_rows or self.max_batch_tokens, self.max_batch_tokens)
+        # the memory plan, and the budget gate before anything of it is allocated
+        limits = dict(max_length=self.max_length, page_size=page_size, split_keys=split_keys,
+                      split_max_tokens=split_max_tokens, target_workgroups=target_workgroups)
+        workspace_plan = model.workspace_plan(self.max_batch_tokens, self.max_logits_rows, limits)
+        kv, tables, state = CacheManager.plan(model.cache_entry_specs, self.dtype, page_size, max_tokens, max_slots,
+                                              self.max_length)
+        uses_library = library_gemm and self.dtype == torch.bfloat16
+        self.memory_plan = MemoryPlan(
+            weights=model.arena.planned if model.arena is not None else model.weight_bytes(),
+            kv_pages=kv, block_tables=tables, state=state, workspace=Workspace.plan_bytes(workspace_plan),
+            metadata=4 * 4 * self.max_batch_tokens + 8, library_scratch=LIBRARY_GEMM_WORKSPACE if uses_library else 0)
+        self.memory_plan.check(device_budget_bytes, self.device)
         self.cache = CacheManager(model.cache_entry_specs, self.dtype, self.device, page_size,
                                   max_tokens, max_slots, self.max_length)
+        assert (self.cache.kv_bytes(), self.cache.table_bytes(), self.cache.state_bytes()) == (kv, tables, state), \
+            "the cache holds other sizes than were planned"
         self.workspace = Workspace(self.device)
+        self.workspace.reserve(workspace_plan)
+        if uses_library:
+            self.kernels.reserve_library_workspace(self.device)
+        self.check_finite = bool(check_finite)
+        self._status = torch.zeros(2, dtype=torch.int32, device=self.device)
+        if profile:
+            self.kernels.profiler = Profiler()
+            use_graphs = False                            # events inside a captured graph measure nothing
         self.ctx = StepContext(self.kernels, self.cache, self.workspace, self.dtype, self.max_length,
                                split_keys, split_max_tokens)
         self.ctx.target_workgroups = target_workgroups
+        self.ctx.status = self._status if self.check_finite else None
         self._upload = Uploader(4 * self.max_batch_tokens, self.device)
         self._meta = torch.empty(4 * self.max_batch_tokens, dtype=torch.int32, device=self.device)
         self.poisoned = False
@@ -231,8 +275,15 @@ class Runner:
             for w in e.want:
                 if not 0 <= int(w) < n:
                     raise StepError(f"wanted place {w} is outside the entry's {n} tokens")
+            if len(set(int(w) for w in e.want)) != len(e.want):
+                # (a place named once bounds the wanted rows by the step's tokens, which the metadata
+                # vector is sized for)
+                raise StepError("a wanted place is named twice in one entry")
         if total > self.max_batch_tokens:
             raise StepError(f"{total} tokens exceed the step's limit of {self.max_batch_tokens}")
+        wanted = sum(len(e.want) for e in entries)
+        if wanted > self.max_logits_rows:
+            raise StepError(f"{wanted} wanted places exceed the step's limit of {self.max_logits_rows}")
         return total
 
     def step(self, entries: List[Entry]):
@@ -251,6 +302,7 @@ class Runner:
                 logits = self._graph_step(entries, first, total + fill, sig, fill, fill_first)
                 self.cache.retire(slots)
                 self.steps += 1
+                self._raise_if_not_finite()
                 if fill and logits is not None:           # the scratch rows' logits are dropped
                     return logits[fill:] if fill_first else logits[:len(entries)]
                 return logits
@@ -279,7 +331,38 @@ class Runner:
             logits = self.model.forward(ctx, want_rows)
             self.cache.retire(slots)
             self.steps += 1
+            self._raise_if_not_finite()
             return logits
         except Exception:
             self.poisoned = True
             raise
+
+    def _raise_if_not_finite(self):
+        if not self.check_finite:
+            return
+        bits, where = self._status.tolist()               # (waits for the step: the price of the mode)
+        if bits:
+            kinds = " and ".join(name for bit, name in ((1, "a NaN"), (2, "an infinity")) if bits & bit)
+            raise NonFiniteHidden(f"the hidden state holds {kinds}: first after layer run {where >> 20}, "
+                                  f"batch row {where & 0xFFFFF}")
+
+    # -- reports -------------------------------------------------------------------------------
+    def memory_report(self):
+        """The plan beside what is held now, in bytes."""
+        actual = dict(weights=self.model.arena.used if self.model.arena is not None else self.model.weight_bytes(),
+                      kv_pages=self.cache.kv_bytes(), block_tables=self.cache.table_bytes(),
+                      state=self.cache.state_bytes(), workspace=self.workspace.planned_bytes,
+                      workspace_beyond_plan=self.workspace.unplanned_bytes(),
+                      metadata=self._meta.numel() * 4 + self._status.numel() * 4,
+                      library_scratch=self.kernels.library_workspace_bytes())
+        return {"planned": self.memory_plan.as_dict(), "actual": actual}
+
+    def profile_report(self, reset=False):
+        """Time per kernel class since the runner was built (or the last reset); None without profile=True."""
+        profiler = self.kernels.profiler
+        if profiler is None:
+            return None
+        report = profiler.report()
+        if reset:
+            profiler.reset()
+        return report

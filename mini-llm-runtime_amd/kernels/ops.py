@@ -13,6 +13,7 @@ import ctypes
 import torch
 
 from . import build
+from .profile import timed
 
 _c_int = ctypes.c_int
 _c_float = ctypes.c_float
@@ -26,6 +27,7 @@ LIBRARY_GEMM_WORKSPACE = 128 << 20   # bytes of scratch memory that the library 
 PREFILL_MAX_PAGES = 2048      # page ids of one group that the prompt-portion attention kernel keeps in LDS
 TILES_MAX_HEAD_DIM = 128      # the 32x32-tile kernel for prompt portions keeps two sets of accumulators per lane
 TILES_COLUMNS = (128, 64)     # (token, head) columns of one of its workgroups: the usual and the small one
+MFMA_MAX_PAGES = 4096         # page ids of one key range that the single-token attention kernel keeps in LDS
 MAX_KEY_SPLITS = 1024         # the merge of key splits keeps one weight per split in LDS
 
 
@@ -74,6 +76,40 @@ def _ok(code, what):
         raise KernelError(f"{what}: launch failed with code {code}")
 
 
+def _size(t):
+    return 0 if t is None else t.numel() * t.element_size()
+
+
+def _gemm_work(self, a, w, out, *rest, **kw):
+    return _size(a) + _size(w) + _size(out), 2 * a.shape[0] * w.shape[0] * w.shape[1]
+
+
+def _norm_gemm_work(self, h_in, delta, norm_w, eps, h_out, w, out, *rest, **kw):
+    return _size(h_in) + _size(delta) + _size(h_out) + _size(w) + _size(out), 2 * h_in.shape[0] * w.shape[0] * w.shape[1]
+
+
+def _norm_work(self, h, delta, weight, out, eps, rows=None, write_h=True):
+    n, width = out.shape[0], h.shape[1]
+    moved = n * width * 4 + _size(out)
+    if delta is not None:
+        moved += n * width * (delta.element_size() + (4 if write_h else 0))
+    return moved, 0
+
+
+def _embed_work(self, ids, table, h):
+    return _size(h) + h.numel() * table.element_size(), 0
+
+
+def _rope_work(self, qkv, *rest, **kw):
+    return 2 * _size(qkv), 0
+
+
+def _tensors_work(*names):
+    def work(self, *args, **kw):
+        return sum(_size(a) for a in args if isinstance(a, torch.Tensor)), 0
+    return work
+
+
 class Kernels:
     def __init__(self, dtype, library_gemm=True):
         _need(dtype in (torch.float32, torch.bfloat16), f"no kernels for element type {dtype}")
@@ -83,6 +119,7 @@ class Kernels:
         self.library_gemm = library_gemm
         self._library_workspace = None      # scratch memory of the vendor library's products, allocated once
         self._libs = {}
+        self.profiler = None                # a `Profiler`: every launch is then bracketed by events
 
     # -- libraries ---------------------------------------------------------------------------
     def prepare(self, names):
@@ -104,6 +141,7 @@ class Kernels:
         return lib
 
     # -- row-wise ----------------------------------------------------------------------------
+    @timed("embed", _embed_work)
     def embed_gather(self, ids, table, h):
         """h[m] = float(table[ids[m]])."""
         rows = ids.numel()
@@ -115,6 +153,7 @@ class Kernels:
         _ok(fn(_p(ids), _p(table), _p(h), _c_int(rows), _c_int(width), _c_int(vocab), _stream()),
             "embed_gather")
 
+    @timed("norm", _norm_work)
     def add_rmsnorm(self, h, delta, weight, out, eps, rows=None, write_h=True):
         """x = h[src] + delta[src] (delta may be None); h[src] = x when write_h; out[r] =
         rmsnorm(x) * weight, src = rows[r] or r."""
@@ -134,12 +173,33 @@ class Kernels:
                _c_float(eps), _c_int(1 if (write_h and delta is not None) else 0), _stream()),
             "add_rmsnorm")
 
+    @timed("check")
+    def status_reset(self, status):
+        """status = (0, INT_MAX): nothing seen yet.  A kernel, so that a captured step can hold it."""
+        _tensor(status, "status", torch.int32, (2,))
+        _ok(self._lib("elementwise").mlr_status_reset(_p(status), _stream()), "status_reset")
+
+    @timed("check")
+    def finite_check(self, h, delta, layer, status):
+        """ORs into status[0] which kinds of non-finite values h + delta holds (1: NaN, 2: infinity) and keeps
+        in status[1] the smallest (layer << 20 | row) that held one."""
+        _tensor(h, "h", torch.float32, ndim=2)
+        m, width = h.shape
+        if delta is not None:
+            _tensor(delta, "delta", self.dtype, (m, width))
+        _tensor(status, "status", torch.int32, (2,))
+        _need(0 <= layer < 2047, "finite_check: layer index out of range")
+        _ok(self._lib("elementwise").mlr_finite_check(_p(h), _p(delta), _c_int(m), _c_int(width), _c_int(layer),
+                                                      _p(status), _stream()), "finite_check")
+
+    @timed("norm", _tensors_work())
     def residual_add(self, h, delta):
         _tensor(h, "h", torch.float32, ndim=2)
         _tensor(delta, "delta", self.dtype, tuple(h.shape))
         fn = self._lib("elementwise").mlr_residual_add
         _ok(fn(_p(h), _p(delta), _c_size_t(h.numel()), _stream()), "residual_add")
 
+    @timed("activation", _tensors_work())
     def silu_mul(self, gate_up, act):
         """act[m, f] = silu(gate_up[m, f]) * gate_up[m, F + f]."""
         _tensor(gate_up, "gate_up", self.dtype, ndim=2)
@@ -150,6 +210,7 @@ class Kernels:
         _ok(fn(_p(gate_up), _p(act), _c_int(m), _c_int(two_f // 2), _stream()), "silu_mul")
 
     # -- projections -------------------------------------------------------------------------
+    @timed("gemm", _gemm_work)
     def gemm(self, a, w, out):
         """out[M, N] = a[M, K] . w[N, K]^T; out has the element type or is float32."""
         _tensor(a, "a", self.dtype, ndim=2)
@@ -164,9 +225,7 @@ class Kernels:
             # many rows: a plain matrix product, handed to the vendor library (hipBLASLt), as the reference
             # hands its projections to cuBLAS (src/minillm/cuda/matrix.cpp:11-37).  (Float outputs are
             # logits, a vocabulary wide: there the library wins from 17 rows on at any inner size.)
-            if self._library_workspace is None:
-                self._library_workspace = torch.empty(LIBRARY_GEMM_WORKSPACE, dtype=torch.uint8, device=a.device)
-            ws = self._library_workspace
+            ws = self.reserve_library_workspace(a.device)
             _ok(self._lib("library_gemm").mlr_library_gemm(_p(a), _p(w), _p(out), _c_int(m), _c_int(n), _c_int(k),
                                                            _c_int(1 if out.dtype == torch.float32 else 0),
                                                            _p(ws), _c_size_t(ws.numel()), _stream()), "library_gemm")
@@ -174,6 +233,15 @@ class Kernels:
         fn = self._lib("gemm").mlr_gemm
         _ok(fn(_p(a), _p(w), _p(out), _c_int(m), _c_int(n), _c_int(k),
                _c_int(1 if out.dtype == torch.float32 else 0), _stream()), "gemm")
+
+    def reserve_library_workspace(self, device):
+        """The vendor library's scratch memory, allocated once."""
+        if self._library_workspace is None:
+            self._library_workspace = torch.empty(LIBRARY_GEMM_WORKSPACE, dtype=torch.uint8, device=device)
+        return self._library_workspace
+
+    def library_workspace_bytes(self):
+        return 0 if self._library_workspace is None else self._library_workspace.numel()
 
     def streams_weight(self, rows, k):
         """Whether a projection of this many rows and inner size goes to the kernels that stream the weight
@@ -197,6 +265,7 @@ class Kernels:
             return not self.library_gemm or k <= 1024 or (k <= 2048 and rows <= 256)
         return self.streams_weight(rows, k if k is not None else 1 << 30)
 
+    @timed("gemm", _gemm_work)
     def gemm_gated_silu(self, a, w, out):
         """out[M, N] = silu(a . w[:N]^T) * (a . w[N:]^T), w = [gate; up] stacked: up to 64 rows, or any number
         when the inner size is a multiple of 64 (the wide kernel's gated form)."""
@@ -217,6 +286,7 @@ class Kernels:
         """Whether `norm_gemm` (residual add + RMSNorm inside the projection) serves these sizes."""
         return self.dtype == torch.bfloat16 and rows <= 16 and width % 32 == 0 and width <= 2048
 
+    @timed("gemm", _norm_gemm_work)
     def norm_gemm(self, h_in, delta, norm_w, eps, h_out, w, out, gated=False):
         """x = h_in + delta (delta may be None); h_out = x; out = rmsnorm(x, norm_w) . w^T, or with
         gated=True (w = [gate; up] stacked) silu(. gate^T) * (. up^T).  For few rows: one launch instead
@@ -244,6 +314,7 @@ class Kernels:
               lambda: f"k_pages: expected [pages, {kv_heads}, {page_size}, {head_dim}], got {tuple(k_pages.shape)}")
         _tensor(v_pages, "v_pages", self.dtype, (k_pages.shape[0], kv_heads, head_dim, page_size))
 
+    @timed("rope_kv", _rope_work)
     def qk_norm_rope_kv(self, qkv, q_out, k_pages, v_pages, block_table, slots, positions, q_norm_w,
                         k_norm_w, eps, rope, q_heads, kv_heads, head_dim, page_size, write_cache=True):
         """Per head: RMSNorm of q and k (weights may be None), rotation by `rope`
@@ -276,6 +347,7 @@ class Kernels:
         unnormalised output, its maximum and its sum (the prompt-portion kernel keeps them 16 bytes apart)."""
         return rows * q_heads * max_splits * (head_dim + 4)
 
+    @timed("attention")
     def paged_attention(self, q, k_pages, v_pages, block_table, slots, positions, out, q_heads,
                         kv_heads, head_dim, page_size, scale, window=None, split_keys=0, max_splits=1,
                         partial=None):
@@ -315,6 +387,7 @@ class Kernels:
         return (self.dtype == torch.bfloat16 and page_size % 16 == 0 and head_dim % 16 == 0
                 and head_dim <= MAX_HEAD_DIM and q_heads % kv_heads == 0 and q_heads // kv_heads <= 16)
 
+    @timed("attention")
     def attention_mfma(self, q, k_pages, v_pages, block_table, slots, positions, out, group_row0, group_ntok,
                        groups, q_heads, kv_heads, head_dim, page_size, scale, window=None, split_keys=0,
                        max_splits=1, partial=None):
@@ -342,7 +415,7 @@ class Kernels:
             _tensor(partial, "partial", torch.float32, ndim=1)
             _need(partial.numel() >= self.attention_partial_numel(m, q_heads, head_dim, max_splits),
                   "partial buffer too small")
-        _need((split_keys // page_size + 2 if max_splits > 1 else block_table.shape[1]) <= 4096,
+        _need((split_keys // page_size + 2 if max_splits > 1 else block_table.shape[1]) <= MFMA_MAX_PAGES,
               "attention_mfma: a workgroup's key range spans more than 4096 pages; split the keys")
         fn = self._lib("attention").mlr_attention_mfma
         _ok(fn(_p(q), _p(k_pages), _p(v_pages), _p(block_table), _c_int(block_table.shape[1]), _p(slots),
@@ -350,11 +423,22 @@ class Kernels:
                _c_int(q_heads), _c_int(kv_heads), _c_int(head_dim), _c_int(page_size), _c_int(window or 0),
                _c_float(scale), _c_int(split_keys), _c_int(max_splits), _stream()), "attention_mfma")
 
+    @staticmethod
+    def max_key_splits():
+        return MAX_KEY_SPLITS
+
+    @staticmethod
+    def mfma_longest_context(page_size):
+        """The most keys that one workgroup of `attention_mfma` / `attention_decode_fused` can walk (it keeps
+        their page ids in LDS; a key split that does not start at a page's edge touches one page more)."""
+        return (MFMA_MAX_PAGES - 2) * page_size
+
     def decode_fusion_supported(self, q_heads, kv_heads, head_dim, page_size):
         """Attention for single new tokens that norms, rotates and caches inside itself: the matrix-core
         kernel's sizes and head sizes that are multiples of 64."""
         return self.mfma_attention_supported(q_heads, kv_heads, head_dim, page_size) and head_dim % 64 == 0
 
+    @timed("attention")
     def attention_decode_fused(self, qkv, k_pages, v_pages, block_table, slots, positions, out, group_row0, group_ntok,
                                groups, q_heads, kv_heads, head_dim, page_size, scale, q_norm_w, k_norm_w, eps, rope,
                                partial, window=None, split_keys=0, max_splits=1):
@@ -390,7 +474,7 @@ class Kernels:
                   lambda: f"split_keys must be a multiple of {ATTENTION_TILE_KEYS}")
         _tensor(partial, "partial", torch.float32, ndim=1)
         _need(partial.numel() >= self.attention_partial_numel(m, q_heads, head_dim, max_splits), "partial buffer too small")
-        _need((split_keys // page_size + 2 if max_splits > 1 else block_table.shape[1]) <= 4096,
+        _need((split_keys // page_size + 2 if max_splits > 1 else block_table.shape[1]) <= MFMA_MAX_PAGES,
               "attention_decode_fused: a workgroup's key range spans more than 4096 pages; split the keys")
         fn = self._lib("attention").mlr_attention_decode_fused
         _ok(fn(_p(qkv), _c_int(width), _p(k_pages), _p(v_pages), _p(block_table), _c_int(block_table.shape[1]),
@@ -405,6 +489,7 @@ class Kernels:
         return (self.mfma_attention_supported(q_heads, kv_heads, head_dim, page_size) and head_dim <= 192
                 and max_context <= PREFILL_MAX_PAGES * page_size)
 
+    @timed("attention")
     def attention_prefill(self, q, k_pages, v_pages, block_table, slots, positions, out, group_row0, group_ntok,
                           groups, q_heads, kv_heads, head_dim, page_size, scale, window=None, max_context=None):
         """Attention for prompt portions: groups of up to 4 * (16 // (q_heads // kv_heads)) consecutive rows
@@ -453,6 +538,7 @@ class Kernels:
         """The most tokens of a group of `attention_tiles` with workgroups of `columns` columns."""
         return columns // (q_heads // kv_heads)
 
+    @timed("attention")
     def attention_tiles(self, q, k_pages, v_pages, block_table, slots, positions, out, group_row0, group_ntok,
                         groups, q_heads, kv_heads, head_dim, page_size, scale, window=None, max_context=None,
                         columns=TILES_COLUMNS[0], split_keys=0, max_splits=1, partial=None):
@@ -502,6 +588,7 @@ class Kernels:
         lib = self._lib("sampling")
         return lib.mlr_sample_scratch_floats(_c_int(rows)), lib.mlr_sample_scratch_ints(_c_int(rows))
 
+    @timed("sampler")
     def sample(self, logits, temperature, uniform, tokens, status, scratch_f, scratch_i, any_sampling=True):
         """tokens[r] = argmax (temperature <= 0) or the inverse-CDF draw at uniform[r]."""
         _tensor(logits, "logits", torch.float32, ndim=2)

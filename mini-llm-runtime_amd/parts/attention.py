@@ -8,7 +8,7 @@ from __future__ import annotations
 import torch
 
 from ..cache.manager import KvSpec
-from ..weights.loader import WeightSpec
+from ..weights.loader import WeightSpec, stacked
 from .registry import PartError, build_part, register_part
 
 
@@ -20,8 +20,10 @@ class GqaAttention:
         s = spec
         if s.q_heads % s.kv_heads != 0:
             raise PartError(f"q_heads {s.q_heads} is no multiple of kv_heads {s.kv_heads}")
-        if s.head_dim % 16 != 0 or s.head_dim > 256:
-            raise PartError(f"head_dim {s.head_dim}: the attention kernels take multiples of 16 up to 256")
+        if s.head_dim % 2 != 0 or not 2 <= s.head_dim <= 256:
+            # (multiples of 16 run on the matrix cores in the bfloat16 engine, other even sizes on the
+            # scalar kernels that serve the float engine)
+            raise PartError(f"head_dim {s.head_dim}: the attention kernels take even sizes up to 256")
         if s.window is not None and s.window < 1:
             raise PartError("window must be positive")
         self.q_norm = build_part("norm", s.qk_norm) if s.qk_norm is not None else None
@@ -37,9 +39,9 @@ class GqaAttention:
     def weight_specs(self):
         s = self.spec
         specs = {
-            "q_proj": WeightSpec((s.q_heads * s.head_dim, s.hidden)),
-            "k_proj": WeightSpec((s.kv_heads * s.head_dim, s.hidden)),
-            "v_proj": WeightSpec((s.kv_heads * s.head_dim, s.hidden)),
+            "q_proj": WeightSpec((s.q_heads * s.head_dim, s.hidden), stack="qkv"),
+            "k_proj": WeightSpec((s.kv_heads * s.head_dim, s.hidden), stack="qkv"),
+            "v_proj": WeightSpec((s.kv_heads * s.head_dim, s.hidden), stack="qkv"),
             "o_proj": WeightSpec((s.hidden, s.q_heads * s.head_dim)),
         }
         if self.q_norm is not None:
@@ -48,8 +50,9 @@ class GqaAttention:
         return specs
 
     def bind(self, weights):
-        # rows of a projection are independent sums, so stacking q, k, v changes no result
-        self.qkv = torch.cat([weights["q_proj"], weights["k_proj"], weights["v_proj"]], dim=0).contiguous()
+        # rows of a projection are independent sums, so stacking q, k, v changes no result (the loader has
+        # laid them out one after the other already: no copy then)
+        self.qkv = stacked([weights["q_proj"], weights["k_proj"], weights["v_proj"]])
         self.o = weights["o_proj"]
         if self.q_norm is not None:
             self.q_norm.bind({"weight": weights["q_norm.weight"]})
@@ -57,6 +60,53 @@ class GqaAttention:
 
     def cache_spec(self):
         return KvSpec(self.spec.kv_heads, self.spec.head_dim, self.spec.window)
+
+    def check_limits(self, kernels, max_length, page_size, split_keys):
+        """Called once when a runner is built: whether every context up to `max_length` can be served
+        with these pages and this smallest key range of a workgroup.  What cannot is refused here and
+        not in the middle of a step."""
+        s = self.spec
+        if not kernels.mfma_attention_supported(s.q_heads, s.kv_heads, s.head_dim, page_size):
+            return                        # the scalar kernel walks the block table itself: no limit
+        longest = kernels.mfma_longest_context(page_size)
+        if max_length <= longest:
+            return
+        if split_keys <= 0:
+            raise PartError(f"max_length {max_length} with pages of {page_size} tokens needs key splits "
+                            f"(split_keys > 0): one workgroup walks at most {longest} keys")
+        if split_keys > longest:
+            raise PartError(f"split_keys {split_keys} exceeds the {longest} keys one workgroup can walk "
+                            f"with pages of {page_size} tokens")
+        keys = split_keys
+        while keys * 2 <= longest:
+            keys *= 2
+        if max_length > keys * kernels.max_key_splits():
+            raise PartError(f"max_length {max_length} needs more than {kernels.max_key_splits()} key splits "
+                            f"of {keys} keys")
+
+    def workspace_plan(self, rows, dtype, limits):
+        """{(buffer name, dtype): elements} that `forward` asks the workspace for in a step of `rows` tokens
+        at most.  The partial results of split attention are bounded by how splits are chosen: a split is
+        made only while (workgroups without it) x (splits) stays below twice `target_workgroups`, each
+        workgroup serving at most 128 (token, head) columns; a context beyond one workgroup's reach is
+        split for every row."""
+        s = self.spec
+        width = s.q_heads * s.head_dim
+        forced = 1
+        longest = (4096 - 2) * limits["page_size"]
+        if limits["max_length"] > longest and limits["split_keys"] > 0:
+            keys = limits["split_keys"]
+            while keys * 2 <= longest:
+                keys *= 2
+            forced = -(-limits["max_length"] // keys)
+        partial = max(2 * limits["target_workgroups"] * 128, rows * s.q_heads * forced) * (s.head_dim + 4)
+        tq = max(1, 16 // (s.q_heads // s.kv_heads))
+        plan = {("qkv", dtype): rows * (width + 2 * s.kv_heads * s.head_dim), ("q", dtype): rows * width,
+                ("attn", dtype): rows * width, ("mixer_out", dtype): rows * s.hidden,
+                ("attn_partial", torch.float32): partial}
+        for big_factor in (0, 4, 8):
+            plan[(f"token_groups_{tq}_{big_factor}", torch.int32)] = 2 * rows + 2
+        return plan
 
     def libraries(self):
         tiles = ["attention_tiles"] if self.qkv is not None and self.qkv.dtype == torch.bfloat16 else []
@@ -78,9 +128,33 @@ class GqaAttention:
         ctx.kernels.gemm(x, self.qkv, qkv)
         return self._attend(ctx, qkv, cache_id, write_cache)
 
+    def _attention_work(self, ctx, element_size):
+        """For the profile: (bytes, flops) of this step's attention, from the host's view of the contexts."""
+        s = self.spec
+        keys_read = pairs = 0
+        for _, _, n, p0 in ctx.segments:
+            last = p0 + n
+            keys_read += min(last, s.window + n - 1) if s.window else last
+            for p in (range(p0, last) if s.window else ()):
+                pairs += min(p + 1, s.window)
+            if not s.window:
+                pairs += n * p0 + n * (n + 1) // 2
+        moved = keys_read * 2 * s.kv_heads * s.head_dim * element_size \
+            + 2 * ctx.n_tokens * s.q_heads * s.head_dim * element_size
+        return moved, 4 * pairs * s.q_heads * s.head_dim
+
+    def _hint(self, kernels):
+        if self._work is not None:                        # the step's attention work goes to its first launch
+            kernels.profiler.next_work(*self._work)
+            self._work = None
+
     def _attend(self, ctx, qkv, cache_id, write_cache):
         s = self.spec
         k = ctx.kernels
+        if k.profiler is not None and not ctx.fixed_groups:
+            self._work = self._attention_work(ctx, qkv.element_size())
+        else:
+            self._work = None
         x = qkv
         m = qkv.shape[0]
         view = ctx.cache.kv_view(cache_id)
@@ -90,10 +164,12 @@ class GqaAttention:
             # decoding: norm, rotation and cache write ride in the attention's two launches
             attn = ctx.workspace.get("attn", (m, s.q_heads * s.head_dim), x.dtype)
             groups, _, _ = ctx.token_groups(max(1, 16 // (s.q_heads // s.kv_heads)), 0)
-            split_keys, max_splits, partial = ctx.attention_split(m, m, s.kv_heads, s.q_heads, s.head_dim)
+            split_keys, max_splits, partial = ctx.attention_split(m, m, s.kv_heads, s.q_heads, s.head_dim,
+                                                                  longest=k.mfma_longest_context(view.page_size))
             if partial is None:
                 partial = ctx.workspace.get("attn_partial", (k.attention_partial_numel(m, s.q_heads, s.head_dim, 1),),
                                             torch.float32)
+            self._hint(k)
             k.attention_decode_fused(
                 qkv, view.k_pages, view.v_pages, view.block_table, ctx.slots, ctx.positions, attn, groups[0], groups[1],
                 groups[2], s.q_heads, s.kv_heads, s.head_dim, view.page_size, float(s.scale),
@@ -120,7 +196,8 @@ class GqaAttention:
             g = s.q_heads // s.kv_heads
             tq = max(1, 16 // g)
             # (with key splits the 32x32-tile kernel takes any context length)
-            tiles = k.tiles_attention_supported(*sizes, num_pages=view.k_pages.shape[0], split_keys=ctx.split_keys)
+            tiles = k.tiles_attention_supported(*sizes, max_context=ctx.max_context, num_pages=view.k_pages.shape[0],
+                                                split_keys=ctx.split_keys)
             # workgroups of 128 columns (launched in pairs) unless they would leave half of the compute
             # units idle: then of 64
             columns = 128 if m * s.q_heads > 128 * ctx.compute_units else 64
@@ -130,22 +207,27 @@ class GqaAttention:
             if big[2] and tiles:
                 split_keys, max_splits, partial = ctx.group_split(
                     big[2], m, s.kv_heads, s.q_heads, s.head_dim, longest=k.tiles_longest_context(view.page_size))
+                self._hint(k)
                 k.attention_tiles(q, view.k_pages, view.v_pages, view.block_table, ctx.slots, ctx.positions, attn,
                                   big[0], big[1], big[2], s.q_heads, s.kv_heads, s.head_dim, view.page_size,
                                   float(s.scale), window=s.window, max_context=ctx.max_context, columns=columns,
                                   split_keys=split_keys, max_splits=max_splits, partial=partial)
             elif big[2]:
+                self._hint(k)
                 k.attention_prefill(q, view.k_pages, view.v_pages, view.block_table, ctx.slots, ctx.positions, attn,
                                     big[0], big[1], big[2], s.q_heads, s.kv_heads, s.head_dim, view.page_size,
                                     float(s.scale), window=s.window, max_context=ctx.max_context)
             if small[2]:
-                split_keys, max_splits, partial = ctx.attention_split(small_rows, m, s.kv_heads, s.q_heads, s.head_dim)
+                split_keys, max_splits, partial = ctx.attention_split(
+                    small_rows, m, s.kv_heads, s.q_heads, s.head_dim, longest=k.mfma_longest_context(view.page_size))
+                self._hint(k)
                 k.attention_mfma(q, view.k_pages, view.v_pages, view.block_table, ctx.slots, ctx.positions, attn,
                                  small[0], small[1], small[2], s.q_heads, s.kv_heads, s.head_dim, view.page_size,
                                  float(s.scale), window=s.window, split_keys=split_keys, max_splits=max_splits,
                                  partial=partial)
         else:
             split_keys, max_splits, partial = ctx.attention_split(m, m, s.kv_heads, s.q_heads, s.head_dim)
+            self._hint(k)
             k.paged_attention(q, view.k_pages, view.v_pages, view.block_table, ctx.slots, ctx.positions, attn,
                               s.q_heads, s.kv_heads, s.head_dim, view.page_size, float(s.scale),
                               window=s.window, split_keys=split_keys, max_splits=max_splits, partial=partial)

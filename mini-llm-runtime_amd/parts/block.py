@@ -19,6 +19,11 @@ class PreNormBlock:
     def parts(self):
         return {"norm1": self.norm1, "mixer": self.mixer, "norm2": self.norm2, "ffn": self.ffn}
 
+    def workspace_plan(self, rows, dtype, limits):
+        import torch
+        width = self.norm1.size
+        return {("hidden_alt", torch.float32): min(rows, 16) * width, ("normed", dtype): rows * width}
+
     def forward(self, ctx, h, pending, cache_id, write_cache=True):
         if (ctx.kernels.norm_gemm_supported(h.shape[0], h.shape[1])
                 and getattr(self.norm1, "fusable_rmsnorm", False) and getattr(self.norm2, "fusable_rmsnorm", False)

@@ -4,7 +4,7 @@ from __future__ import annotations
 
 import torch
 
-from ..weights.loader import WeightSpec
+from ..weights.loader import WeightSpec, stacked
 from .registry import PartError, register_part
 
 
@@ -20,16 +20,21 @@ class SwiGluMlp:
 
     def weight_specs(self):
         s = self.spec
-        return {"gate_proj": WeightSpec((s.intermediate, s.hidden)),
-                "up_proj": WeightSpec((s.intermediate, s.hidden)),
+        return {"gate_proj": WeightSpec((s.intermediate, s.hidden), stack="gate_up"),
+                "up_proj": WeightSpec((s.intermediate, s.hidden), stack="gate_up"),
                 "down_proj": WeightSpec((s.hidden, s.intermediate))}
 
     def bind(self, weights):
-        self.gate_up = torch.cat([weights["gate_proj"], weights["up_proj"]], dim=0).contiguous()
+        self.gate_up = stacked([weights["gate_proj"], weights["up_proj"]])
         self.down = weights["down_proj"]
 
     def libraries(self):
         return ["gemm", "elementwise"]
+
+    def workspace_plan(self, rows, dtype, limits):
+        s = self.spec
+        return {("act", dtype): rows * s.intermediate, ("gate_up", dtype): rows * 2 * s.intermediate,
+                ("ffn_out", dtype): rows * s.hidden}
 
     def forward_prenorm(self, ctx, h, delta, norm, h_out):
         """As `forward` on norm(h + delta), add and norm done inside the first projection (few rows)."""

@@ -7,6 +7,8 @@ class (`global_tensor_name`, `layer_tensor_name`).  The model itself knows no ar
 """
 from __future__ import annotations
 
+from dataclasses import replace
+
 import torch
 
 from ..config import load_config
@@ -30,6 +32,8 @@ def _tensor_plan(config, spec, blocks):
     for i, block in enumerate(blocks):
         for part_name, part in block.parts().items():
             for local, ws in part.weight_specs().items():
+                if ws.stack is not None:              # a stack belongs to one part of one layer
+                    ws = replace(ws, stack=f"{i}.{part_name}.{ws.stack}")
                 plan.append((config.layer_tensor_name(i, part_name, local), ws, (i, part_name), local))
     names = [p[0] for p in plan]
     if len(set(names)) != len(names):
@@ -50,6 +54,7 @@ class DecoderModel:
         self.config = config
         self.spec = spec = config.model_spec()
         self.dtype, self.device = dtype, torch.device(device)
+        self.arena = None                     # the planned allocation that holds the weights (set by `load`)
         if len(spec.schedule) == 0:
             raise PartError("the schedule runs no layer")
         for run in spec.schedule:
@@ -90,10 +95,15 @@ class DecoderModel:
                 raise PartError(f"cache entry {cid} is read but never written")
 
     @classmethod
-    def load(cls, folder, dtype, device="cuda:0"):
+    def load(cls, folder, dtype, device="cuda:0", device_budget_bytes=None):
+        """`device_budget_bytes`: None for no gate; else the weights' planned bytes are checked against
+        min(this cap (0: none), 80 % of the free device memory, free - 512 MiB) before anything is allocated."""
         config = load_config(folder)
-        weights = load_weights(folder, expected_tensors(config), dtype, device)
-        return cls(config, weights, dtype, device)
+        arena = []
+        weights = load_weights(folder, expected_tensors(config), dtype, device, device_budget_bytes, arena)
+        model = cls(config, weights, dtype, device)
+        model.arena = arena[0]
+        return model
 
     def libraries(self):
         names = {"elementwise", "gemm"}
@@ -105,12 +115,26 @@ class DecoderModel:
                     names.update(part.libraries())
         return sorted(names)
 
+    def workspace_plan(self, rows, logits_rows, limits):
+        """{(buffer name, dtype): elements} of every scratch buffer that a step of at most `rows` tokens with
+        at most `logits_rows` wanted places asks for: this model's own and those of the parts that state
+        theirs (`workspace_plan(rows, dtype, limits)`; a part without one gets its buffers on demand)."""
+        plan = {("hidden", torch.float32): rows * self.spec.hidden, ("final", self.dtype): logits_rows * self.spec.hidden,
+                ("logits", torch.float32): logits_rows * self.spec.vocab_size}
+        for block in self.blocks:
+            for part in [block, *block.parts().values()]:
+                if hasattr(part, "workspace_plan"):
+                    for key, count in part.workspace_plan(rows, self.dtype, limits).items():
+                        plan[key] = max(plan.get(key, 0), count)
+        return plan
+
     def graph_safe(self):
         """True when every part of every layer may be captured in a graph."""
         return all(getattr(part, "graph_safe", False) for block in self.blocks
                    for part in [block, *block.parts().values()]) and getattr(self.final_norm, "graph_safe", False)
 
     def weight_bytes(self):
+        """Bytes of the tensors the model uses (each once; without the padding between them)."""
         seen, total = set(), 0
         tensors = [self.embed, self.lm_head, self.final_norm.weight]
         for block in self.blocks:
@@ -128,10 +152,15 @@ class DecoderModel:
         k = ctx.kernels
         m = ctx.n_tokens
         h = ctx.workspace.get("hidden", (m, self.spec.hidden), torch.float32)
+        status = getattr(ctx, "status", None)            # the debug mode that looks at the hidden state
+        if status is not None:
+            k.status_reset(status)
         k.embed_gather(ctx.token_ids, self.embed, h)
         pending = None
-        for run in self.spec.schedule:
+        for i, run in enumerate(self.spec.schedule):
             pending = self.blocks[run.layer].forward(ctx, h, pending, run.cache, run.write_cache)
+            if status is not None:                        # h + pending is the hidden state after this run
+                k.finite_check(h, pending, i, status)
         r = 0 if want_rows is None else want_rows.numel()
         if r == 0:
             return None

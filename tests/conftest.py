@@ -42,8 +42,14 @@ TINY = {
               num_attention_heads=6, num_key_value_heads=3, head_dim=48, intermediate_size=100,
               vocab_size=517, max_position_embeddings=4096, rms_norm_eps=3e-6, rope_theta=500000.0,
               tie_word_embeddings=False, eos_token_id=5),
+    # 2 layers, 5 q / 5 kv heads (no sharing), head 20: an even head size that is no multiple of 16, which
+    # the matrix-core kernels do not take (both engines run it on the scalar kernels); pages of 4
+    "D": dict(architectures=["Qwen3ForCausalLM"], hidden_size=100, num_hidden_layers=2,
+              num_attention_heads=5, num_key_value_heads=5, head_dim=20, intermediate_size=70,
+              vocab_size=97, max_position_embeddings=512, rms_norm_eps=2e-5, rope_theta=20000.0,
+              tie_word_embeddings=True),
 }
-PAGE_SIZE = {"A": 16, "B": 8, "C": 32}
+PAGE_SIZE = {"A": 16, "B": 8, "C": 32, "D": 4}
 
 
 @pytest.fixture(scope="session")

@@ -75,6 +75,25 @@ def test_every_way_of_cutting_gives_the_plain_logits(model_folders, expected, na
         assert max_difference(results["whole"], results[mode]) <= limit, mode
 
 
+@pytest.mark.parametrize("name", TINY)
+def test_the_engine_without_the_vendor_library_gives_the_plain_logits(model_folders, expected, name):
+    """`Runner(library_gemm=False)`: every matrix product of the bfloat16 engine on the hand-written kernels
+    (the kernel for inner sizes that are no multiple of 64, the wide kernel's plain form, weight streaming up
+    to 64 rows), whole, in portions, one by one and mixed, against the plain logits."""
+    reqs, want = expected[name]
+    model = load(model_folders, name, "bfloat16")
+    r = runner_for(model, name, max_tokens=192, library_gemm=False)
+    assert not r.kernels.library_gemm and r.memory_plan.library_scratch == 0
+    for steps in (whole(reqs), last_one_by_one(reqs), portions(reqs)):
+        compare(run_steps(r, steps), want, "bfloat16")
+    steps, peak = mixed(reqs, seed=5)
+    r = runner_for(model, name, max_tokens=peak, library_gemm=False)
+    compare(run_steps(r, steps), want, "bfloat16")
+    r.cache.check()
+    assert r.cache.free_pages() == r.cache.num_pages
+    assert r.kernels.library_workspace_bytes() == 0          # the library was never asked
+
+
 @pytest.mark.parametrize("dtype_name", DTYPES)
 @pytest.mark.parametrize("name", TINY)
 @pytest.mark.parametrize("split_keys,split_max_tokens", [(64, 10 ** 6), (0, 0)])
@@ -282,6 +301,7 @@ def test_refused_batches_change_nothing(model_folders, plain_models):
     bad = [[], [Entry(s, [], [])], [Entry(s, [256], [0])], [Entry(s, [-1], [0])], [Entry(s, [1, 2], [2])],
            [Entry(s, [1], [-1])], [Entry(7, [1], [0])], [Entry(s, [1], [0]), Entry(s, [2], [0])],
            [Entry(s, [1] * 41, [])], [Entry(s, [1] * 29, [])],            # beyond the step's limit; beyond max_length
+           [Entry(s, [1, 2], [0, 0])], [Entry(s, [1] * 28, [3] * 60)],    # a place named twice; more rows than tokens
            [Entry(s, [1] * 10, []), Entry(other, [1] * 40, [])]]          # `other` needs 3 pages, 2 are free
     for batch in bad:
         with pytest.raises((StepError, CacheError, CacheFull)):

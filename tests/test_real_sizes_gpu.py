@@ -85,6 +85,30 @@ def test_prompt_of_256_tokens_every_way(folders, expectations, name, dtype_name)
 
 
 @pytest.mark.parametrize("name", list(CONFIGS))
+def test_prompt_of_256_tokens_without_the_vendor_library(folders, expectations, name):
+    """The same prompt with every product on the hand-written kernels (`library_gemm=False`): whole (256 rows:
+    the wide kernel, plain and gated), in portions of 7 to 96 tokens (17 to 64 rows: weight streaming, the
+    16x16-tile kernel where the inner size allows) and one by one."""
+    from helpers import run_steps
+    from mini_llm_runtime_amd.engine import Runner
+    from mini_llm_runtime_amd.parts import DecoderModel
+    toks, want = expectations[name]
+    model = DecoderModel.load(folders[name], torch.bfloat16)
+    r = Runner(model, max_tokens=512, max_slots=2, max_batch_tokens=256, page_size=16, library_gemm=False)
+    cuts = [0, 7, 16, 34, 98, 128, 224]
+    steps = [dict(step=0, entries=[dict(id="w", tokens=toks, want=WANT)], end=["w"])]
+    steps += [dict(step=1 + i, entries=[dict(id="r0", tokens=toks[lo:hi], want=[p - lo for p in WANT if lo <= p < hi])],
+                   end=[]) for i, (lo, hi) in enumerate(zip(cuts, cuts[1:]))]
+    steps += [dict(step=100 + p, entries=[dict(id="r0", tokens=[toks[p]], want=[0] if p in WANT else [])], end=[])
+              for p in range(224, 256)]
+    steps[-1]["end"] = ["r0"]
+    got = run_steps(r, steps)
+    compare({k: v for k, v in got.items() if k[0] == "w"}, {("w", p): v for (_, p), v in want.items()}, "bfloat16")
+    compare({k: v for k, v in got.items() if k[0] == "r0"}, want, "bfloat16")
+    assert r.kernels.library_workspace_bytes() == 0
+
+
+@pytest.mark.parametrize("name", list(CONFIGS))
 def test_graph_replays_with_library_products_match_eager(folders, name):
     """24 requests decode together: their projections have more than 16 rows and go to the vendor library,
     inside the captured graph.  Every replay (with eager work and synchronisations between the replays) must
