@@ -15,6 +15,11 @@
 //   pass 4 (rows): scan of the chunk sums, the chunk that holds u * total, then the token inside it.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <stdio.h>
+
+#include <mutex>
+
+#include "no_alloc.h"
 
 #define CHUNKS 64
 #define THREADS 256
@@ -181,13 +186,11 @@ __global__ __launch_bounds__(THREADS) void pick_kernel(const float* __restrict__
 extern "C" int mlr_sample_scratch_floats(int rows) { return rows * (2 * CHUNKS + 1); }
 extern "C" int mlr_sample_scratch_ints(int rows) { return rows * 2 * CHUNKS; }
 
-// scratch_f: rows * (2 CHUNKS + 1) floats; scratch_i: rows * 2 CHUNKS ints.  `any_sampling` = 0 skips
-// passes 3 and 4 (every temperature <= 0).
-extern "C" int mlr_sample(const float* logits, int rows, int vocab, const float* temperature,
-                          const float* uniform, int32_t* tokens, int32_t* status, float* scratch_f,
-                          int32_t* scratch_i, int any_sampling, hipStream_t stream) {
-    if (rows <= 0) return 0;
-    if (vocab <= 0) return -1;
+// The four passes over scratch memory scratch_f (rows * (2 CHUNKS + 1) floats) and scratch_i (rows * 2 CHUNKS
+// ints), wherever it comes from.
+static int launch_sample(const float* logits, int rows, int vocab, const float* temperature, const float* uniform,
+                         int32_t* tokens, int32_t* status, float* scratch_f, int32_t* scratch_i, int any_sampling,
+                         hipStream_t stream) {
     float* cmax = scratch_f;
     float* csum = scratch_f + (size_t)rows * CHUNKS;
     float* rmax = scratch_f + (size_t)rows * 2 * CHUNKS;
@@ -200,4 +203,64 @@ extern "C" int mlr_sample(const float* logits, int rows, int vocab, const float*
         pick_kernel<<<rows, THREADS, 0, stream>>>(logits, vocab, temperature, uniform, rmax, csum, tokens);
     }
     return (int)hipGetLastError();
+}
+
+// scratch_f: rows * (2 CHUNKS + 1) floats; scratch_i: rows * 2 CHUNKS ints.  `any_sampling` = 0 skips
+// passes 3 and 4 (every temperature <= 0).
+extern "C" int mlr_sample(const float* logits, int rows, int vocab, const float* temperature,
+                          const float* uniform, int32_t* tokens, int32_t* status, float* scratch_f,
+                          int32_t* scratch_i, int any_sampling, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    if (vocab <= 0) return -1;
+    return launch_sample(logits, rows, vocab, temperature, uniform, tokens, status, scratch_f, scratch_i, any_sampling,
+                         stream);
+}
+
+// ------------------------------------------------------------------------------------------------
+// The same without workspace arguments (no_alloc.h).  `scratch` is part of this library's code object; every
+// GPU that loads it holds a copy at an address of its own.  In host code the array's NAME is only a stand-in
+// for the symbol, not a device address: the address on the current device is asked for once per device and
+// kept, and only that pointer is ever handed to a kernel.
+static_assert(CHUNKS == 64, "no_alloc.h states the scratch size for 64 chunks");
+static __device__ __align__(256) unsigned char scratch[MLR_SAMPLE_STATIC_BYTES];
+
+#define MLR_MAX_DEVICES 64
+static void* g_scratch_on_device[MLR_MAX_DEVICES];        // [device index] -> address of `scratch` there, or null
+static std::mutex g_scratch_lock;
+
+static int scratch_on_current_device(unsigned char** out) {
+    int device = -1;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= MLR_MAX_DEVICES) return MLR_SAMPLE_STATIC_NO_DEVICE;
+    std::lock_guard<std::mutex> guard(g_scratch_lock);
+    if (g_scratch_on_device[device] == nullptr) {
+        void* address = nullptr;
+        const hipError_t err = hipGetSymbolAddress(&address, HIP_SYMBOL(scratch));     // (with `device` current)
+        if (err != hipSuccess || address == nullptr) {
+            fprintf(stderr, "mlr_sample_static: hipGetSymbolAddress failed on device %d: %s\n", device,
+                    hipGetErrorString(err));
+            return MLR_SAMPLE_STATIC_NO_SYMBOL;
+        }
+        g_scratch_on_device[device] = address;
+    }
+    *out = static_cast<unsigned char*>(g_scratch_on_device[device]);
+    return 0;
+}
+
+extern "C" int mlr_sample_static(const float* logits, int rows, int vocab, const float* temperature,
+                                 const float* uniform, int32_t* tokens, int32_t* status, int any_sampling,
+                                 hipStream_t stream) {
+    if (rows > MLR_SAMPLE_STATIC_MAX_ROWS) {
+        fprintf(stderr, "mlr_sample_static: %d rows exceed the %d that the static scratch memory holds\n", rows,
+                MLR_SAMPLE_STATIC_MAX_ROWS);
+        return MLR_SAMPLE_STATIC_TOO_MANY_ROWS;
+    }
+    unsigned char* base = nullptr;
+    const int rc = scratch_on_current_device(&base);
+    if (rc != 0) return rc;
+    if (rows <= 0) return 0;                               // the set-up call: the address is known now
+    if (vocab <= 0) return MLR_SAMPLE_STATIC_BAD_VOCAB;
+    float* scratch_f = reinterpret_cast<float*>(base);
+    int32_t* scratch_i = reinterpret_cast<int32_t*>(base + (size_t)MLR_SAMPLE_STATIC_MAX_ROWS * (2 * CHUNKS + 1) * sizeof(float));
+    return launch_sample(logits, rows, vocab, temperature, uniform, tokens, status, scratch_f, scratch_i, any_sampling,
+                         stream);
 }

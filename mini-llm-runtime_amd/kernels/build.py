@@ -33,7 +33,7 @@ HIP_LIBRARIES = {
     "attention": (["attention.hip"], ["common.h"], True),
     "gemm": (["gemm.hip"], ["common.h"], True),
     "attention_tiles": (["attention_tiles.hip"], [], False),      # bfloat16 only by nature
-    "sampling": (["sampling.hip"], [], False),
+    "sampling": (["sampling.hip"], ["no_alloc.h"], False),
     "library_gemm": (["library_gemm.hip"], [], False, ["-lhipblaslt"]),      # host code around hipBLASLt
 }
 HOST_LIBRARIES = {
