@@ -207,6 +207,31 @@ __global__ void silu_mul_kernel(const elem_t* __restrict__ gate_up, elem_t* __re
     }
 }
 
+// The first half of an RMSNorm whose scale is applied by the projection that follows (few rows): x = h + delta
+// (delta may be null; written back to h when write_h), out = elem(x * weight) WITHOUT the scale, and the row's
+// sum of squares ss[r] (one "partial" sum a row).  One workgroup per row, sums in a fixed order.
+__global__ void rows_prenorm_kernel(float* __restrict__ h, const elem_t* __restrict__ delta,
+                                    const float* __restrict__ weight, elem_t* __restrict__ out,
+                                    float* __restrict__ ss, int width) {
+    __shared__ float scratch[16];
+    const int r = blockIdx.x;
+    float* hrow = h + (size_t)r * width;
+    const elem_t* drow = delta ? delta + (size_t)r * width : nullptr;
+    elem_t* orow = out + (size_t)r * width;
+    float sum = 0.f;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) {
+        float x = hrow[i];
+        if (drow) {
+            x += to_float(drow[i]);
+            hrow[i] = x;
+        }
+        sum += x * x;
+        orow[i] = from_float<elem_t>(x * weight[i]);
+    }
+    sum = block_sum(sum, scratch);
+    if (threadIdx.x == 0) ss[r] = sum;
+}
+
 // The check of the hidden state (a debug mode; the reference runs the like after every layer and poisons
 // its runtime, src/minillm/cuda/layer.cpp:71, src/minillm/cuda/ops.cu:29-43).  status[0] collects bits
 // (1: a NaN, 2: an infinity), status[1] the smallest (layer << 20 | row) at which one was seen.
@@ -269,6 +294,13 @@ int mlr_add_rmsnorm(float* h, const void* delta, const float* weight, void* out,
     }
     add_rmsnorm_kernel<<<n_out, 256, 0, stream>>>(h, (const elem_t*)delta, weight, (elem_t*)out, rows,
                                                   width, eps, write_h);
+    return (int)hipGetLastError();
+}
+
+int mlr_rows_prenorm(float* h, const void* delta, const float* weight, void* out, float* ss, int rows, int width,
+                     hipStream_t stream) {
+    if (rows <= 0) return 0;
+    rows_prenorm_kernel<<<rows, 256, 0, stream>>>(h, (const elem_t*)delta, weight, (elem_t*)out, ss, width);
     return (int)hipGetLastError();
 }
 

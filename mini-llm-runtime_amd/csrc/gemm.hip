@@ -184,13 +184,41 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_bf16_kernel(
 #define SKINNY_WAVES 8
 #define SKINNY_STAGE_PITCH(U) ((U) * 128 + 16)        // bytes a row of the staged activation takes
 #define SKINNY_STAGE_LDS (66 * 1024)                  // the most dynamic LDS a workgroup asks for
-template <int MT, bool OUT_FLOAT, bool GATED, int UMAX = 4, bool STAGE = false>   // UMAX: the most groups of k a turn takes
+
+// What a skinny product of up to 16 rows may do with its sums before it stores them: the two halves of an
+// RMSNorm that is handed from the projection before it to the projection after it.
+//   EPI_SCALE (the projection after the norm): its input is x * norm_w, rounded, WITHOUT the row's scale
+//     rsqrt(mean(x^2) + eps), because whoever produced x knew only partial sums of squares; the scale is a
+//     factor per row, so it is applied here, in 32-bit, to the finished sums: out[m] *= rsqrt(sum_p ss[m][p] *
+//     inv_size + eps).  The partial sums are added in a fixed order (see the kernel).
+//   EPI_RESIDUAL (the projection before the norm, which ends a mixer or a feed-forward): its sums are added
+//     to the residual stream, h[m][n] += out[m][n], in 32-bit and in place (every element belongs to one
+//     lane); when a norm follows (next_w != null) it also writes x_out = bf16(h * next_w) and, per row and
+//     workgroup (16 columns), the sum of squares of its 16 new values of h: ss_out[m][workgroup].
+#define EPI_NONE 0
+#define EPI_SCALE 1
+#define EPI_RESIDUAL 2
+struct SkinnyEpilogue {
+    const float* ss;          // EPI_SCALE: [M][ss_parts] partial sums of squares of the rows
+    int ss_parts;
+    float eps, inv_size;
+    float* h;                 // EPI_RESIDUAL: [M][N] the residual stream
+    const float* next_w;      // [N] weights of the norm that follows, or null
+    __bf16* x_out;            // [M][N]
+    float* ss_out;            // [M][gridDim.x]
+};
+
+template <int MT, bool OUT_FLOAT, bool GATED, int UMAX = 4, bool STAGE = false, int EPI = EPI_NONE>   // UMAX: the most groups of k a turn takes
 __global__ __launch_bounds__(SKINNY_WAVES * 64) void gemm_skinny_kernel(const __bf16* __restrict__ a,
                                                                const __bf16* __restrict__ w,
-                                                               void* __restrict__ out_raw, int M, int N, int K) {
+                                                               void* __restrict__ out_raw, int M, int N, int K,
+                                                               SkinnyEpilogue epi) {
     constexpr int NW = GATED ? 2 : 1;
     static_assert(!STAGE || MT == 1, "the activation is staged for at most 16 rows");
+    static_assert(EPI == EPI_NONE || MT == 1, "the norm is handed over for at most 16 rows");
+    static_assert(EPI != EPI_RESIDUAL || (!GATED && !OUT_FLOAT), "the residual sum follows a plain projection");
     __shared__ float part[SKINNY_WAVES - 1][NW][MT][64][4];
+    __shared__ float ss_lds[SKINNY_WAVES][16];
     extern __shared__ __attribute__((aligned(16))) char staged[];   // [SKINNY_WAVES][M][pitch] when STAGE
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r16 = lane & 15, b = lane >> 4;
@@ -199,6 +227,31 @@ __global__ __launch_bounds__(SKINNY_WAVES * 64) void gemm_skinny_kernel(const __
     const int steps = (K + 31) / 32;
     const int per_wave = (steps + SKINNY_WAVES - 1) / SKINNY_WAVES;
     const int s_begin = wave * per_wave, s_end = min(steps, s_begin + per_wave);
+    // What the epilogue needs from memory is asked for here, before the weight, by every wavefront alike
+    // (no branch around a load); only wavefront 0 uses it.
+    float ss_mine = 0.f;                                   // EPI_SCALE: this lane's share of the row's partial sums
+    float4 h4 = make_float4(0.f, 0.f, 0.f, 0.f), nw4 = h4;  // EPI_RESIDUAL: h and the next norm's weights at (row r16, columns n0 + 4 b ..)
+    if constexpr (EPI == EPI_SCALE) {
+        // the row's partial sums are dealt out to the 32 (wavefront, lane block) pairs in runs of q; a run is
+        // added in ascending order, the four runs of a wavefront as (0 + 1) + (2 + 3), the wavefronts in the
+        // order 0..7: an order that depends on nothing but the number of partial sums
+        const int q = (epi.ss_parts + 4 * SKINNY_WAVES - 1) / (4 * SKINNY_WAVES);
+        const float* row = epi.ss + (size_t)min(r16, M - 1) * epi.ss_parts;
+        const int first = (wave * 4 + b) * q;
+        for (int j = 0; j < q; ++j) {
+            const int at = first + j;
+            const float v = row[min(at, epi.ss_parts - 1)];
+            ss_mine += at < epi.ss_parts ? v : 0.f;
+        }
+    }
+    if constexpr (EPI == EPI_RESIDUAL) {
+        const int n = min(n0 + 4 * b, max(N - 4, 0));      // (clamped: a narrow last strip is handled element by element below)
+        const size_t at = (size_t)min(r16, M - 1) * N + n;
+        if ((N & 3) == 0) {
+            h4 = *reinterpret_cast<const float4*>(epi.h + at);
+            if (epi.next_w) nw4 = *reinterpret_cast<const float4*>(epi.next_w + n);
+        }
+    }
     floatx4 acc[NW][MT];
 #pragma unroll
     for (int g = 0; g < NW; ++g)
@@ -308,11 +361,23 @@ __global__ __launch_bounds__(SKINNY_WAVES * 64) void gemm_skinny_kernel(const __
 #pragma unroll
                 for (int r = 0; r < 4; ++r) part[wave - 1][g][i][lane][r] = acc[g][i][r];
     }
+    if constexpr (EPI == EPI_SCALE) {
+        ss_mine += __shfl_xor(ss_mine, 16, MLR_WAVE);
+        ss_mine += __shfl_xor(ss_mine, 32, MLR_WAVE);
+        if (b == 0) ss_lds[wave][r16] = ss_mine;
+    }
     __syncthreads();
     if (wave != 0) return;
+    float row_scale = 1.f;
+    if constexpr (EPI == EPI_SCALE) {
+        float total = 0.f;
+#pragma unroll
+        for (int i = 0; i < SKINNY_WAVES; ++i) total += ss_lds[i][r16];
+        row_scale = 1.0f / sqrtf(total * epi.inv_size + epi.eps);
+    }
+    float y4[MT][4];
 #pragma unroll
     for (int i = 0; i < MT; ++i) {
-        const int m = 16 * i + r16;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             float v[NW];
@@ -320,160 +385,94 @@ __global__ __launch_bounds__(SKINNY_WAVES * 64) void gemm_skinny_kernel(const __
             for (int g = 0; g < NW; ++g) {
                 v[g] = acc[g][i][r];
                 for (int p = 0; p < SKINNY_WAVES - 1; ++p) v[g] += part[p][g][i][lane][r];
+                if constexpr (EPI == EPI_SCALE) v[g] *= row_scale;
             }
             float y = v[0];
             if (GATED) y = (v[0] / (1.0f + expf(-v[0]))) * v[NW - 1];
+            y4[i][r] = y;
+        }
+    }
+    if constexpr (EPI == EPI_RESIDUAL) {
+        // this lane: row r16, columns n0 + 4 b .. + 3 of h
+        const int n = n0 + 4 * b;
+        const bool row_ok = r16 < M;
+        float x[4];
+        float sq = 0.f;
+        if ((N & 3) == 0) {
+            const bool ok = row_ok && n < N;
+            const float hv[4] = {h4.x, h4.y, h4.z, h4.w}, wv[4] = {nw4.x, nw4.y, nw4.z, nw4.w};
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                x[r] = ok ? hv[r] + y4[0][r] : 0.f;
+                sq += x[r] * x[r];
+            }
+            if (ok) {
+                *reinterpret_cast<float4*>(epi.h + (size_t)r16 * N + n) = make_float4(x[0], x[1], x[2], x[3]);
+                if (epi.next_w) {
+                    typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;
+                    *reinterpret_cast<bf16x4*>(epi.x_out + (size_t)r16 * N + n) =
+                        bf16x4{(__bf16)(x[0] * wv[0]), (__bf16)(x[1] * wv[1]), (__bf16)(x[2] * wv[2]), (__bf16)(x[3] * wv[3])};
+                }
+            }
+        } else {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const bool ok = row_ok && n + r < N;
+                const size_t at = (size_t)min(r16, M - 1) * N + min(n + r, N - 1);
+                x[r] = ok ? epi.h[at] + y4[0][r] : 0.f;
+                sq += x[r] * x[r];
+                if (ok) {
+                    epi.h[at] = x[r];
+                    if (epi.next_w) epi.x_out[at] = (__bf16)(x[r] * epi.next_w[n + r]);
+                }
+            }
+        }
+        if (epi.next_w) {
+            sq += __shfl_xor(sq, 16, MLR_WAVE);            // (0 + 1) + (2 + 3) over the lane blocks: the strip's 16 columns
+            sq += __shfl_xor(sq, 32, MLR_WAVE);
+            if (b == 0 && row_ok) epi.ss_out[(size_t)r16 * gridDim.x + blockIdx.x] = sq;
+        }
+        return;
+    }
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+        const int m = 16 * i + r16;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
             const int n = n0 + 4 * b + r;
             if (m < M && n < N) {
-                if (OUT_FLOAT) ((float*)out_raw)[(size_t)m * N + n] = y;
-                else ((__bf16*)out_raw)[(size_t)m * N + n] = (__bf16)y;
+                if (OUT_FLOAT) ((float*)out_raw)[(size_t)m * N + n] = y4[i][r];
+                else ((__bf16*)out_raw)[(size_t)m * N + n] = (__bf16)y4[i][r];
             }
         }
     }
 }
 
-// Up to 16 rows: the residual add and the RMSNorm that precede a projection, done inside it.
-//   x = h_in + delta (delta may be null);  h_out = x (written by workgroup 0; h_out != h_in);
-//   out = (bf16((x * rsqrt(mean(x^2) + eps)) * norm_w)) . w^T      [GATED: silu(. gate) * (. up)]
-// Every workgroup recomputes the norm of the few rows (they come from the L2 cache); each wavefront
-// holds the slice of x that belongs to its part of k, the sums of squares meet in LDS and are added in
-// the order of the wavefronts.  K <= 2048 (a lane keeps its slice in registers).
-#define NORM_MAX_STEPS 8                              // 32-wide k steps per wavefront: K <= 8 * 8 * 32
-template <bool GATED, int PW>                         // PW: k steps a wavefront takes (1, 2, 4 or 8)
-__global__ __launch_bounds__(SKINNY_WAVES * 64) void gemm_skinny_norm_kernel(
-    const float* __restrict__ h_in, const __bf16* __restrict__ delta, const float* __restrict__ norm_w, float eps,
-    float* __restrict__ h_out, const __bf16* __restrict__ w, __bf16* __restrict__ out, int M, int N, int K) {
-    constexpr int NW = GATED ? 2 : 1;
-    __shared__ float part[SKINNY_WAVES - 1][NW][64][4];
-    __shared__ float sumsq[SKINNY_WAVES][16];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int r16 = lane & 15, b = lane >> 4;
-    const int n0 = blockIdx.x * 16;
-    const int steps = K / 32;                         // K % 32 == 0
-    const int s_begin = wave * PW, s_end = min(steps, s_begin + PW);
-    const bool row_ok = r16 < M;
-
-    // Every load is asked for here, before anything waits and with no branch in between, in the order of
-    // need (loads come back in the order they were asked for): the rows, which the sums of squares wait
-    // for and which come from the cache; the norm's weights; the weight, which comes from memory and
-    // flies while the norm is computed.  A step beyond the end of k and a row beyond M read a valid
-    // place and count as zero; without a delta the load reads the rows' own memory (which is longer)
-    // and its value is dropped.
-    const __bf16* delta_or_any = delta ? delta : reinterpret_cast<const __bf16*>(h_in);
-    float4 a0[PW], a1[PW];
-    bf16x8 d8[PW];
-#pragma unroll
-    for (int i = 0; i < PW; ++i) {
-        const size_t at = (size_t)min(r16, M - 1) * K + min(s_begin + i, steps - 1) * 32 + b * 8;
-        a0[i] = *reinterpret_cast<const float4*>(h_in + at);
-        a1[i] = *reinterpret_cast<const float4*>(h_in + at + 4);
-        d8[i] = *reinterpret_cast<const bf16x8*>(delta_or_any + at);
-    }
-    float4 nw0[PW], nw1[PW];
-#pragma unroll
-    for (int i = 0; i < PW; ++i) {
-        const int k = min(s_begin + i, steps - 1) * 32 + b * 8;
-        nw0[i] = *reinterpret_cast<const float4*>(norm_w + k);
-        nw1[i] = *reinterpret_cast<const float4*>(norm_w + k + 4);
-    }
-    bf16x8 wf[NW][PW];
-#pragma unroll
-    for (int i = 0; i < PW; ++i) {
-        const int k = min(s_begin + i, steps - 1) * 32 + b * 8;
-#pragma unroll
-        for (int g = 0; g < NW; ++g)
-            wf[g][i] = *reinterpret_cast<const bf16x8*>(w + ((size_t)g * N + min(n0 + r16, N - 1)) * K + k);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    float x[PW][8];
-    float sq = 0.f;
-#pragma unroll
-    for (int i = 0; i < PW; ++i) {
-        const bool valid = s_begin + i < s_end && row_ok;
-        const float a[8] = {a0[i].x, a0[i].y, a0[i].z, a0[i].w, a1[i].x, a1[i].y, a1[i].z, a1[i].w};
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const float v = delta ? a[e] + (float)d8[i][e] : a[e];
-            x[i][e] = valid ? v : 0.f;
-        }
-        if (h_out && blockIdx.x == 0 && valid) {
-            const size_t at = (size_t)r16 * K + (s_begin + i) * 32 + b * 8;
-            *reinterpret_cast<float4*>(h_out + at) = make_float4(x[i][0], x[i][1], x[i][2], x[i][3]);
-            *reinterpret_cast<float4*>(h_out + at + 4) = make_float4(x[i][4], x[i][5], x[i][6], x[i][7]);
-        }
-#pragma unroll
-        for (int e = 0; e < 8; ++e) sq += x[i][e] * x[i][e];
-    }
-    sq += __shfl_xor(sq, 16, MLR_WAVE);
-    sq += __shfl_xor(sq, 32, MLR_WAVE);
-    if (b == 0) sumsq[wave][r16] = sq;
-    __syncthreads();
-    float total = 0.f;
-#pragma unroll
-    for (int i = 0; i < SKINNY_WAVES; ++i) total += sumsq[i][r16];
-    const float scale = 1.0f / sqrtf(total / (float)K + eps);
-
-    floatx4 acc[NW];
-#pragma unroll
-    for (int g = 0; g < NW; ++g) acc[g] = floatx4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int i = 0; i < PW; ++i) {
-        const int s = s_begin + i;
-        if (s >= s_end) break;
-        const float nw[8] = {nw0[i].x, nw0[i].y, nw0[i].z, nw0[i].w, nw1[i].x, nw1[i].y, nw1[i].z, nw1[i].w};
-        bf16x8 xf;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) xf[e] = (__bf16)((x[i][e] * scale) * nw[e]);
-#pragma unroll
-        for (int g = 0; g < NW; ++g)
-            acc[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[g][i], xf, acc[g], 0, 0, 0);
-    }
-    if (wave > 0) {
-#pragma unroll
-        for (int g = 0; g < NW; ++g)
-#pragma unroll
-            for (int r = 0; r < 4; ++r) part[wave - 1][g][lane][r] = acc[g][r];
-    }
-    __syncthreads();
-    if (wave != 0) return;
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-        float v[NW];
-#pragma unroll
-        for (int g = 0; g < NW; ++g) {
-            v[g] = acc[g][r];
-            for (int p = 0; p < SKINNY_WAVES - 1; ++p) v[g] += part[p][g][lane][r];
-        }
-        float y = v[0];
-        if (GATED) y = (v[0] / (1.0f + expf(-v[0]))) * v[NW - 1];
-        const int n = n0 + 4 * b + r;
-        if (row_ok && n < N) out[(size_t)r16 * N + n] = (__bf16)y;
-    }
-}
-
-template <int MT, bool OUT_FLOAT, bool GATED, int UMAX, bool STAGE>
+template <int MT, bool OUT_FLOAT, bool GATED, int UMAX, bool STAGE, int EPI>
 static int launch_skinny_kernel(const void* a, const void* w, void* out, int M, int N, int K, size_t lds,
-                                hipStream_t stream) {
-    auto* kernel = gemm_skinny_kernel<MT, OUT_FLOAT, GATED, UMAX, STAGE>;
+                                const SkinnyEpilogue& epi, hipStream_t stream) {
+    auto* kernel = gemm_skinny_kernel<MT, OUT_FLOAT, GATED, UMAX, STAGE, EPI>;
     if (STAGE) {                                          // static and dynamic LDS together may pass 64 KB
         static const hipError_t allowed = hipFuncSetAttribute(
             reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, SKINNY_STAGE_LDS);
         if (allowed != hipSuccess) return (int)allowed;
     }
-    kernel<<<dim3((N + 15) / 16), SKINNY_WAVES * 64, lds, stream>>>((const __bf16*)a, (const __bf16*)w, out, M, N, K);
+    kernel<<<dim3((N + 15) / 16), SKINNY_WAVES * 64, lds, stream>>>((const __bf16*)a, (const __bf16*)w, out, M, N, K, epi);
     return (int)hipGetLastError();
 }
 
-template <int MT, bool GATED, int UMAX, bool STAGE>
+template <int MT, bool GATED, int UMAX, bool STAGE, int EPI>
 static int launch_skinny_as(const void* a, const void* w, void* out, int M, int N, int K, int out_float,
-                            size_t lds, hipStream_t stream) {
-    if (out_float) return launch_skinny_kernel<MT, true, GATED, UMAX, STAGE>(a, w, out, M, N, K, lds, stream);
-    return launch_skinny_kernel<MT, false, GATED, UMAX, STAGE>(a, w, out, M, N, K, lds, stream);
+                            size_t lds, const SkinnyEpilogue& epi, hipStream_t stream) {
+    if constexpr (EPI == EPI_NONE) {
+        if (out_float) return launch_skinny_kernel<MT, true, GATED, UMAX, STAGE, EPI>(a, w, out, M, N, K, lds, epi, stream);
+    }
+    return launch_skinny_kernel<MT, false, GATED, UMAX, STAGE, EPI>(a, w, out, M, N, K, lds, epi, stream);
 }
 
-template <int MT, bool GATED>
+template <int MT, bool GATED, int EPI = EPI_NONE>
 static int launch_skinny(const void* a, const void* w, void* out, int M, int N, int K, int out_float,
-                         hipStream_t stream) {
+                         hipStream_t stream, const SkinnyEpilogue& epi = SkinnyEpilogue{}) {
     // A short k (at most two groups of 64 a wavefront) takes the variant whose turns hold two groups: it
     // needs fewer registers, so more of its short-lived workgroups fit a compute unit.
     const bool short_k = MT * (GATED ? 2 : 1) <= 2 && K <= 64 * 2 * SKINNY_WAVES;
@@ -483,10 +482,10 @@ static int launch_skinny(const void* a, const void* w, void* out, int M, int N, 
         // within the registers of two workgroups a compute unit, gains nothing.)
         const size_t lds = (size_t)SKINNY_WAVES * M * SKINNY_STAGE_PITCH(4);
         if (M >= 2 && K % 64 == 0 && K > 2048 && lds <= SKINNY_STAGE_LDS)
-            return launch_skinny_as<MT, GATED, 4, true>(a, w, out, M, N, K, out_float, lds, stream);
+            return launch_skinny_as<MT, GATED, 4, true, EPI>(a, w, out, M, N, K, out_float, lds, epi, stream);
     }
-    if (short_k) return launch_skinny_as<MT, GATED, 2, false>(a, w, out, M, N, K, out_float, 0, stream);
-    return launch_skinny_as<MT, GATED, 4, false>(a, w, out, M, N, K, out_float, 0, stream);
+    if (short_k) return launch_skinny_as<MT, GATED, 2, false, EPI>(a, w, out, M, N, K, out_float, 0, epi, stream);
+    return launch_skinny_as<MT, GATED, 4, false, EPI>(a, w, out, M, N, K, out_float, 0, epi, stream);
 }
 
 // Many rows (prompt portions), K a multiple of 64: 32x32 tiles of v_mfma_f32_32x32x16_bf16, the operands
@@ -838,30 +837,35 @@ extern "C" int mlr_gemm_gated_silu(const void* a, const void* w, void* out, int 
     return 1;
 }
 
-// Residual add + RMSNorm + projection in one launch, for M <= 16, K % 32 == 0, K <= 2048 (see the kernel).
-// gated != 0: w is [2N, K] = [gate; up] and out = silu(gate) * up.
-extern "C" int mlr_norm_gemm(const float* h_in, const void* delta, const float* norm_w, float eps, float* h_out,
-                             const void* w, void* out, int M, int N, int K, int gated, hipStream_t stream) {
+// The two halves of an RMSNorm handed from one projection to the next, for M <= 16 (see SkinnyEpilogue).
+// out = rsqrt(sum_p ss[m][p] / norm_size + eps) * (x . w^T); gated != 0: w is [2N, K] = [gate; up] and
+// out = silu(scale * gate) * (scale * up).  x is bf16(h * norm_w) as `mlr_gemm_residual` or the row kernel
+// `mlr_rows_prenorm` left it.
+extern "C" int mlr_gemm_prenormed(const void* x, const float* ss, int ss_parts, float eps, int norm_size, const void* w,
+                                  void* out, int M, int N, int K, int gated, hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
-    if (M > 16 || K <= 0 || K % 32 != 0 || K > 32 * SKINNY_WAVES * NORM_MAX_STEPS) return -1;
-    if (h_out == h_in) return -2;
-    dim3 grid((N + 15) / 16);
-    const int per_wave = (K / 32 + SKINNY_WAVES - 1) / SKINNY_WAVES;
-#define MLR_NORM_LAUNCH(G, PWV)                                                                      \
-    gemm_skinny_norm_kernel<G, PWV><<<grid, SKINNY_WAVES * 64, 0, stream>>>(                          \
-        h_in, (const __bf16*)delta, norm_w, eps, h_out, (const __bf16*)w, (__bf16*)out, M, N, K)
-    if (gated) {
-        if (per_wave <= 1) MLR_NORM_LAUNCH(true, 1);
-        else if (per_wave <= 2) MLR_NORM_LAUNCH(true, 2);
-        else if (per_wave <= 4) MLR_NORM_LAUNCH(true, 4);
-        else MLR_NORM_LAUNCH(true, 8);
-    } else {
-        if (per_wave <= 1) MLR_NORM_LAUNCH(false, 1);
-        else if (per_wave <= 2) MLR_NORM_LAUNCH(false, 2);
-        else if (per_wave <= 4) MLR_NORM_LAUNCH(false, 4);
-        else MLR_NORM_LAUNCH(false, 8);
-    }
-#undef MLR_NORM_LAUNCH
-    return (int)hipGetLastError();
+    if (M > 16 || K <= 0 || ss_parts <= 0 || norm_size <= 0 || ss == nullptr) return -1;
+    SkinnyEpilogue epi{};
+    epi.ss = ss;
+    epi.ss_parts = ss_parts;
+    epi.eps = eps;
+    epi.inv_size = 1.0f / (float)norm_size;
+    if (gated) return launch_skinny<1, true, EPI_SCALE>(x, w, out, M, N, K, 0, stream, epi);
+    return launch_skinny<1, false, EPI_SCALE>(x, w, out, M, N, K, 0, stream, epi);
+}
+
+// h[M, N] += a[M, K] . w[N, K]^T in 32-bit, in place.  With next_w != null also x_out[M, N] = bf16(h * next_w)
+// and ss_out[M, ceil(N / 16)]: per row and strip of 16 columns the sum of squares of the new h.
+extern "C" int mlr_gemm_residual(const void* a, const void* w, float* h, const float* next_w, void* x_out,
+                                 float* ss_out, int M, int N, int K, hipStream_t stream) {
+    if (M <= 0 || N <= 0) return 0;
+    if (M > 16 || K <= 0 || h == nullptr) return -1;
+    if (next_w != nullptr && (x_out == nullptr || ss_out == nullptr)) return -2;
+    SkinnyEpilogue epi{};
+    epi.h = h;
+    epi.next_w = next_w;
+    epi.x_out = (__bf16*)x_out;
+    epi.ss_out = ss_out;
+    return launch_skinny<1, false, EPI_RESIDUAL>(a, w, nullptr, M, N, K, 0, stream, epi);
 }
 #endif

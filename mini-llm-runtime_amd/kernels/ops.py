@@ -84,8 +84,16 @@ def _gemm_work(self, a, w, out, *rest, **kw):
     return _size(a) + _size(w) + _size(out), 2 * a.shape[0] * w.shape[0] * w.shape[1]
 
 
-def _norm_gemm_work(self, h_in, delta, norm_w, eps, h_out, w, out, *rest, **kw):
-    return _size(h_in) + _size(delta) + _size(h_out) + _size(w) + _size(out), 2 * h_in.shape[0] * w.shape[0] * w.shape[1]
+def _rows_prenorm_work(self, h, delta, weight, out, ss):
+    return 2 * _size(h) + _size(delta) + _size(out), 0
+
+
+def _prenormed_work(self, x, ss, eps, w, out, *rest, **kw):
+    return _size(x) + _size(ss) + _size(w) + _size(out), 2 * x.shape[0] * w.shape[0] * w.shape[1]
+
+
+def _residual_work(self, a, w, h, *rest, **kw):
+    return _size(a) + _size(w) + 2 * _size(h), 2 * a.shape[0] * w.shape[0] * w.shape[1]
 
 
 def _norm_work(self, h, delta, weight, out, eps, rows=None, write_h=True):
@@ -282,30 +290,70 @@ class Kernels:
         fn = self._lib("gemm").mlr_gemm_gated_silu
         _ok(fn(_p(a), _p(w), _p(out), _c_int(m), _c_int(two_n // 2), _c_int(k), _stream()), "gemm_gated_silu")
 
-    def norm_gemm_supported(self, rows, width):
-        """Whether `norm_gemm` (residual add + RMSNorm inside the projection) serves these sizes."""
-        return self.dtype == torch.bfloat16 and rows <= 16 and width % 32 == 0 and width <= 2048
+    # -- an RMSNorm handed from one projection to the next (few rows) ------------------------------
+    HANDOFF_MAX_ROWS = 16
 
-    @timed("gemm", _norm_gemm_work)
-    def norm_gemm(self, h_in, delta, norm_w, eps, h_out, w, out, gated=False):
-        """x = h_in + delta (delta may be None); h_out = x; out = rmsnorm(x, norm_w) . w^T, or with
-        gated=True (w = [gate; up] stacked) silu(. gate^T) * (. up^T).  For few rows: one launch instead
-        of two."""
-        _tensor(h_in, "h_in", torch.float32, ndim=2)
-        m, k = h_in.shape
-        _need(self.norm_gemm_supported(m, k), "norm_gemm: bfloat16, at most 16 rows, width % 32 == 0 and <= 2048")
+    def handoff_supported(self, rows):
+        """Whether the projections before and after a norm can share it between them: the bfloat16 engine, up to
+        16 rows.  The projection before the norm adds its sums to the residual stream h and leaves
+        x = bf16(h * norm_w) and partial sums of squares of h's rows (`gemm_residual`); the projection after it
+        multiplies its finished sums by the rows' scale rsqrt(mean(h^2) + eps) (`gemm_prenormed`): the scale is
+        a factor per row, so the product with it commutes with the projection."""
+        return self.dtype == torch.bfloat16 and 1 <= rows <= self.HANDOFF_MAX_ROWS
+
+    @staticmethod
+    def handoff_parts(width):
+        """Partial sums of squares a row that `gemm_residual` leaves for an output `width` wide."""
+        return (width + 15) // 16
+
+    @timed("norm", _rows_prenorm_work)
+    def rows_prenorm(self, h, delta, weight, out, ss):
+        """h += delta (delta may be None); out = T(h * weight), without the norm's scale; ss[r, 0] = sum(h[r]^2)."""
+        _tensor(h, "h", torch.float32, ndim=2)
+        m, width = h.shape
         if delta is not None:
-            _tensor(delta, "delta", self.dtype, (m, k))
-        _tensor(norm_w, "norm_w", torch.float32, (k,))
-        _tensor(h_out, "h_out", torch.float32, (m, k))
-        _need(h_out.data_ptr() != h_in.data_ptr(), "norm_gemm: h_out must not be h_in")
+            _tensor(delta, "delta", self.dtype, (m, width))
+        _tensor(weight, "weight", torch.float32, (width,))
+        _tensor(out, "out", self.dtype, (m, width))
+        _tensor(ss, "ss", torch.float32, (m, 1))
+        fn = self._lib("elementwise").mlr_rows_prenorm
+        _ok(fn(_p(h), _p(delta), _p(weight), _p(out), _p(ss), _c_int(m), _c_int(width), _stream()), "rows_prenorm")
+
+    @timed("gemm", _prenormed_work)
+    def gemm_prenormed(self, x, ss, eps, w, out, gated=False):
+        """out = rsqrt(sum(ss[m]) / K + eps) * (x . w^T), x being T(h * norm_w) [M, K] and ss [M, parts] partial
+        sums of squares of h's rows; gated=True (w = [gate; up] stacked): silu(scale * gate) * (scale * up)."""
+        _tensor(x, "x", self.dtype, ndim=2)
+        m, k = x.shape
+        _need(self.handoff_supported(m), "gemm_prenormed: bfloat16, at most 16 rows")
+        _tensor(ss, "ss", torch.float32, ndim=2)
+        _need(ss.shape[0] == m and ss.shape[1] >= 1, "gemm_prenormed: one row of partial sums per row of x")
         _tensor(w, "w", self.dtype, ndim=2)
         n = w.shape[0] // 2 if gated else w.shape[0]
-        _need(w.shape[1] == k and (not gated or w.shape[0] % 2 == 0), "norm_gemm: weight does not fit")
+        _need(w.shape[1] == k and (not gated or w.shape[0] % 2 == 0), "gemm_prenormed: weight does not fit")
         _tensor(out, "out", self.dtype, (m, n))
-        fn = self._lib("gemm").mlr_norm_gemm
-        _ok(fn(_p(h_in), _p(delta), _p(norm_w), _c_float(eps), _p(h_out), _p(w), _p(out), _c_int(m), _c_int(n),
-               _c_int(k), _c_int(1 if gated else 0), _stream()), "norm_gemm")
+        fn = self._lib("gemm").mlr_gemm_prenormed
+        _ok(fn(_p(x), _p(ss), _c_int(ss.shape[1]), _c_float(eps), _c_int(k), _p(w), _p(out), _c_int(m), _c_int(n),
+               _c_int(k), _c_int(1 if gated else 0), _stream()), "gemm_prenormed")
+
+    @timed("gemm", _residual_work)
+    def gemm_residual(self, a, w, h, next_w=None, x_out=None, ss_out=None):
+        """h += a . w^T (32-bit, in place).  With next_w (the weights of the norm that follows) also
+        x_out = T(h * next_w) and ss_out[m, p] = the sum of squares of h[m, 16 p : 16 p + 16]."""
+        _tensor(a, "a", self.dtype, ndim=2)
+        m, k = a.shape
+        _need(self.handoff_supported(m), "gemm_residual: bfloat16, at most 16 rows")
+        _tensor(w, "w", self.dtype, ndim=2)
+        n = w.shape[0]
+        _need(w.shape[1] == k, "gemm_residual: inner sizes differ")
+        _tensor(h, "h", torch.float32, (m, n))
+        if next_w is not None:
+            _tensor(next_w, "next_w", torch.float32, (n,))
+            _tensor(x_out, "x_out", self.dtype, (m, n))
+            _tensor(ss_out, "ss_out", torch.float32, (m, self.handoff_parts(n)))
+        fn = self._lib("gemm").mlr_gemm_residual
+        _ok(fn(_p(a), _p(w), _p(h), _p(next_w), _p(x_out if next_w is not None else None),
+               _p(ss_out if next_w is not None else None), _c_int(m), _c_int(n), _c_int(k), _stream()), "gemm_residual")
 
     # -- attention ---------------------------------------------------------------------------
     def _check_cache(self, k_pages, v_pages, kv_heads, head_dim, page_size):

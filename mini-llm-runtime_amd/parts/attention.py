@@ -9,7 +9,7 @@ import torch
 
 from ..cache.manager import KvSpec
 from ..weights.loader import WeightSpec, stacked
-from .registry import PartError, build_part, register_part
+from .registry import Handoff, PartError, build_part, register_part
 
 
 @register_part("mixer", "gqa_attention")
@@ -112,21 +112,32 @@ class GqaAttention:
         tiles = ["attention_tiles"] if self.qkv is not None and self.qkv.dtype == torch.bfloat16 else []
         return ["gemm", "rope_kv", "attention"] + tiles
 
-    def forward_prenorm(self, ctx, h, delta, norm, h_out, cache_id, write_cache=True):
-        """As `forward` on norm(h + delta), the residual add and the norm done inside the first
-        projection (few rows); h_out receives h + delta."""
+    def forward_handoff(self, ctx, hand, h, norm_after, cache_id, write_cache=True):
+        """As `forward` on the norm that `hand` describes, its scale applied inside the q/k/v projection; the
+        output projection adds into h and prepares `norm_after` (None: nothing follows)."""
         s = self.spec
         m = h.shape[0]
+        k = ctx.kernels
         qkv = ctx.workspace.get("qkv", (m, (s.q_heads + 2 * s.kv_heads) * s.head_dim), ctx.dtype)
-        ctx.kernels.norm_gemm(h, delta, norm.weight, norm.eps, h_out, self.qkv, qkv)
-        return self._attend(ctx, qkv, cache_id, write_cache)
+        k.gemm_prenormed(hand.x, hand.ss, hand.norm.eps, self.qkv, qkv)
+        attn = self._attend(ctx, qkv, cache_id, write_cache)
+        if norm_after is None:
+            k.gemm_residual(attn, self.o, h)
+            return None
+        x = ctx.workspace.get("handoff_x", (m, s.hidden), ctx.dtype)
+        ss = ctx.workspace.get("handoff_ss", (m, k.handoff_parts(s.hidden)), torch.float32)
+        k.gemm_residual(attn, self.o, h, norm_after.weight, x, ss)
+        return Handoff(norm_after, x, ss)
 
     def forward(self, ctx, x, cache_id, write_cache=True):
         s = self.spec
         m = x.shape[0]
         qkv = ctx.workspace.get("qkv", (m, (s.q_heads + 2 * s.kv_heads) * s.head_dim), x.dtype)
         ctx.kernels.gemm(x, self.qkv, qkv)
-        return self._attend(ctx, qkv, cache_id, write_cache)
+        attn = self._attend(ctx, qkv, cache_id, write_cache)
+        out = ctx.workspace.get("mixer_out", (m, s.hidden), x.dtype)
+        ctx.kernels.gemm(attn, self.o, out)
+        return out
 
     def _attention_work(self, ctx, element_size):
         """For the profile: (bytes, flops) of this step's attention, from the host's view of the contexts."""
@@ -149,6 +160,8 @@ class GqaAttention:
             self._work = None
 
     def _attend(self, ctx, qkv, cache_id, write_cache):
+        """Norm of q and k, rotation, cache write and attention on the fused projection's output; the heads'
+        outputs [B, q_heads * head_dim] (before the output projection)."""
         s = self.spec
         k = ctx.kernels
         if k.profiler is not None and not ctx.fixed_groups:
@@ -177,9 +190,7 @@ class GqaAttention:
                 self.k_norm.weight if self.k_norm is not None else None,
                 self.q_norm.eps if self.q_norm is not None else 0.0, rope, partial,
                 window=s.window, split_keys=split_keys, max_splits=max_splits)
-            out = ctx.workspace.get("mixer_out", (m, s.hidden), x.dtype)
-            k.gemm(attn, self.o, out)
-            return out
+            return attn
         q = ctx.workspace.get("q", (m, s.q_heads * s.head_dim), x.dtype)
         k.qk_norm_rope_kv(
             qkv, q, view.k_pages, view.v_pages, view.block_table, ctx.slots, ctx.positions,
@@ -231,6 +242,4 @@ class GqaAttention:
             k.paged_attention(q, view.k_pages, view.v_pages, view.block_table, ctx.slots, ctx.positions, attn,
                               s.q_heads, s.kv_heads, s.head_dim, view.page_size, float(s.scale),
                               window=s.window, split_keys=split_keys, max_splits=max_splits, partial=partial)
-        out = ctx.workspace.get("mixer_out", (m, s.hidden), x.dtype)
-        k.gemm(attn, self.o, out)
-        return out
+        return attn

@@ -4,7 +4,7 @@ fused with the norm that follows, so a block hands its last output on as `pendin
 adding it itself."""
 from __future__ import annotations
 
-from .registry import build_part, register_part
+from .registry import Handoff, build_part, register_part
 
 
 @register_part("block", "prenorm")
@@ -22,17 +22,22 @@ class PreNormBlock:
     def workspace_plan(self, rows, dtype, limits):
         import torch
         width = self.norm1.size
-        return {("hidden_alt", torch.float32): min(rows, 16) * width, ("normed", dtype): rows * width}
+        few = min(rows, 16)
+        return {("normed", dtype): rows * width, ("handoff_x", dtype): few * width,
+                ("handoff_ss", torch.float32): few * max(1, (width + 15) // 16)}
 
-    def forward(self, ctx, h, pending, cache_id, write_cache=True):
-        if (ctx.kernels.norm_gemm_supported(h.shape[0], h.shape[1])
-                and getattr(self.norm1, "fusable_rmsnorm", False) and getattr(self.norm2, "fusable_rmsnorm", False)
-                and hasattr(self.mixer, "forward_prenorm") and hasattr(self.ffn, "forward_prenorm")):
-            # few rows: each norm rides in the projection that follows it; the residual stream goes to a
-            # second buffer and back, so that no workgroup reads a row that another one is updating
-            h_alt = ctx.workspace.get("hidden_alt", tuple(h.shape), h.dtype)
-            mixed = self.mixer.forward_prenorm(ctx, h, pending, self.norm1, h_alt, cache_id, write_cache)
-            return self.ffn.forward_prenorm(ctx, h_alt, mixed, self.norm2, h)
+    def forward(self, ctx, h, pending, cache_id, write_cache=True, next_norm=None):
+        fusable = lambda norm: norm is not None and getattr(norm, "fusable_rmsnorm", False) and norm.size == h.shape[1]
+        if (ctx.kernels.handoff_supported(h.shape[0]) and fusable(self.norm1) and fusable(self.norm2)
+                and hasattr(self.mixer, "forward_handoff") and hasattr(self.ffn, "forward_handoff")):
+            # few rows: every norm is shared between the projection before it (which adds into h and leaves
+            # h * weight and partial sums of squares) and the projection after it (which applies the scale)
+            hand = pending if isinstance(pending, Handoff) and pending.norm is self.norm1 else \
+                self.norm1.prenorm(ctx, h, None if isinstance(pending, Handoff) else pending)
+            hand = self.mixer.forward_handoff(ctx, hand, h, self.norm2, cache_id, write_cache)
+            return self.ffn.forward_handoff(ctx, hand, h, next_norm if fusable(next_norm) else None)
+        if isinstance(pending, Handoff):                  # h is complete already
+            pending = None
         normed = ctx.workspace.get("normed", tuple(h.shape), ctx.dtype)
         self.norm1.forward(ctx, h, pending, normed)
         mixed = self.mixer.forward(ctx, normed, cache_id, write_cache)

@@ -5,7 +5,7 @@ from __future__ import annotations
 import torch
 
 from ..weights.loader import WeightSpec, stacked
-from .registry import PartError, register_part
+from .registry import Handoff, PartError, register_part
 
 
 @register_part("ffn", "swiglu")
@@ -36,15 +36,21 @@ class SwiGluMlp:
         return {("act", dtype): rows * s.intermediate, ("gate_up", dtype): rows * 2 * s.intermediate,
                 ("ffn_out", dtype): rows * s.hidden}
 
-    def forward_prenorm(self, ctx, h, delta, norm, h_out):
-        """As `forward` on norm(h + delta), add and norm done inside the first projection (few rows)."""
+    def forward_handoff(self, ctx, hand, h, norm_after):
+        """As `forward` on the norm that `hand` describes, its scale applied inside the first projection; the
+        second projection adds into h and prepares `norm_after` (None: nothing follows)."""
         s = self.spec
         m = h.shape[0]
+        k = ctx.kernels
         act = ctx.workspace.get("act", (m, s.intermediate), ctx.dtype)
-        ctx.kernels.norm_gemm(h, delta, norm.weight, norm.eps, h_out, self.gate_up, act, gated=True)
-        out = ctx.workspace.get("ffn_out", (m, s.hidden), ctx.dtype)
-        ctx.kernels.gemm(act, self.down, out)
-        return out
+        k.gemm_prenormed(hand.x, hand.ss, hand.norm.eps, self.gate_up, act, gated=True)
+        if norm_after is None:
+            k.gemm_residual(act, self.down, h)
+            return None
+        x = ctx.workspace.get("handoff_x", (m, s.hidden), ctx.dtype)
+        ss = ctx.workspace.get("handoff_ss", (m, k.handoff_parts(s.hidden)), torch.float32)
+        k.gemm_residual(act, self.down, h, norm_after.weight, x, ss)
+        return Handoff(norm_after, x, ss)
 
     def forward(self, ctx, x):
         s = self.spec

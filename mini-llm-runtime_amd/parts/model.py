@@ -13,7 +13,7 @@ import torch
 
 from ..config import load_config
 from ..weights.loader import WeightSpec, load_weights
-from .registry import PartError, build_part
+from .registry import Handoff, PartError, build_part
 
 
 def build_blocks(spec):
@@ -157,10 +157,15 @@ class DecoderModel:
             k.status_reset(status)
         k.embed_gather(ctx.token_ids, self.embed, h)
         pending = None
-        for i, run in enumerate(self.spec.schedule):
-            pending = self.blocks[run.layer].forward(ctx, h, pending, run.cache, run.write_cache)
+        schedule = self.spec.schedule
+        for i, run in enumerate(schedule):
+            # (the norm the next run starts with: a block may prepare it while it adds its last output into h)
+            next_norm = self.blocks[schedule[i + 1].layer].norm1 if i + 1 < len(schedule) else None
+            pending = self.blocks[run.layer].forward(ctx, h, pending, run.cache, run.write_cache, next_norm=next_norm)
+            if isinstance(pending, Handoff) and i + 1 == len(schedule):
+                pending = None                            # (h is complete)
             if status is not None:                        # h + pending is the hidden state after this run
-                k.finite_check(h, pending, i, status)
+                k.finite_check(h, None if isinstance(pending, Handoff) else pending, i, status)
         r = 0 if want_rows is None else want_rows.numel()
         if r == 0:
             return None

@@ -15,8 +15,16 @@ Interfaces (B = the tokens of a step, E = the model width, T = the engine's elem
                   forward(ctx, x, cache_id, write_cache) -> T [B, E], x being the normed input.
   feed-forward    weight_specs(), bind(), libraries();  forward(ctx, x) -> T [B, E].
   block           built from (norm1, mixer, norm2, ffn);  forward(ctx, h, pending, cache_id,
-                  write_cache) -> the next pending delta: a block adds `pending` (the previous
-                  block's last output) into h itself, fused with its first norm.
+                  write_cache, next_norm=None) -> the next pending delta: a block adds `pending`
+                  (the previous block's last output) into h itself, fused with its first norm.
+                  `pending` may also be a `Handoff` (h is complete and the first half of a norm is
+                  done); a block may return one for `next_norm`, the norm the next block starts with.
+  Optional, for steps of few rows (each falls back to forward when a part lacks it):
+  norm            handoff-capable norms set `fusable_rmsnorm = True` and offer
+                  prenorm(ctx, h, delta) -> Handoff.
+  mixer           forward_handoff(ctx, hand, h, norm_after, cache_id, write_cache) -> Handoff | None:
+                  the first projection takes `hand`, the last adds into h and prepares `norm_after`.
+  feed-forward    forward_handoff(ctx, hand, h, norm_after) -> Handoff | None, likewise.
 
 A part may set the class attribute `graph_safe = True` when what it launches depends only on the step's
 SHAPE -- how many tokens each entry brings (ctx.n_tokens, the lengths in ctx.segments, ctx.single_tokens,
@@ -30,7 +38,21 @@ No part is told which model it is in; sizes and constants arrive through its spe
 """
 from __future__ import annotations
 
+from dataclasses import dataclass
+
 _REGISTRIES = {"norm": {}, "position": {}, "mixer": {}, "ffn": {}, "block": {}}
+
+
+@dataclass
+class Handoff:
+    """A norm shared between the projection before it and the projection after it (few rows, see
+    `Kernels.handoff_supported`): the residual stream h is complete (nothing is pending), `x` holds
+    T(h * norm.weight) without the rows' scale and `ss` [rows, parts] partial sums of squares of h's rows.
+    Whoever runs the first projection after `norm` applies rsqrt(sum(ss) / width + norm.eps) to its sums
+    (`Kernels.gemm_prenormed`).  A block may hand one to the next block instead of a pending delta."""
+    norm: object
+    x: object
+    ss: object
 
 
 class PartError(ValueError):

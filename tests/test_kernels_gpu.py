@@ -698,32 +698,91 @@ def test_silu_mul_wide(dtype, inter):
     torch.testing.assert_close(act.double(), g / (1 + torch.exp(-g)) * u, **tol(dtype))
 
 
+@pytest.mark.parametrize("rows,width", [(1, 64), (8, 1024), (16, 100), (5, 97), (3, 4096)])
+def test_rows_prenorm(rows, width):
+    """The first half of a norm that is handed to the projection after it: h += delta, out = bf16(h * w) without
+    the scale, and the rows' sums of squares."""
+    k = kernels(torch.bfloat16)
+    h0 = rnd((rows, width), torch.float32, 94, 2.0)
+    delta = rnd((rows, width), torch.bfloat16, 95)
+    nw = rnd((width,), torch.float32, 96) + 1
+    for d in (delta, None):
+        h = h0.clone()
+        out = torch.full((rows, width), float("nan"), dtype=torch.bfloat16, device="cuda")
+        ss = torch.full((rows, 1), float("nan"), device="cuda")
+        k.rows_prenorm(h, d, nw, out, ss)
+        x = h0.double() + (d.double() if d is not None else 0)
+        torch.testing.assert_close(h.double(), x, atol=1e-6, rtol=1e-6)
+        torch.testing.assert_close(out.double(), (x * nw.double()).to(torch.bfloat16).double(), atol=0, rtol=2 ** -7)
+        torch.testing.assert_close(ss[:, 0].double(), (x * x).sum(-1), rtol=1e-5, atol=1e-5)
+
+
 @pytest.mark.parametrize("gated", [False, True])
-@pytest.mark.parametrize("mnk", [(1, 48, 64), (8, 4096, 1024), (16, 100, 1024), (5, 208, 96), (3, 40, 2048), (7, 24, 32)])
-def test_norm_gemm(mnk, gated):
-    """Residual add + RMSNorm inside the projection (few rows, bfloat16): h_out = h + delta and
-    out = rmsnorm(h + delta) W^T (or the gated activation of two such products)."""
+@pytest.mark.parametrize("mnk,parts", [((1, 48, 64), 1), ((8, 4096, 1024), 64), ((16, 100, 1024), 3), ((5, 208, 96), 6),
+                                       ((3, 40, 4096), 256), ((7, 24, 32), 2), ((2, 50, 100), 7), ((16, 333, 2048), 128)])
+def test_projection_after_a_handed_over_norm(mnk, parts, gated):
+    """`gemm_prenormed`: the rows' scale rsqrt(sum of the partial sums / K + eps), applied to the finished sums
+    of x . w^T (or inside the gated activation), equals the projection of the normed rows."""
     m, n, kk = mnk
     k = kernels(torch.bfloat16)
-    assert k.norm_gemm_supported(m, kk) and not k.norm_gemm_supported(17, kk) and not k.norm_gemm_supported(m, 40)
-    h = rnd((m, kk), torch.float32, 90, 2.0)
-    delta = rnd((m, kk), torch.bfloat16, 91)
+    assert k.handoff_supported(m) and not k.handoff_supported(17) and not kernels(torch.float32).handoff_supported(m)
+    xf = rnd((m, kk), torch.float32, 90, 2.0)
     nw = rnd((kk,), torch.float32, 92) + 1
+    x = (xf * nw).to(torch.bfloat16)
+    # the rows' sums of squares, cut into parts of any sizes (some of them zero)
+    cuts = torch.linspace(0, kk, parts + 1).long().tolist()
+    ss = torch.stack([(xf[:, a:b].double() ** 2).sum(-1) for a, b in zip(cuts, cuts[1:])], dim=1).float().contiguous()
     w = rnd(((2 if gated else 1) * n, kk), torch.bfloat16, 93, 0.2)
     eps = 1e-5
-    for d in (delta, None):
-        h_out = torch.full((m, kk), float("nan"), device="cuda")
-        out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
-        k.norm_gemm(h, d, nw, eps, h_out, w, out, gated=gated)
-        x = h.double() + (d.double() if d is not None else 0)
-        torch.testing.assert_close(h_out.double(), x, atol=1e-6, rtol=1e-6)
-        xn = (x * torch.rsqrt((x * x).mean(-1, keepdim=True) + eps) * nw.double()).to(torch.bfloat16).double()
-        if gated:
-            g, u = xn @ w.double()[:n].T, xn @ w.double()[n:].T
-            want = g / (1 + torch.exp(-g)) * u
-        else:
-            want = xn @ w.double().T
-        torch.testing.assert_close(out.double(), want, atol=2e-2 * float(want.abs().max()), rtol=2e-2)
+    out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    k.gemm_prenormed(x, ss, eps, w, out, gated=gated)
+    scale = torch.rsqrt((xf.double() ** 2).mean(-1, keepdim=True) + eps)
+    if gated:
+        g, u = scale * (x.double() @ w.double()[:n].T), scale * (x.double() @ w.double()[n:].T)
+        want = g / (1 + torch.exp(-g)) * u
+    else:
+        want = scale * (x.double() @ w.double().T)
+    torch.testing.assert_close(out.double(), want, atol=1e-2 * float(want.abs().max()), rtol=1e-2)
+    # a row's result does not depend on the rows beside it
+    if m > 1:
+        one = torch.full((1, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+        k.gemm_prenormed(x[m - 1:].contiguous(), ss[m - 1:].contiguous(), eps, w, one, gated=gated)
+        assert torch.equal(one[0], out[m - 1])
+
+
+@pytest.mark.parametrize("mnk", [(1, 64, 48), (8, 1024, 2048), (16, 1024, 3072), (5, 96, 208), (3, 4096, 4096), (7, 50, 96),
+                                 (2, 97, 100), (16, 40, 64), (9, 4096, 12288)])
+def test_projection_that_adds_into_the_residual_stream(mnk):
+    """`gemm_residual`: h += a . w^T in 32-bit; with a norm to follow also bf16(h * next_w) and, per row and strip
+    of 16 columns, the sum of squares of the new h."""
+    m, n, kk = mnk
+    k = kernels(torch.bfloat16)
+    a = rnd((m, kk), torch.bfloat16, 97)
+    w = rnd((n, kk), torch.bfloat16, 98, 0.2)
+    h0 = rnd((m, n), torch.float32, 99, 2.0)
+    nw = rnd((n,), torch.float32, 100) + 1
+    want_h = h0.double() + a.double() @ w.double().T
+    tol_h = dict(atol=2e-5 * float(want_h.abs().max()) * max(1, kk // 512), rtol=1e-5)
+    h = h0.clone()
+    k.gemm_residual(a, w, h)
+    torch.testing.assert_close(h.double(), want_h, **tol_h)
+    h2 = h0.clone()
+    parts = k.handoff_parts(n)
+    x = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    ss = torch.full((m, parts), float("nan"), device="cuda")
+    k.gemm_residual(a, w, h2, nw, x, ss)
+    assert torch.equal(h2, h)
+    torch.testing.assert_close(x.double(), (h.double() * nw.double()).to(torch.bfloat16).double(), atol=0, rtol=2 ** -7)
+    padded = torch.zeros((m, parts * 16), dtype=torch.float64, device="cuda")
+    padded[:, :n] = h.double() ** 2
+    torch.testing.assert_close(ss.double(), padded.view(m, parts, 16).sum(-1), rtol=1e-5, atol=1e-6)
+    # the two halves together are the norm: the next projection on (x, ss) gives rmsnorm(h) . w2^T
+    w2 = rnd((64, n), torch.bfloat16, 101, 0.2)
+    out = torch.full((m, 64), float("nan"), dtype=torch.bfloat16, device="cuda")
+    k.gemm_prenormed(x, ss, 1e-6, w2, out)
+    hn = h.double() * torch.rsqrt((h.double() ** 2).mean(-1, keepdim=True) + 1e-6) * nw.double()
+    want = hn @ w2.double().T
+    torch.testing.assert_close(out.double(), want, atol=2e-2 * float(want.abs().max()), rtol=2e-2)
 
 
 def test_prompt_portion_beyond_the_page_cache_of_a_workgroup():

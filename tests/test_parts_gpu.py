@@ -230,3 +230,56 @@ def test_block_part(dtype):
     start = h0.double().numpy() + pending0.double().numpy()
     want = P.decoder_layer(start, pw, cfg, np.arange(25))
     np.testing.assert_allclose(h.double().cpu().numpy() + pending, want, **tol(dtype, want))
+
+
+def test_block_part_with_few_rows_shares_its_norms_between_the_projections():
+    """Up to 16 rows in the bfloat16 engine: every norm is split between the projection before it (which adds
+    into h and leaves h * weight and partial sums of squares) and the projection after it (which applies the
+    scale).  Two blocks in a row: the first hands the second's first norm over; the second, with nothing to
+    follow, leaves a complete h.  Against the plain layers."""
+    from mini_llm_runtime_amd.config import AttentionSpec, LayerSpec, MlpSpec, NormSpec, PositionSpec
+    from mini_llm_runtime_amd.parts import build_part
+    from mini_llm_runtime_amd.parts.registry import Handoff
+    dtype = torch.bfloat16
+    hidden, hq, hkv, d, inter, eps = 80, 4, 2, 32, 112, 1e-5
+    norm = NormSpec("rmsnorm", hidden, eps)
+    spec = LayerSpec("prenorm", norm, AttentionSpec("gqa_attention", hidden, hq, hkv, d, d ** -0.5,
+                                                     NormSpec("rmsnorm", d, eps),
+                                                     PositionSpec("rope_split_half", d, 10000.0), None),
+                     norm, MlpSpec("swiglu", hidden, inter))
+    blocks, plain_weights = [], []
+    for i in range(2):
+        block = build_part("block", spec)
+        aw = {k: v.to(dtype).float() for k, v in attention_weights(hidden, hq, hkv, d, 150 + 10 * i).items()}
+        fw = {k: v.to(dtype).float() for k, v in
+              {"gate_proj": rnd((inter, hidden), 156 + i, 0.3), "up_proj": rnd((inter, hidden), 166 + i, 0.3),
+               "down_proj": rnd((hidden, inter), 176 + i, 0.3)}.items()}
+        n1, n2 = 1 + rnd(hidden, 186 + i, 0.2), 1 + rnd(hidden, 196 + i, 0.2)
+        bind(block.norm1, {"weight": n1}, dtype)
+        bind(block.norm2, {"weight": n2}, dtype)
+        bind(block.mixer, aw, dtype)
+        bind(block.ffn, fw, dtype)
+        pw = {k.replace(".weight", ""): v.double().numpy() for k, v in {**aw, **fw}.items()}
+        pw["input_layernorm"], pw["post_attention_layernorm"] = n1.double().numpy(), n2.double().numpy()
+        blocks.append(block)
+        plain_weights.append(pw)
+    rows = 11
+    ctx = make_ctx(dtype, [blocks[0].mixer.cache_spec(), blocks[1].mixer.cache_spec()])
+    slot = ctx.cache.acquire_slot()
+    feed(ctx, [(slot, rows)])
+    assert ctx.kernels.handoff_supported(rows)
+    h0 = rnd((rows, hidden), 161)
+    pending0 = rnd((rows, hidden), 162).to(dtype)
+    h = h0.cuda().clone()
+    hand = blocks[0].forward(ctx, h, pending0.cuda(), 0, next_norm=blocks[1].norm1)
+    assert isinstance(hand, Handoff) and hand.norm is blocks[1].norm1
+    cfg = dict(num_attention_heads=hq, num_key_value_heads=hkv, head_dim=d, rms_norm_eps=eps, rope_theta=10000.0)
+    want1 = P.decoder_layer(h0.double().numpy() + pending0.double().numpy(), plain_weights[0], cfg, np.arange(rows))
+    np.testing.assert_allclose(h.double().cpu().numpy(), want1, **tol(dtype, want1))
+    got_h = h.double().cpu().numpy()
+    np.testing.assert_allclose(hand.ss.double().sum(-1).cpu().numpy(), (got_h ** 2).sum(-1), rtol=1e-5)
+    np.testing.assert_allclose(hand.x.double().cpu().numpy(), got_h * plain_weights[1]["input_layernorm"], rtol=2 ** -7)
+    last = blocks[1].forward(ctx, h, hand, 1, next_norm=None)
+    assert last is None
+    want2 = P.decoder_layer(want1, plain_weights[1], cfg, np.arange(rows))
+    np.testing.assert_allclose(h.double().cpu().numpy(), want2, **tol(dtype, want2))
