@@ -1,16 +1,23 @@
-"""Decode throughput of the Qwen3-0.6B-sized model (random weights, synthetic token ids) on one MI355X.
+"""Decode and prefill throughput of Qwen3-sized models (random weights, synthetic token ids) on one MI355X.
 
-    python bench.py [--gpus 1] [--steps 64] [--warmup 8] [--layers 28] [--batch 8] [--context 4096]
+    python bench.py [--gpus 1] [--steps 64] [--warmup 8] [--size 0.6b] [--layers 0] [--batch 8] [--context 4096]
 
-A "step" is one decode step of the whole batch: one token per request through the engine's step
-function and the greedy sampler.  Requests are first filled by real prefill (portions of 2048 tokens)
-so that the timed steps end at the context length.  One JSON line is printed with decoded tokens a
-second, the same at batch 1 and 64, the prefill of 2048 tokens and the decode step's share of the
-HBM roofline.
+A "step" is one decode step of the whole batch: one token per request through the engine's step function
+and the greedy sampler.  Requests are first filled by real prefill (portions of 2048 tokens) so that the
+timed steps end at the context length.  One JSON line is printed:
+
+  * value / ms_per_step / roofline: decode at --batch (8) of the --size (0.6b) model, with the step's share of
+    the HBM roofline (bytes it has to read: every weight once and the live requests' cache; 8 TB/s);
+  * points: the same at batch 1 and 64;  prefill: 2048 tokens in one step, with its share of the MFMA peak;
+  * with the default size, a block "8b": decode at batch 1, 8 and 64, prefill and a mixed step (64 decoding
+    requests beside a 2048-token prompt portion in ONE step) at the Qwen3-8B sizes, each with its share of
+    its roofline.  `--size 32b --only mixed` measures the mixed step at the 32B sizes.
+  * --profile: time per kernel class (event pairs around every launch, steps run eagerly) beside the line.
 """
 import argparse
 import json
 import os
+import statistics
 import sys
 import time
 
@@ -34,6 +41,218 @@ SIZES = {
 PREFILL_TOKENS = 2048
 
 
+class Bench:
+    """One model of the given sizes on the GPU and the measurements on it."""
+
+    def __init__(self, size, layers, args):
+        import torch
+        from mini_llm_runtime_amd.api import parse_dtype
+        from mini_llm_runtime_amd.config import config_from_dict
+        from mini_llm_runtime_amd.parts import DecoderModel, expected_tensors
+        self.torch, self.args, self.size = torch, args, size
+        self.dtype = parse_dtype(args.dtype)
+        self.tag = "bf16" if self.dtype == torch.bfloat16 else "fp32"
+        self.full_layers, sizes = SIZES[size]
+        self.layers = layers if layers > 0 else self.full_layers
+        self.cfg = c = config_from_dict(dict(sizes, architectures=["Qwen3ForCausalLM"], num_hidden_layers=self.layers))
+        # Random weights N(0, 0.02) (norm weights 1 + N(0, 0.1)) drawn on the GPU: the same tensors that the
+        # random-weights mode would write to a model folder, without the trip through a file of many gigabytes.
+        torch.manual_seed(0)
+        weights = {}
+        for name, spec in expected_tensors(c).items():
+            if spec.optional:
+                continue
+            if spec.keep_float32:
+                weights[name] = 1.0 + 0.1 * torch.randn(spec.shape, device="cuda", dtype=torch.float32)
+            else:
+                weights[name] = torch.randn(spec.shape, device="cuda", dtype=self.dtype).mul_(0.02)
+        self.model = DecoderModel(c, weights, self.dtype, "cuda:0")
+        del weights
+        self.layer_params = c.hidden_size * (c.num_attention_heads + 2 * c.num_key_value_heads) * c.head_dim \
+            + c.num_attention_heads * c.head_dim * c.hidden_size + 3 * c.hidden_size * c.intermediate_size
+        self.elem = 2 if self.dtype == torch.bfloat16 else 4
+        self.weight_bytes = (self.layers * self.layer_params + c.vocab_size * c.hidden_size) * self.elem
+        self.kv_bytes_per_token = self.layers * 2 * c.num_key_value_heads * c.head_dim * self.elem
+        self.g = torch.Generator().manual_seed(0)
+
+    def close(self):
+        self.model = None
+        self.torch.cuda.empty_cache()
+
+    def runner(self, slots, max_tokens, max_length, max_batch_tokens, **kwargs):
+        from mini_llm_runtime_amd.engine import Runner
+        a = self.args
+        return Runner(self.model, max_tokens=max_tokens, max_slots=slots, max_length=max_length,
+                      max_batch_tokens=max_batch_tokens, page_size=a.page_size, target_workgroups=a.attn_workgroups,
+                      library_gemm=bool(a.library), split_keys=a.split_keys, max_logits_rows=slots,
+                      profile=bool(a.profile), **kwargs)
+
+    def fill(self, runner, slots, tokens):
+        """`tokens` tokens into every slot's cache: by real prefill (default) or, as a profiling aid, at random."""
+        from mini_llm_runtime_amd.engine import Entry
+        torch, c = self.torch, self.cfg
+        if self.args.fill == "random":
+            runner.cache.commit(slots, [tokens] * len(slots))
+            for slab in runner.cache._k + runner.cache._v:
+                slab.normal_()
+            return
+        for s in slots:
+            ids = torch.randint(0, c.vocab_size, (tokens,), generator=self.g).tolist()
+            for at in range(0, tokens, PREFILL_TOKENS):
+                runner.step([Entry(s, ids[at:at + PREFILL_TOKENS], [])])
+
+    def decode(self, batch, steps, warmup):
+        """Fill `batch` requests so that warmup + steps decode steps end at the context length; time `steps`.
+        Returns (seconds, mean context, profile report or None)."""
+        from mini_llm_runtime_amd.engine import Entry
+        from mini_llm_runtime_amd.sampling import Sampler
+        torch, a, c = self.torch, self.args, self.cfg
+        runner = self.runner(batch, batch * (-(-a.context // 64) * 64), a.context, max(PREFILL_TOKENS, batch))
+        sampler = Sampler(runner.kernels, runner.device, max_rows=batch)
+        fill = a.context - steps - warmup
+        assert fill >= 1
+        slots = [runner.open_request() for _ in range(batch)]
+        self.fill(runner, slots, fill)
+        tokens = torch.randint(0, c.vocab_size, (batch,), generator=self.g).tolist()
+        zeros = [0.0] * batch
+
+        def one(tokens):
+            logits = runner.step([Entry(s, [t], [0]) for s, t in zip(slots, tokens)])
+            return sampler.sample(logits, zeros, zeros)
+        for _ in range(warmup):
+            tokens = one(tokens)
+        runner.profile_report(reset=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            tokens = one(tokens)
+        torch.cuda.synchronize()
+        seconds = time.perf_counter() - t0
+        report = runner.profile_report()
+        for s in slots:
+            runner.close_request(s)
+        del runner, sampler
+        torch.cuda.empty_cache()
+        return seconds, a.context - steps / 2.0, report
+
+    def decode_point(self, batch, steps, warmup):
+        """{tok_s, ms, frac}: decoded tokens a second, milliseconds a step, share of the HBM roofline."""
+        seconds, mean_context, report = self.decode(batch, steps, warmup)
+        step_bytes = self.weight_bytes + batch * mean_context * self.kv_bytes_per_token
+        out = dict(tok_s=round(batch * steps / seconds, 1), ms=round(seconds / steps * 1e3, 4),
+                   frac=round(step_bytes / (seconds / steps) / HBM_PEAK, 5))
+        return out, step_bytes, report
+
+    def prefill(self):
+        from mini_llm_runtime_amd.engine import Entry
+        torch, a, c = self.torch, self.args, self.cfg
+        runner = self.runner(1, PREFILL_TOKENS, PREFILL_TOKENS, PREFILL_TOKENS,
+                             graph_max_tokens=PREFILL_TOKENS if a.prefill_graph and not a.profile else 512)
+        ids = torch.randint(0, c.vocab_size, (PREFILL_TOKENS,), generator=self.g).tolist()
+        times = []
+        for i in range(a.prefill_reps):
+            s = runner.open_request()
+            if i == 1:
+                runner.profile_report(reset=True)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            runner.step([Entry(s, ids, [PREFILL_TOKENS - 1])])
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t0)
+            runner.close_request(s)
+        seconds = min(times[1:])
+        t = PREFILL_TOKENS
+        flops = 2.0 * t * self.layers * self.layer_params \
+            + 2.0 * t * t * c.num_attention_heads * c.head_dim * self.layers \
+            + 2.0 * c.vocab_size * c.hidden_size
+        out = dict(value=round(t / seconds, 1), tokens=t, ms=round(seconds * 1e3, 3),
+                   ms_median=round(statistics.median(times[1:]) * 1e3, 3),
+                   frac=round(flops / seconds / MFMA_PEAK[self.tag], 5))
+        report = runner.profile_report()
+        if report is not None:
+            out["profile"] = report
+        del runner
+        torch.cuda.empty_cache()
+        return out
+
+    def mixed(self, decoding=64, reps=6):
+        """ONE step that holds `decoding` single tokens of requests at the context length beside a portion of
+        2048 tokens of another request's prompt (the reference's mixed workload,
+        benchmarks/runtime-inputs/qwen3-cuda-v0.json:96-97).  Milliseconds a step (median, and the fastest)
+        against max(bytes / 8 TB/s, flops / MFMA peak)."""
+        from mini_llm_runtime_amd.engine import Entry
+        from mini_llm_runtime_amd.sampling import Sampler
+        torch, a, c = self.torch, self.args, self.cfg
+        ctx_tokens = -(-a.context // 64) * 64
+        runner = self.runner(decoding + 1, decoding * ctx_tokens + PREFILL_TOKENS, a.context, PREFILL_TOKENS + decoding)
+        sampler = Sampler(runner.kernels, runner.device, max_rows=decoding)
+        slots = [runner.open_request() for _ in range(decoding)]
+        start = a.context - reps - 1
+        self.fill(runner, slots, start)
+        ids = torch.randint(0, c.vocab_size, (PREFILL_TOKENS,), generator=self.g).tolist()
+        tokens = torch.randint(0, c.vocab_size, (decoding,), generator=self.g).tolist()
+        zeros = [0.0] * decoding
+        times = []
+        for i in range(reps + 1):
+            prompt = runner.open_request()
+            if i == 1:
+                runner.profile_report(reset=True)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            logits = runner.step([Entry(s, [t], [0]) for s, t in zip(slots, tokens)] + [Entry(prompt, ids, [])])
+            tokens = sampler.sample(logits, zeros, zeros)
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t0)
+            runner.close_request(prompt)
+        times = times[1:]
+        t, hq, d = PREFILL_TOKENS, c.num_attention_heads, c.head_dim
+        context = start + (reps + 1) / 2.0
+        step_bytes = self.weight_bytes + (decoding * context + t) * self.kv_bytes_per_token
+        flops = 2.0 * (t + decoding) * self.layers * self.layer_params \
+            + (2.0 * t * t + 4.0 * decoding * context) * hq * d * self.layers + 2.0 * decoding * c.vocab_size * c.hidden_size
+        floor = max(step_bytes / HBM_PEAK, flops / MFMA_PEAK[self.tag])
+        seconds = statistics.median(times)
+        out = dict(ms=round(seconds * 1e3, 3), ms_best=round(min(times) * 1e3, 3), decode_rows=decoding, prefill_tokens=t,
+                   context=a.context, floor_ms=round(floor * 1e3, 3),
+                   bound="mfma" if flops / MFMA_PEAK[self.tag] > step_bytes / HBM_PEAK else "hbm",
+                   frac=round(floor / seconds, 5), tok_s=round((t + decoding) / seconds, 1))
+        report = runner.profile_report()
+        if report is not None:
+            out["profile"] = report
+        for s in slots:
+            runner.close_request(s)
+        del runner, sampler
+        torch.cuda.empty_cache()
+        return out
+
+    def engine_burst(self):
+        from mini_llm_runtime_amd.engine import Engine, EngineOptions
+        torch, a, c = self.torch, self.args, self.cfg
+        slots, prompt, output = a.batch, 512, 128
+        engine = Engine(self.model, EngineOptions(context_tokens=slots * 1024, max_model_len=1024, max_active=slots,
+                                                  batch_tokens=max(256, 16 * slots), prefill_chunk=max(128, 8 * slots),
+                                                  block_size=a.page_size))
+        requests = 3 * slots
+
+        def burst(n):
+            for _ in range(n):
+                engine.submit(torch.randint(0, c.vocab_size, (prompt,), generator=self.g).tolist(), max_tokens=output,
+                              ignore_eos=True)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            engine.run_until_done()
+            torch.cuda.synchronize()
+            return time.perf_counter() - t0
+        first = burst(requests)                 # a server's first minute: step shapes are met and captured
+        before = dict(engine.stats)
+        seconds = burst(requests)               # the same burst again: what a server that has run a while does
+        return {"requests": requests, "slots": slots, "prompt_tokens": prompt, "output_tokens": output,
+                "seconds": round(seconds, 3), "generated_tok_s": round(requests * output / seconds, 1),
+                "total_tok_s": round(requests * (prompt + output) / seconds, 1), "first_burst_seconds": round(first, 3),
+                "batches": engine.stats["batches"] - before["batches"],
+                "mixed_batches": engine.stats["mixed_batches"] - before["mixed_batches"]}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -47,170 +266,55 @@ def main():
     ap.add_argument("--page-size", type=int, default=16, help="tokens in a page of the cache")
     ap.add_argument("--attn-workgroups", type=int, default=512,
                     help="tuning aid: workgroups that the split of a token's keys aims for")
-    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points and the prefill")
-    ap.add_argument("--only", default="all", choices=["all", "decode", "prefill", "engine"],
-                    help="profiling aid: run just the decode steps or just the prefill; engine: the scheduler "
-                         "over a burst of requests (3 x batch requests of 512 prompt and 128 output tokens, "
+    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points, the prefill and the 8B block")
+    ap.add_argument("--no-8b", action="store_true", help="skip the block of 8B measurements in the default run")
+    ap.add_argument("--only", default="all", choices=["all", "decode", "prefill", "engine", "mixed"],
+                    help="profiling aid: run just the decode steps, just the prefill or just the mixed step; engine: the "
+                         "scheduler over a burst of requests (3 x batch requests of 512 prompt and 128 output tokens, "
                          "batch slots), printed as one line of its own")
     ap.add_argument("--library", type=int, default=1,
                     help="0: every matrix product on the hand-written kernels, none in the vendor library")
     ap.add_argument("--split-keys", type=int, default=256, help="the smallest range of keys of one attention workgroup")
     ap.add_argument("--tune", type=int, default=1,
-                    help="0: the vendor library's first candidate for every shape, none timed")
+                    help="0: the vendor library's first candidate for every shape, none timed (the engine's default is 1)")
     ap.add_argument("--prefill-graph", type=int, default=1,
                     help="1: the prefill step may be captured as a graph once its shape has come often enough")
     ap.add_argument("--prefill-reps", type=int, default=10, help="prefill steps; the fastest but the first counts")
     ap.add_argument("--fill", default="prefill", choices=["prefill", "random"],
                     help="how the requests' caches are filled before the timed steps: by real prefill "
                          "(default) or, as a profiling aid, with random keys and values")
+    ap.add_argument("--profile", action="store_true",
+                    help="time per kernel class (event pairs around every launch; steps then run eagerly, so the "
+                         "step times themselves are those of the eager engine)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not built (single-GPU engine)")
         return 2
 
-    import torch
-    from mini_llm_runtime_amd.api import parse_dtype
-    from mini_llm_runtime_amd.config import config_from_dict
-    from mini_llm_runtime_amd.engine import Entry, Runner
-    from mini_llm_runtime_amd.parts import DecoderModel, expected_tensors
-    from mini_llm_runtime_amd.sampling import Sampler
-
-    dtype = parse_dtype(args.dtype)
     if not args.tune:
         from mini_llm_runtime_amd.kernels import build
         build.load("library_gemm").mlr_library_gemm_tuning(0)
-    tag = "bf16" if dtype == torch.bfloat16 else "fp32"
-    FULL_LAYERS, sizes = SIZES[args.size]
-    if args.layers <= 0:
-        args.layers = FULL_LAYERS
-    cfg = config_from_dict(dict(sizes, architectures=["Qwen3ForCausalLM"], num_hidden_layers=args.layers))
-    # Random weights N(0, 0.02) (norm weights 1 + N(0, 0.1)) drawn on the GPU: the same tensors that the
-    # random-weights mode would write to a model folder, without the trip through a file of many gigabytes.
-    torch.manual_seed(0)
-    weights = {}
-    for name, spec in expected_tensors(cfg).items():
-        if spec.optional:
-            continue
-        if spec.keep_float32:
-            weights[name] = 1.0 + 0.1 * torch.randn(spec.shape, device="cuda", dtype=torch.float32)
-        else:
-            weights[name] = (0.02 * torch.randn(spec.shape, device="cuda", dtype=torch.float32)).to(dtype)
-    model = DecoderModel(cfg, weights, dtype, "cuda:0")
-    del weights
-    c = cfg
-    layer_params = c.hidden_size * (c.num_attention_heads + 2 * c.num_key_value_heads) * c.head_dim \
-        + c.num_attention_heads * c.head_dim * c.hidden_size + 3 * c.hidden_size * c.intermediate_size
-    elem = 2 if dtype == torch.bfloat16 else 4
-    weight_bytes = (args.layers * layer_params + c.vocab_size * c.hidden_size) * elem     # layers + output projection
-    kv_bytes_per_token = args.layers * 2 * c.num_key_value_heads * c.head_dim * elem
-    g = torch.Generator().manual_seed(0)
-
-    def decode_run(batch, steps, warmup):
-        """Fill `batch` requests so that warmup + steps decode steps end at the context length; time `steps`."""
-        runner = Runner(model, max_tokens=batch * (-(-args.context // 64) * 64), max_slots=batch,
-                        max_length=args.context, max_batch_tokens=max(PREFILL_TOKENS, batch), page_size=args.page_size,
-                        target_workgroups=args.attn_workgroups, library_gemm=bool(args.library),
-                        split_keys=args.split_keys)
-        sampler = Sampler(runner.kernels, runner.device, max_rows=batch)
-        fill = args.context - steps - warmup
-        assert fill >= 1
-        slots = [runner.open_request() for _ in range(batch)]
-        if args.fill == "random":
-            runner.cache.commit(slots, [fill] * batch)
-            for slab in runner.cache._k + runner.cache._v:
-                slab.normal_()
-        else:
-            for s in slots:
-                ids = torch.randint(0, c.vocab_size, (fill,), generator=g).tolist()
-                for at in range(0, fill, PREFILL_TOKENS):
-                    runner.step([Entry(s, ids[at:at + PREFILL_TOKENS], [])])
-        tokens = torch.randint(0, c.vocab_size, (batch,), generator=g).tolist()
-        zeros = [0.0] * batch
-
-        def one(tokens):
-            logits = runner.step([Entry(s, [t], [0]) for s, t in zip(slots, tokens)])
-            return sampler.sample(logits, zeros, zeros)
-        for _ in range(warmup):
-            tokens = one(tokens)
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(steps):
-            tokens = one(tokens)
-        torch.cuda.synchronize()
-        seconds = time.perf_counter() - t0
-        mean_context = args.context - steps / 2.0
-        for s in slots:
-            runner.close_request(s)
-        del runner
-        torch.cuda.empty_cache()
-        return seconds, mean_context
-
-    def prefill_run():
-        runner = Runner(model, max_tokens=PREFILL_TOKENS, max_slots=1, max_length=PREFILL_TOKENS,
-                        max_batch_tokens=PREFILL_TOKENS, page_size=args.page_size,
-                        graph_max_tokens=PREFILL_TOKENS if args.prefill_graph else 512,
-                        library_gemm=bool(args.library))
-        ids = torch.randint(0, c.vocab_size, (PREFILL_TOKENS,), generator=g).tolist()
-        times = []
-        for i in range(args.prefill_reps):
-            s = runner.open_request()
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            runner.step([Entry(s, ids, [PREFILL_TOKENS - 1])])
-            torch.cuda.synchronize()
-            times.append(time.perf_counter() - t0)
-            runner.close_request(s)
-        seconds = min(times[1:])
-        t = PREFILL_TOKENS
-        flops = 2.0 * t * args.layers * layer_params \
-            + 2.0 * t * t * c.num_attention_heads * c.head_dim * args.layers \
-            + 2.0 * c.vocab_size * c.hidden_size
-        return dict(value=round(t / seconds, 1), tokens=t, ms=round(seconds * 1e3, 3),
-                    frac=round(flops / seconds / MFMA_PEAK[tag], 5))
-
+    bench = Bench(args.size, args.layers, args)
+    c = bench.cfg
     if args.only == "prefill":
-        print(json.dumps({"prefill": prefill_run()}))
+        print(json.dumps({"prefill": bench.prefill()}))
         return 0
     if args.only == "engine":
-        from mini_llm_runtime_amd.engine import Engine, EngineOptions
-        slots, prompt, output = args.batch, 512, 128
-        engine = Engine(model, EngineOptions(context_tokens=slots * 1024, max_model_len=1024, max_active=slots,
-                                             batch_tokens=max(256, 16 * slots), prefill_chunk=max(128, 8 * slots),
-                                             block_size=args.page_size))
-        requests = 3 * slots
-
-        def burst(n):
-            for _ in range(n):
-                engine.submit(torch.randint(0, c.vocab_size, (prompt,), generator=g).tolist(), max_tokens=output,
-                              ignore_eos=True)
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            engine.run_until_done()
-            torch.cuda.synchronize()
-            return time.perf_counter() - t0
-        first = burst(requests)                 # a server's first minute: step shapes are met and captured
-        before = dict(engine.stats)
-        seconds = burst(requests)               # the same burst again: what a server that has run a while does
-        print(json.dumps({"engine": {"requests": requests, "slots": slots, "prompt_tokens": prompt,
-                                     "output_tokens": output, "seconds": round(seconds, 3),
-                                     "generated_tok_s": round(requests * output / seconds, 1),
-                                     "total_tok_s": round(requests * (prompt + output) / seconds, 1),
-                                     "first_burst_seconds": round(first, 3),
-                                     "batches": engine.stats["batches"] - before["batches"],
-                                     "mixed_batches": engine.stats["mixed_batches"] - before["mixed_batches"]}}))
+        print(json.dumps({"engine": bench.engine_burst()}))
         return 0
-    seconds, mean_context = decode_run(args.batch, args.steps, args.warmup)
-    ms_per_step = seconds / args.steps * 1e3
-    value = args.batch * args.steps / seconds
-    step_bytes = weight_bytes + args.batch * mean_context * kv_bytes_per_token
-    achieved = step_bytes / (seconds / args.steps) / 1e9
+    if args.only == "mixed":
+        print(json.dumps({"mixed": dict(bench.mixed(), model=f"Qwen3-{args.size.upper()} sizes", layers=bench.layers,
+                                        layers_full=bench.full_layers, fill=args.fill)}))
+        return 0
+    point, step_bytes, report = bench.decode_point(args.batch, args.steps, args.warmup)
+    achieved = step_bytes / (point["ms"] / 1e3) / 1e9
     line = {
         "metric": f"decode tok/s, Qwen3-{args.size.upper()} sizes, batch {args.batch}, context {args.context}",
-        "value": round(value, 1),
+        "value": point["tok_s"],
         "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": tag, "data": "synthetic token ids, random weights N(0, 0.02)",
-        "config": {"model": f"Qwen3-{args.size.upper()} sizes", "layers": args.layers, "layers_full": FULL_LAYERS,
+        "ms_per_step": point["ms"], "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": bench.tag, "data": "synthetic token ids, random weights N(0, 0.02)",
+        "config": {"model": f"Qwen3-{args.size.upper()} sizes", "layers": bench.layers, "layers_full": bench.full_layers,
                    "hidden_size": c.hidden_size, "q_heads": c.num_attention_heads,
                    "kv_heads": c.num_key_value_heads, "head_dim": c.head_dim,
                    "intermediate_size": c.intermediate_size, "vocab_size": c.vocab_size,
@@ -219,14 +323,34 @@ def main():
                    "sampling": "greedy", "parallelism": "single GPU"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                      "frac": round(achieved * 1e9 / HBM_PEAK, 5)},
+        "library_tuning": bool(args.tune),
     }
+    if report is not None:
+        line["profile"] = report
     if not args.no_points and args.only == "all":
-        line["prefill"] = prefill_run()
+        line["prefill"] = bench.prefill()
         points = {}
         for batch in (1, 64):
-            s, _ = decode_run(batch, max(8, args.steps // 2), max(2, args.warmup // 2))
-            points[f"decode_b{batch}"] = round(batch * max(8, args.steps // 2) / s, 1)
+            p, _, _ = bench.decode_point(batch, max(8, args.steps // 2), max(2, args.warmup // 2))
+            points[f"decode_b{batch}"] = p["tok_s"]
+            points[f"frac_b{batch}"] = p["frac"]
         line["points"] = points
+        if args.size == "0.6b" and not args.no_8b and args.layers <= 0:
+            # the other half of the headline metric: the same measurements at the Qwen3-8B sizes (all 36 layers)
+            bench.close()
+            big = Bench("8b", 0, args)
+            block = {"layers": big.layers}
+            for batch in (1, 8, 64):
+                p, _, _ = big.decode_point(batch, max(8, args.steps // 2), max(2, args.warmup // 2))
+                block[f"decode_b{batch}"] = p["tok_s"]
+                block[f"ms_b{batch}"] = p["ms"]
+                block[f"frac_b{batch}"] = p["frac"]
+            pre = big.prefill()
+            block.update(prefill_tok_s=pre["value"], prefill_ms=pre["ms"], prefill_frac=pre["frac"])
+            mixed = big.mixed()
+            block.update(mixed_ms=mixed["ms"], mixed_floor_ms=mixed["floor_ms"], mixed_frac=mixed["frac"],
+                         mixed_bound=mixed["bound"], mixed_tok_s=mixed["tok_s"])
+            line["8b"] = block
     print(json.dumps(line))
     return 0
 

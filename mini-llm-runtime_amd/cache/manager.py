@@ -270,6 +270,7 @@ class CacheManager:
             table = torch.full((max_slots + 1, self.book.max_blocks(g)), -1, dtype=torch.int32, device=self.device)
             table[max_slots, 0] = self.num_pages
             self._tables.append(table)
+        self._stages = {}                # group -> [pinned copy of its table, event of the last upload, in use]
         self._states = {}
         for cid, spec in enumerate(self.entry_specs):
             if isinstance(spec, StateSpec):
@@ -327,16 +328,33 @@ class CacheManager:
         return self.book.retire(slots)
 
     def sync_tables(self):
+        """Changed rows of the block tables go to the device through a pinned staging copy of the table, with
+        asynchronous copies on the current stream (a copy from pageable memory would block the host on every
+        step that crosses a page's edge); an event guards the staging rows until the copies have left them."""
         for g, dev in enumerate(self._tables):
             rows = self.book.take_dirty(g)
             if not rows:
                 continue
             host = torch.from_numpy(self.book.table(g))
-            if len(rows) * 4 >= self.max_slots:
+            if dev.device.type != "cuda":
                 dev[:self.max_slots].copy_(host)
+                continue
+            stage = self._stages.get(g)
+            if stage is None:
+                stage = self._stages[g] = [torch.empty(tuple(host.shape), dtype=torch.int32).pin_memory(),
+                                           torch.cuda.Event(), False]
+            pinned, event, busy = stage
+            if busy:
+                event.synchronize()
+            if len(rows) * 4 >= self.max_slots:
+                pinned.copy_(host)
+                dev[:self.max_slots].copy_(pinned, non_blocking=True)
             else:
                 for s in rows:
-                    dev[s].copy_(host[s])
+                    pinned[s].copy_(host[s])
+                    dev[s].copy_(pinned[s], non_blocking=True)
+            event.record()
+            stage[2] = True
 
     def check(self):
         self.book.check()

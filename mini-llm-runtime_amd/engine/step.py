@@ -38,7 +38,7 @@ class Entry:
 class Runner:
     def __init__(self, model, max_tokens, max_slots=4, max_length=None, max_batch_tokens=None,
                  page_size=16, split_keys=256, split_max_tokens=256, use_graphs=True, graph_max_batch=256,
-                 target_workgroups=512, graph_max_tokens=512, graph_after=4, max_graphs=64, library_gemm=True,
+                 target_workgroups=512, graph_max_tokens=512, graph_after=4, max_graphs=128, library_gemm=True,
                  max_logits_rows=None, device_budget_bytes=None, check_finite=False, profile=False):
         """`max_tokens`: tokens the page pool holds; `max_length`: longest request; `max_batch_tokens`: most
         tokens of one step; `max_logits_rows`: most wanted places of one step (default: every token).
@@ -145,6 +145,16 @@ class Runner:
             return 0, False
         return fill, mixed
 
+    def _context_bucket(self, longest):
+        """The context length a captured step is laid out for: the smallest of 512, 1024, 2048, ... that holds
+        the step's longest context (at most max_length).  A graph fixes how many workgroups split a token's
+        keys; laid out for max_length, a server with a long limit would launch splits for keys that do not
+        exist on every short-context step.  A shape is captured once per bucket it is met in."""
+        bucket = 512
+        while bucket < longest:
+            bucket *= 2
+        return min(bucket, self.max_length)
+
     def _graph_wanted(self, entries, total, sig):
         """Steps are launch-bound unless they bring many tokens.  Steps of single tokens with logits for
         each (decoding) are captured the second time they come, others (portions beside decoded tokens)
@@ -153,7 +163,8 @@ class Runner:
             return False
         if sig in self._graphs:
             return True
-        if total == len(sig) and all(w == (0,) for _, w in sig):
+        shape = sig[0]
+        if total == len(shape) and all(w == (0,) for _, w in shape):
             return total <= self.graph_max_batch
         seen = self._seen.get(sig, 0) + 1
         self._seen[sig] = seen
@@ -183,9 +194,10 @@ class Runner:
         replayed twice on the same inputs and compared with the eager result, and a shape whose replays
         differ (a library call that records a clearing node would do that) stays eager for good."""
         state = self._graphs.get(sig)
+        shape, bucket = sig
         if state is None:
             rows, base = [], 0
-            for n, want in sig:
+            for n, want in shape:
                 rows.extend(base + w for w in want)
                 base += n
             meta = torch.empty(3 * total + max(len(rows), 1), dtype=torch.int32, device=self.device)
@@ -232,7 +244,7 @@ class Runner:
         if state["eager"]:                                # a shape whose capture did not hold
             ctx.max_context = max(p0 + n for (_, _, n, p0) in segments)
             return self.model.forward(ctx, want_rows)
-        ctx.max_context = self.max_length                 # the graph must serve every later context
+        ctx.max_context = bucket                          # the graph must serve every context of its bucket
         ctx.fixed_groups = state["groups"]
         state["runs"] += 1
         if state["runs"] == 1:                            # first time: eager, sizes the scratch buffers
@@ -298,6 +310,8 @@ class Runner:
             fill, fill_first = self._decode_fill(entries) if sig is not None else (0, False)
             if fill:
                 sig = ((1, (0,)),) * fill + sig if fill_first else sig + ((1, (0,)),) * fill
+            if sig is not None:                           # a captured step is keyed by its shape and its context bucket
+                sig = (sig, self._context_bucket(max(p0 + n for p0, n in zip(first, counts))))
             if sig is not None and self._graph_wanted(entries, total + fill, sig):
                 logits = self._graph_step(entries, first, total + fill, sig, fill, fill_first)
                 self.cache.retire(slots)

@@ -28,7 +28,8 @@ Interfaces (B = the tokens of a step, E = the model width, T = the engine's elem
 
 A part may set the class attribute `graph_safe = True` when what it launches depends only on the step's
 SHAPE -- how many tokens each entry brings (ctx.n_tokens, the lengths in ctx.segments, ctx.single_tokens,
-ctx.token_groups) and ctx.max_context, which is the runner's max_length in a step that is to be captured --
+ctx.token_groups) and ctx.max_context, which in a step that is to be captured is its context bucket (512, 1024,
+2048, ... up to the runner's max_length: the smallest that holds the step's longest context) --
 and everything else reaches its kernels through device memory (ctx.token_ids, positions, slots, the cache
 views).  Steps of a shape that comes again are then captured once as a HIP graph and replayed.  A part
 that reads the slots or positions of ctx.segments on the host, or keeps host-side state per request, must

@@ -129,7 +129,7 @@ def test_a_step_shape_that_comes_again_is_captured_and_stays_right(model_folders
     compare(got, {k: v for k, v in want.items() if k in got}, dtype_name)
     assert len(got) == 3 + 10 * 4
     shape = ((20, (0, 19)), (1, (0,)), (1, (0,)))
-    assert r.graph_failures == 0 and r._graphs[shape]["graph"] is not None
+    assert r.graph_failures == 0 and r._graphs[(shape, 512)]["graph"] is not None
     r.cache.check()
     assert r.cache.free_pages() == r.cache.num_pages
 
@@ -167,7 +167,7 @@ def test_decode_batches_are_filled_up_to_a_size_that_comes_again(model_folders, 
                 at[rid] += 1
         compare(got, {k: want[k] for k in got}, dtype_name)
         if use_graphs:
-            sizes = sorted(len(sig) for sig, st in r._graphs.items() if st["graph"] is not None)
+            sizes = sorted(len(sig[0]) for sig, st in r._graphs.items() if st["graph"] is not None)
             assert sizes == [10, 12] and r.graph_failures == 0
         for rid in live:
             r.close_request(slots[rid])
@@ -219,7 +219,7 @@ def test_mixed_batches_fill_their_single_tokens_too(model_folders, plain_models,
             got[(long_id, 16 * step + 3)], got[(long_id, 16 * step + 15)] = rows[len(live)], rows[len(live) + 1]
         compare(got, {k: want[k] for k in got}, dtype_name)
         if use_graphs:
-            shapes = sorted(len(sig) for sig, st in r._graphs.items() if st["graph"] is not None)
+            shapes = sorted(len(sig[0]) for sig, st in r._graphs.items() if st["graph"] is not None)
             assert shapes == [11, 13] and r.graph_failures == 0        # ten and twelve single tokens + the portion
         for rid in list(slots):
             r.close_request(slots[rid])
@@ -270,6 +270,11 @@ def test_long_decoding(model_folders, plain_models, name, dtype_name):
     steps += [dict(step=i, entries=[dict(id="r0", tokens=[toks[i]], want=[0])], end=[]) for i in range(5, 605)]
     steps[-1]["end"] = ["r0"]
     compare(run_steps(r, steps), want, dtype_name)
+    # the single-token step was captured once for contexts up to 512 and once for the longer ones: a graph is
+    # laid out (key splits) for its context bucket, not for the longest request the runner allows
+    one = ((1, (0,)),)
+    assert r._graphs[(one, 512)]["graph"] is not None and r._graphs[(one, 1024)]["graph"] is not None
+    assert r.graph_failures == 0
 
 
 @pytest.mark.parametrize("dtype_name", DTYPES)
