@@ -215,8 +215,8 @@ class CacheManager:
     def plan(entry_specs, dtype, page_size, max_tokens, max_slots, max_length):
         """(bytes of pages, of block tables, of state slabs) that a manager with these sizes allocates:
         per group of equal `KvSpec`s keys and values [entries, pages + 1, kv_heads, page_size, head_dim]
-        and a table [max_slots + 1, ceil(max_length / page_size)] of int32; per `StateSpec` a slab
-        [max_slots, *shape]."""
+        and a table [max_slots + 1, ceil(max_length / page_size)] of int32; per `StateSpec` two slabs
+        [max_slots + 1, *shape] (live and staged)."""
         element = torch.empty((), dtype=dtype).element_size()
         pages = (max_tokens + page_size - 1) // page_size + 1
         blocks = (max_length + page_size - 1) // page_size
@@ -226,7 +226,7 @@ class CacheManager:
             if isinstance(spec, KvSpec):
                 groups[spec] = groups.get(spec, 0) + 1
             elif isinstance(spec, StateSpec):
-                count = max_slots
+                count = 2 * (max_slots + 1)          # live and staged rows, one more for the scratch request
                 for extent in spec.shape:
                     count *= int(extent)
                 state += count * torch.empty((), dtype=spec.dtype).element_size()
@@ -256,11 +256,11 @@ class CacheManager:
         self.group_specs = [None] * len(members)
         for spec, g in self._group_of_spec.items():
             self.group_specs[g] = spec
-        # Beyond the pool and the slots of the bookkeeping, every group has one page more and every block
-        # table one row more: a scratch request of one token (slot `scratch_slot`, its only block mapped to
-        # that page), with which a step may fill a batch up to a size it has a captured graph for.  Models
-        # with per-request state have no such request (its state would have to be kept apart too).
-        self.scratch_slot = max_slots if all(not isinstance(s, StateSpec) for s in self.entry_specs) else None
+        # Beyond the pool and the slots of the bookkeeping, every group has one page more, every block
+        # table one row more and every state slab one row more: a scratch request of one token (slot
+        # `scratch_slot`, its only block mapped to that page), with which a step may fill a batch up to a
+        # size it has a captured graph for.
+        self.scratch_slot = max_slots
         self._k, self._v, self._tables = [], [], []
         for g, spec in enumerate(self.group_specs):
             shape = (len(members[g]), self.num_pages + 1, spec.kv_heads, page_size, spec.head_dim)
@@ -271,10 +271,14 @@ class CacheManager:
             table[max_slots, 0] = self.num_pages
             self._tables.append(table)
         self._stages = {}                # group -> [pinned copy of its table, event of the last upload, in use]
-        self._states = {}
+        # State of fixed size: a live slab, which mixers read, and a staged one, into which they write the
+        # state their step leads to; the staged rows of a step's requests become live when every layer has
+        # run (`commit_state`), so a step that fails on the way leaves the live state as it was.
+        self._states, self._staged = {}, {}
         for cid, spec in enumerate(self.entry_specs):
             if isinstance(spec, StateSpec):
-                self._states[cid] = torch.zeros((max_slots, *spec.shape), dtype=spec.dtype, device=self.device)
+                self._states[cid] = torch.zeros((max_slots + 1, *spec.shape), dtype=spec.dtype, device=self.device)
+                self._staged[cid] = torch.zeros_like(self._states[cid])
 
     # -- views for the parts ---------------------------------------------------------------------
     def kv_view(self, cache_id):
@@ -283,7 +287,32 @@ class CacheManager:
         return KvView(self._k[g][i], self._v[g][i], self._tables[g], self.page_size, spec.window, g)
 
     def state_view(self, cache_id):
+        """[max_slots + 1, *shape]: the requests' live state (row = slot); read it, do not write it."""
         return self._states[cache_id]
+
+    def state_stage(self, cache_id):
+        """[max_slots + 1, *shape]: where a mixer leaves the state that its step leads to, in the rows of the
+        step's slots (every slot of the step, in every step that writes the entry)."""
+        return self._staged[cache_id]
+
+    def has_state(self):
+        return bool(self._states)
+
+    def commit_state(self, segment_slots):
+        """The staged rows of the step's requests (`segment_slots`: device integer vector, one slot per
+        entry of the batch) become live.  Device work only, so a captured step holds it.  The scratch
+        request's state starts every step at zero."""
+        index = segment_slots.long()
+        for cid, live in self._states.items():
+            live.index_copy_(0, index, self._staged[cid].index_select(0, index))
+            live[self.max_slots].zero_()
+
+    def snapshot_state(self):
+        return {cid: live.clone() for cid, live in self._states.items()}
+
+    def restore_state(self, snapshot):
+        for cid, saved in snapshot.items():
+            self._states[cid].copy_(saved)
 
     def kv_bytes(self):
         return sum(t.numel() * t.element_size() for t in self._k + self._v)
@@ -292,7 +321,7 @@ class CacheManager:
         return sum(t.numel() * t.element_size() for t in self._tables)
 
     def state_bytes(self):
-        return sum(t.numel() * t.element_size() for t in self._states.values())
+        return sum(t.numel() * t.element_size() for t in list(self._states.values()) + list(self._staged.values()))
 
     # -- requests --------------------------------------------------------------------------------
     def acquire_slot(self):

@@ -98,6 +98,7 @@ class StepContext:
         self.n_tokens = 0
         self.token_ids = self.positions = self.slots = None
         self.segments = []            # (slot, first row, number of tokens, first position)
+        self.segment_slots = None     # device int32, one slot per segment (set when the model keeps state per request)
         self.single_tokens = False    # every segment brings exactly one token (a decoding step)
         self.max_context = 0          # largest position + 1 among the step's tokens
         self._groups = {}

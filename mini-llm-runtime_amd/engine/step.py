@@ -71,7 +71,7 @@ class Runner:
         self.memory_plan = MemoryPlan(
             weights=model.arena.planned if model.arena is not None else model.weight_bytes(),
             kv_pages=kv, block_tables=tables, state=state, workspace=Workspace.plan_bytes(workspace_plan),
-            metadata=4 * 4 * self.max_batch_tokens + 8, library_scratch=LIBRARY_GEMM_WORKSPACE if uses_library else 0)
+            metadata=5 * 4 * self.max_batch_tokens + 8, library_scratch=LIBRARY_GEMM_WORKSPACE if uses_library else 0)
         self.memory_plan.check(device_budget_bytes, self.device)
         self.cache = CacheManager(model.cache_entry_specs, self.dtype, self.device, page_size,
                                   max_tokens, max_slots, self.max_length)
@@ -90,8 +90,10 @@ class Runner:
                                split_keys, split_max_tokens)
         self.ctx.target_workgroups = target_workgroups
         self.ctx.status = self._status if self.check_finite else None
-        self._upload = Uploader(4 * self.max_batch_tokens, self.device)
-        self._meta = torch.empty(4 * self.max_batch_tokens, dtype=torch.int32, device=self.device)
+        # one vector a step: token ids, positions, slots (a value a token), wanted rows, and -- for a model that
+        # keeps state per request -- one slot per entry
+        self._upload = Uploader(5 * self.max_batch_tokens, self.device)
+        self._meta = torch.empty(5 * self.max_batch_tokens, dtype=torch.int32, device=self.device)
         self.poisoned = False
         self.steps = 0
         # steps of few tokens are launch-bound: after a first eager run a step's shape is captured once
@@ -173,11 +175,13 @@ class Runner:
         return seen > self.graph_after
 
     @staticmethod
-    def _replays_match(graph, result, expect):
+    def _replays_match(graph, result, expect, rewind=lambda: None):
         """Replays the fresh capture twice on the inputs of the eager run that gave `expect`; `result` is
-        the tensor that the graph writes."""
+        the tensor that the graph writes.  `rewind` is called before each replay (it puts per-request state
+        back to where the step found it)."""
         scale = max(float(expect.abs().nan_to_num(0.0).max()), 1e-30)
         for _ in range(2):
+            rewind()
             graph.replay()
             if bool(torch.isfinite(result).all()) != bool(torch.isfinite(expect).all()):
                 return False
@@ -200,10 +204,13 @@ class Runner:
             for n, want in shape:
                 rows.extend(base + w for w in want)
                 base += n
-            meta = torch.empty(3 * total + max(len(rows), 1), dtype=torch.int32, device=self.device)
+            # ids | positions | slots | one slot per entry (these change from step to step) | wanted rows (fixed)
+            n_seg = len(shape)
+            meta = torch.empty(3 * total + n_seg + max(len(rows), 1), dtype=torch.int32, device=self.device)
             if rows:
-                meta[3 * total:3 * total + len(rows)] = torch.tensor(rows, dtype=torch.int32, device=self.device)
-            state = dict(meta=meta, upload=Uploader(3 * total, self.device), graph=None, logits=None, runs=0,
+                meta[3 * total + n_seg:3 * total + n_seg + len(rows)] = torch.tensor(rows, dtype=torch.int32,
+                                                                                      device=self.device)
+            state = dict(meta=meta, upload=Uploader(3 * total + n_seg, self.device), graph=None, logits=None, runs=0,
                          rows=len(rows), groups={}, keep=None, eager=False)
             self._graphs[sig] = state
             while len(self._graphs) > self.max_graphs:
@@ -229,7 +236,8 @@ class Runner:
             slot_of.extend([e.slot] * n)
         if not fill_first:
             scratch_rows()
-        state["upload"].send(ids + pos + slot_of, meta)
+        n_seg = len(segments)
+        state["upload"].send(ids + pos + slot_of + [seg[0] for seg in segments], meta)
         if state["graph"] is not None:
             state["graph"].replay()
             return state["logits"]
@@ -237,10 +245,11 @@ class Runner:
         ctx.begin_step()
         ctx.n_tokens = total
         ctx.token_ids, ctx.positions, ctx.slots = meta[0:total], meta[total:2 * total], meta[2 * total:3 * total]
+        ctx.segment_slots = meta[3 * total:3 * total + n_seg]
         ctx.segments = segments
         ctx.single_tokens = total == len(segments)
         r = state["rows"]
-        want_rows = meta[3 * total:3 * total + r] if r else None
+        want_rows = meta[3 * total + n_seg:3 * total + n_seg + r] if r else None
         if state["eager"]:                                # a shape whose capture did not hold
             ctx.max_context = max(p0 + n for (_, _, n, p0) in segments)
             return self.model.forward(ctx, want_rows)
@@ -249,7 +258,12 @@ class Runner:
         state["runs"] += 1
         if state["runs"] == 1:                            # first time: eager, sizes the scratch buffers
             return self.model.forward(ctx, want_rows)
-        reference = self.model.forward(ctx, want_rows)    # (running a step again writes the same cache entries)
+        # The capture runs the step more than once: eagerly (the reference), then twice as a replay of the
+        # fresh graph.  Running a step again writes the same keys and values into the same pages; state of
+        # fixed size, which a step ADVANCES, is put back to where the step found it before every further run,
+        # so that it has advanced exactly once when this returns.
+        before = self.cache.snapshot_state()
+        reference = self.model.forward(ctx, want_rows)
         probe = reference if reference is not None else self.workspace.get("hidden", (total, self.model.spec.hidden),
                                                                            torch.float32)
         expect = probe.clone()
@@ -257,13 +271,16 @@ class Runner:
         with torch.cuda.graph(graph):
             logits = self.model.forward(ctx, want_rows)
         state["keep"] = self.workspace.buffers()
-        ok = self._replays_match(graph, logits if logits is not None else probe, expect)
+        ok = self._replays_match(graph, logits if logits is not None else probe, expect,
+                                 lambda: self.cache.restore_state(before))
         if not ok:
             state["eager"], state["keep"] = True, None
             self.graph_failures += 1
             ctx.fixed_groups = None
             ctx.begin_step()
+            ctx.segment_slots = meta[3 * total:3 * total + n_seg]
             ctx.max_context = max(p0 + n for (_, _, n, p0) in segments)
+            self.cache.restore_state(before)
             return self.model.forward(ctx, want_rows)
         state["graph"], state["logits"] = graph, logits
         return logits
@@ -331,7 +348,8 @@ class Runner:
                 slot_of.extend([e.slot] * n)
                 rows.extend(base + int(w) for w in e.want)
             r = len(rows)
-            self._upload.send(ids + pos + slot_of + rows, self._meta)
+            stateful = self.cache.has_state()
+            self._upload.send(ids + pos + slot_of + rows + ([seg[0] for seg in segments] if stateful else []), self._meta)
             ctx = self.ctx
             ctx.begin_step()
             ctx.n_tokens = total
@@ -342,6 +360,7 @@ class Runner:
             ctx.single_tokens = total == len(entries)
             ctx.max_context = max(p0 + n for (_, _, n, p0) in segments)
             want_rows = self._meta[3 * total:3 * total + r] if r else None
+            ctx.segment_slots = self._meta[3 * total + r:3 * total + r + len(segments)] if stateful else None
             logits = self.model.forward(ctx, want_rows)
             self.cache.retire(slots)
             self.steps += 1

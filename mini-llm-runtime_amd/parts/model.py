@@ -166,6 +166,8 @@ class DecoderModel:
                 pending = None                            # (h is complete)
             if status is not None:                        # h + pending is the hidden state after this run
                 k.finite_check(h, None if isinstance(pending, Handoff) else pending, i, status)
+        if ctx.cache is not None and ctx.cache.has_state():
+            ctx.cache.commit_state(ctx.segment_slots)     # every layer has run: the staged state becomes live
         r = 0 if want_rows is None else want_rows.numel()
         if r == 0:
             return None

@@ -26,6 +26,12 @@ Interfaces (B = the tokens of a step, E = the model width, T = the engine's elem
                   the first projection takes `hand`, the last adds into h and prepares `norm_after`.
   feed-forward    forward_handoff(ctx, hand, h, norm_after) -> Handoff | None, likewise.
 
+A mixer with state of fixed size (cache_spec() -> StateSpec) reads a request's live state from
+ctx.cache.state_view(cache_id)[slot] and leaves the state its step leads to in
+ctx.cache.state_stage(cache_id)[slot], for every slot of the step (when write_cache).  The staged rows become
+live when every layer of the step has run, so a step that fails on the way leaves the live state as it was.
+ctx.segment_slots holds the step's slots as a device vector (one a segment).
+
 A part may set the class attribute `graph_safe = True` when what it launches depends only on the step's
 SHAPE -- how many tokens each entry brings (ctx.n_tokens, the lengths in ctx.segments, ctx.single_tokens,
 ctx.token_groups) and ctx.max_context, which in a step that is to be captured is its context bucket (512, 1024,
@@ -33,7 +39,10 @@ ctx.token_groups) and ctx.max_context, which in a step that is to be captured is
 and everything else reaches its kernels through device memory (ctx.token_ids, positions, slots, the cache
 views).  Steps of a shape that comes again are then captured once as a HIP graph and replayed.  A part
 that reads the slots or positions of ctx.segments on the host, or keeps host-side state per request, must
-leave it unset; a model with such a part runs every step eagerly.
+leave it unset; a model with such a part runs every step eagerly.  The capture of a shape runs the step three
+times (an eager reference and two replays of the fresh graph, which are compared): writes of keys and values
+are the same each time, and the live state of fixed size is put back before every further run, so a part needs
+no care of its own for that.
 
 No part is told which model it is in; sizes and constants arrive through its spec.
 """

@@ -240,7 +240,7 @@ def test_graphs_that_are_dropped_or_do_not_hold(model_folders, plain_models, mod
     want = plain_logits(plain_models[name], reqs)
     model = load(model_folders, name, dtype_name)
     if mode == "mismatch":
-        monkeypatch.setattr(Runner, "_replays_match", staticmethod(lambda graph, result, expect: False))
+        monkeypatch.setattr(Runner, "_replays_match", staticmethod(lambda graph, result, expect, rewind=None: False))
     r = runner_for(model, name, max_tokens=256, max_graphs=1 if mode == "evict" else 48, graph_after=0)
     a, b = reqs["r0"], reqs["r1"]
     steps = [dict(step=0, entries=[dict(id="r0", tokens=a[:20], want=[19]), dict(id="r1", tokens=b[:30], want=[29])], end=[])]

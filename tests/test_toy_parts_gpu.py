@@ -34,7 +34,11 @@ def register_toys():
 
     @register_part("mixer", "toy_running_mean")
     class RunningMean:
-        """out_t = gain * mean(x_0 .. x_t): the state of a request is the running sum and the count."""
+        """out_t = gain * mean(x_0 .. x_t): the state of a request is the running sum and the count.  It reads
+        the live state, leaves the state its step leads to in the staged rows (the engine makes them live when
+        every layer has run), and names requests by device values only (`ctx.segment_slots`), so steps of a
+        shape that comes again are captured and replayed like any other model's."""
+        graph_safe = True
 
         def __init__(self, spec):
             self.hidden = spec.hidden
@@ -53,16 +57,17 @@ def register_toys():
             return []
 
         def forward(self, ctx, x, cache_id, write_cache=True):
-            state = ctx.cache.state_view(cache_id)
+            live, staged = ctx.cache.state_view(cache_id), ctx.cache.state_stage(cache_id)
             out = torch.empty_like(x)
-            for slot, first, n, _ in ctx.segments:
+            for i, (_, first, n, _) in enumerate(ctx.segments):       # (first, n): the step's shape
+                slot = ctx.segment_slots[i:i + 1].long()               # which request: a device value
+                row = live.index_select(0, slot)[0]
                 seg = x[first:first + n].float()
-                sums = state[slot, :self.hidden] + torch.cumsum(seg, dim=0)
-                count = state[slot, self.hidden] + torch.arange(1, n + 1, device=x.device, dtype=torch.float32)
+                sums = row[:self.hidden] + torch.cumsum(seg, dim=0)
+                count = row[self.hidden] + torch.arange(1, n + 1, device=x.device, dtype=torch.float32)
                 out[first:first + n] = (self.gain * sums / count[:, None]).to(x.dtype)
                 if write_cache:
-                    state[slot, :self.hidden] = sums[-1]
-                    state[slot, self.hidden] = count[-1]
+                    staged.index_copy_(0, slot, torch.cat([sums[-1], count[-1:]])[None])
             return out
 
     def attention(hidden, heads, kv_heads, head_dim, eps, position=None):
@@ -311,13 +316,44 @@ def test_toy_architectures_step_like_their_plain_twins(tmp_path, arch, plain, dt
     reqs = make_requests(97, [50, 23, 70, 9, 31], seed=8)
     want = {(rid, p): row for rid, toks in reqs.items() for p, row in enumerate(plain(w, toks))}
     name = "float32" if dtype == torch.float32 else "bfloat16"
+    from helpers import last_one_by_one
     r = Runner(model, max_tokens=128, max_slots=4, page_size=8)
     compare(run_steps(r, whole(reqs)), want, name)
     compare(run_steps(r, portions(reqs)), want, name)          # slots and their state are used again
+    # the last tokens one by one: the single-token step is captured (the capture runs it three times; state
+    # of fixed size must have advanced once all the same) and replayed
+    compare(run_steps(r, last_one_by_one(reqs)), want, name)
+    assert r.use_graphs and r.graph_failures == 0
+    assert r._graphs[(((1, (0,)),), 512)]["graph"] is not None
     steps, peak = mixed(reqs, seed=2)
-    r = Runner(model, max_tokens=peak, max_slots=4, page_size=8)
+    r = Runner(model, max_tokens=peak, max_slots=4, page_size=8, graph_after=1)
     compare(run_steps(r, steps), want, name)
+    assert r.use_graphs and r.graph_failures == 0 and any(st["graph"] is not None for st in r._graphs.values())
     r.cache.check()
+
+
+def test_a_step_that_fails_on_the_way_leaves_the_state_of_fixed_size_as_it_was(tmp_path):
+    """State is staged by the mixers and becomes live only when every layer has run: a step that raises in a
+    later layer leaves the live state untouched."""
+    from mini_llm_runtime_amd.engine import Entry, Runner
+    from mini_llm_runtime_amd.parts import DecoderModel
+    folder = write_folder(tmp_path, "ToyStateForTests", seed=4)
+    model = DecoderModel.load(folder, torch.float32)
+    r = Runner(model, max_tokens=128, max_slots=2, page_size=8, use_graphs=False)
+    s = r.open_request()
+    r.step([Entry(s, [3, 4, 5, 6], [3])])
+    live = r.cache.state_view(1)
+    before = live.clone()
+    assert float(before[s, -1]) == 4.0                       # the count of the running mean
+    original = model.blocks[2].mixer.forward
+
+    def broken(*args, **kwargs):
+        raise RuntimeError("layer 2 fails")
+    model.blocks[2].mixer.forward = broken
+    with pytest.raises(RuntimeError, match="layer 2 fails"):
+        r.step([Entry(s, [7, 8], [1])])
+    model.blocks[2].mixer.forward = original
+    assert r.poisoned and torch.equal(live, before)
 
 
 def plain_toy_routed(w, tokens, margins=None, chosen=None):
