@@ -1,10 +1,16 @@
-// Per-head RMSNorm of q and k, split-half rotation by position, and the write of k and v
-// into their pages of the cache: one kernel, one pass over the projection's output.
+// Per-head RMSNorm of q and k, rotation by position, and the write of k and v into their pages
+// of the cache: one kernel, one pass over the projection's output.
 //
 // Cache layout of one layer: keys pages[num_pages][kv_heads][page_size][head_dim], values transposed
 // pages[num_pages][kv_heads][head_dim][page_size]; token position p of the request in slot s lies in
-// page block_table[s][p / page_size] at row (values: column) p % page_size.  Norm sums and the rotation are computed in 32-bit; cos/sin come from a
-// float table [max_positions][head_dim] (first half cos, second half sin).
+// page block_table[s][p / page_size] at row (values: column) p % page_size.  Norm sums and the rotation are
+// computed in 32-bit.
+//
+// What is rotated is the position part's decision, not this kernel's: the first rot_dim channels of a head
+// (even, <= head_dim; the rest pass through unrotated), in pairs (j, j + rot_dim / 2) ("split-half") or
+// (2 j, 2 j + 1) ("interleaved"); pair j turns by the angle whose cosine is table[p][j] and whose sine is
+// table[p][rot_dim / 2 + j], table being float [max_positions][rot_dim].  The general kernel takes any of
+// these; the vector kernel for many rows takes the whole head in split-half pairs.
 #include "common.h"
 
 #define MAX_PAIRS 4   // head_dim / 2 <= 64 * MAX_PAIRS
@@ -16,15 +22,31 @@ __global__ void qk_norm_rope_kv_kernel(
     const int32_t* __restrict__ slots, const int32_t* __restrict__ positions,
     const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w, float eps,
     const float* __restrict__ rope, int q_heads, int kv_heads, int head_dim, int page_size,
-    int write_cache) {
+    int write_cache, int rot_dim, int interleaved) {
     const int m = blockIdx.x;
     const int lane = threadIdx.x & 63, waves = gridDim.y * (blockDim.x >> 6);
     const int wave = blockIdx.y * (blockDim.x >> 6) + (threadIdx.x >> 6);       // heads are dealt out to these
-    const int half = head_dim >> 1;
+    const int half = head_dim >> 1, rot_half = rot_dim >> 1;
     const int pos = positions[m];
     const int slot = slots[m];
     const elem_t* row = qkv + (size_t)m * ld;
-    const float* cs = rope ? rope + (size_t)pos * head_dim : nullptr;
+    const float* cs = rope ? rope + (size_t)pos * rot_dim : nullptr;
+    // pair j of a head: channels (ia, ib); rotated when j < rot_half (split-half) or 2 j < rot_dim (interleaved)
+    auto pair_of = [&](int j, int& ia, int& ib, bool& turned) {
+        if (interleaved) {
+            ia = 2 * j;
+            ib = 2 * j + 1;
+            turned = 2 * j < rot_dim;
+        } else if (j < rot_half) {
+            ia = j;
+            ib = j + rot_half;
+            turned = true;
+        } else {
+            ia = rot_dim + 2 * (j - rot_half);
+            ib = ia + 1;
+            turned = false;
+        }
+    };
 
     size_t cache_row = 0, cache_page = 0;
     bool cache_ok = false;
@@ -55,8 +77,11 @@ __global__ void qk_norm_rope_kv_kernel(
             const int j = lane + 64 * i;
             a[i] = b[i] = 0.f;
             if (j < half) {
-                a[i] = to_float(src[j]);
-                b[i] = to_float(src[j + half]);
+                int ia, ib;
+                bool turned;
+                pair_of(j, ia, ib, turned);
+                a[i] = to_float(src[ia]);
+                b[i] = to_float(src[ib]);
                 sum += a[i] * a[i] + b[i] * b[i];
             }
         }
@@ -67,8 +92,11 @@ __global__ void qk_norm_rope_kv_kernel(
             for (int i = 0; i < MAX_PAIRS; ++i) {
                 const int j = lane + 64 * i;
                 if (j < half) {
-                    a[i] = (a[i] * scale) * w[j];
-                    b[i] = (b[i] * scale) * w[j + half];
+                    int ia, ib;
+                    bool turned;
+                    pair_of(j, ia, ib, turned);
+                    a[i] = (a[i] * scale) * w[ia];
+                    b[i] = (b[i] * scale) * w[ib];
                 }
             }
         }
@@ -83,14 +111,17 @@ __global__ void qk_norm_rope_kv_kernel(
         for (int i = 0; i < MAX_PAIRS; ++i) {
             const int j = lane + 64 * i;
             if (j < half) {
+                int ia, ib;
+                bool turned;
+                pair_of(j, ia, ib, turned);
                 float x = a[i], y = b[i];
-                if (cs) {
-                    const float c = cs[j], s = cs[j + half];
+                if (cs && turned) {
+                    const float c = cs[j], s = cs[j + rot_half];
                     x = a[i] * c - b[i] * s;
                     y = a[i] * s + b[i] * c;
                 }
-                dst[j] = from_float<elem_t>(x);
-                dst[j + half] = from_float<elem_t>(y);
+                dst[ia] = from_float<elem_t>(x);
+                dst[ib] = from_float<elem_t>(y);
             }
         }
     }
@@ -274,13 +305,18 @@ extern "C" int mlr_qk_norm_rope_kv(
     const void* qkv, int ld, void* q_out, void* k_pages, void* v_pages, const int32_t* block_table,
     int max_blocks, const int32_t* slots, const int32_t* positions, const float* q_norm_w,
     const float* k_norm_w, float eps, const float* rope, int rows, int q_heads, int kv_heads,
-    int head_dim, int page_size, int write_cache, hipStream_t stream) {
+    int head_dim, int page_size, int write_cache, int rot_dim, int interleaved, hipStream_t stream) {
     if (rows <= 0) return 0;
     if (head_dim % 2 != 0 || head_dim / 2 > 64 * MAX_PAIRS) return -1;
+    if (rope == nullptr) {                                 // (no rotation: any pairing covers the head)
+        rot_dim = head_dim;
+        interleaved = 0;
+    }
+    if (rot_dim < 2 || rot_dim > head_dim || rot_dim % 2 != 0) return -2;
     const int total_heads = q_heads + 2 * kv_heads;
 #if MLR_BF16
     const int lph = head_dim / 16;
-    if (rows >= 64 && head_dim % 16 == 0 && (lph & (lph - 1)) == 0 && ld % 8 == 0) {
+    if (rows >= 64 && head_dim % 16 == 0 && (lph & (lph - 1)) == 0 && ld % 8 == 0 && rot_dim == head_dim && !interleaved) {
         // values take workgroups of their own (stores of 16 bytes into the transposed pages) when pages hold
         // a multiple of eight tokens
         const int split_values = write_cache && page_size % 8 == 0;
@@ -309,6 +345,6 @@ extern "C" int mlr_qk_norm_rope_kv(
     qk_norm_rope_kv_kernel<<<dim3(rows, chunks), 256, 0, stream>>>(
         (const elem_t*)qkv, ld, (elem_t*)q_out, (elem_t*)k_pages, (elem_t*)v_pages, block_table,
         max_blocks, slots, positions, q_norm_w, k_norm_w, eps, rope, q_heads, kv_heads, head_dim,
-        page_size, write_cache);
+        page_size, write_cache, rot_dim, interleaved);
     return (int)hipGetLastError();
 }

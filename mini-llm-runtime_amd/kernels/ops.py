@@ -364,9 +364,11 @@ class Kernels:
 
     @timed("rope_kv", _rope_work)
     def qk_norm_rope_kv(self, qkv, q_out, k_pages, v_pages, block_table, slots, positions, q_norm_w,
-                        k_norm_w, eps, rope, q_heads, kv_heads, head_dim, page_size, write_cache=True):
-        """Per head: RMSNorm of q and k (weights may be None), rotation by `rope`
-        [max_positions, head_dim] (may be None), q into q_out, k and v into their pages."""
+                        k_norm_w, eps, rope, q_heads, kv_heads, head_dim, page_size, write_cache=True,
+                        interleaved=False):
+        """Per head: RMSNorm of q and k (weights may be None), rotation by `rope` [max_positions, rot_dim]
+        (cosines | sines; may be None) of the head's first rot_dim channels in pairs (j, j + rot_dim / 2), or
+        (2 j, 2 j + 1) when `interleaved`; q into q_out, k and v into their pages."""
         _need(head_dim % 2 == 0 and 2 <= head_dim <= MAX_HEAD_DIM,
               lambda: f"head_dim {head_dim}: the rotation kernel takes even sizes up to {MAX_HEAD_DIM}")
         width = (q_heads + 2 * kv_heads) * head_dim
@@ -381,14 +383,18 @@ class Kernels:
         if q_norm_w is not None:
             _tensor(q_norm_w, "q_norm_w", torch.float32, (head_dim,))
             _tensor(k_norm_w, "k_norm_w", torch.float32, (head_dim,))
+        rot_dim = head_dim
         if rope is not None:
             _tensor(rope, "rope", torch.float32, ndim=2)
-            _need(rope.shape[1] == head_dim, "rope: table width must equal head_dim")
+            rot_dim = rope.shape[1]
+            _need(2 <= rot_dim <= head_dim and rot_dim % 2 == 0,
+                  lambda: f"rope: the table's width {rot_dim} must be even and at most head_dim {head_dim}")
         fn = self._lib("rope_kv").mlr_qk_norm_rope_kv
         _ok(fn(_p(qkv), _c_int(width), _p(q_out), _p(k_pages), _p(v_pages), _p(block_table),
                _c_int(block_table.shape[1]), _p(slots), _p(positions), _p(q_norm_w), _p(k_norm_w),
                _c_float(eps), _p(rope), _c_int(m), _c_int(q_heads), _c_int(kv_heads), _c_int(head_dim),
-               _c_int(page_size), _c_int(1 if write_cache else 0), _stream()), "qk_norm_rope_kv")
+               _c_int(page_size), _c_int(1 if write_cache else 0), _c_int(rot_dim), _c_int(1 if interleaved else 0),
+               _stream()), "qk_norm_rope_kv")
 
     def attention_partial_numel(self, rows, q_heads, head_dim, max_splits):
         """Floats of scratch memory for the partial results of split attention: per (row, head, split) the

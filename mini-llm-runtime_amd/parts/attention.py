@@ -30,9 +30,9 @@ class GqaAttention:
         self.k_norm = build_part("norm", s.qk_norm) if s.qk_norm is not None else None
         if s.qk_norm is not None and s.qk_norm.size != s.head_dim:
             raise PartError("the q/k norm must span one head")
+        # (how much of a head a position part turns, and in which pairs, is the part's own business: it says
+        # so in the `Rotation` it hands over at run time)
         self.position = build_part("position", s.position) if s.position is not None else None
-        if s.position is not None and s.position.dim != s.head_dim:
-            raise PartError("the rotation must span the whole head")
         self.qkv = None
         self.o = None
 
@@ -171,8 +171,15 @@ class GqaAttention:
         x = qkv
         m = qkv.shape[0]
         view = ctx.cache.kv_view(cache_id)
-        rope = self.position.rotation_table(ctx.max_positions, x.device) if self.position is not None else None
-        if (ctx.single_tokens and write_cache and x.dtype == torch.bfloat16
+        rotation = self.position.rotation(ctx.max_positions, x.device) if self.position is not None else None
+        if rotation is not None and not (2 <= rotation.dim <= s.head_dim and rotation.dim % 2 == 0
+                                         and rotation.table.shape[1] == rotation.dim):
+            raise PartError(f"the position part turns {rotation.dim} channels of a head of {s.head_dim}: must be "
+                            "even, at most the head, and as wide as its table")
+        rope = rotation.table if rotation is not None else None
+        interleaved = rotation is not None and rotation.interleaved
+        whole_split_half = rotation is None or (rotation.dim == s.head_dim and not rotation.interleaved)
+        if (ctx.single_tokens and write_cache and x.dtype == torch.bfloat16 and whole_split_half
                 and k.decode_fusion_supported(s.q_heads, s.kv_heads, s.head_dim, view.page_size)):
             # decoding: norm, rotation and cache write ride in the attention's two launches
             attn = ctx.workspace.get("attn", (m, s.q_heads * s.head_dim), x.dtype)
@@ -197,7 +204,7 @@ class GqaAttention:
             self.q_norm.weight if self.q_norm is not None else None,
             self.k_norm.weight if self.k_norm is not None else None,
             self.q_norm.eps if self.q_norm is not None else 0.0, rope,
-            s.q_heads, s.kv_heads, s.head_dim, view.page_size, write_cache)
+            s.q_heads, s.kv_heads, s.head_dim, view.page_size, write_cache, interleaved=interleaved)
         attn = ctx.workspace.get("attn", (m, s.q_heads * s.head_dim), x.dtype)
         if k.mfma_attention_supported(s.q_heads, s.kv_heads, s.head_dim, view.page_size):
             # prompt portions go to one of the LDS-staged kernels (the 32x32-tile one where it takes the

@@ -8,8 +8,8 @@ Interfaces (B = the tokens of a step, E = the model width, T = the engine's elem
                   forward(ctx, h, delta, out, rows=None, write_h=True): h is the float residual
                   stream [B, E]; x = h + delta (delta may be None) is written back to h when
                   write_h; out[r] = norm(x[rows[r] or r]) as T.
-  position        rotation_table(max_positions, device) -> float [max_positions, dim] with cos
-                  in the first half and sin in the second, or None for "no rotation".
+  position        rotation(max_positions, device) -> Rotation (the table of cosines and sines, how
+                  many channels of a head it turns and how they pair up), or None for "no rotation".
   mixer           weight_specs(), bind();  cache_spec() -> KvSpec | StateSpec | None;
                   libraries() -> names of the kernel libraries it launches;
                   forward(ctx, x, cache_id, write_cache) -> T [B, E], x being the normed input.
@@ -51,6 +51,18 @@ from __future__ import annotations
 from dataclasses import dataclass
 
 _REGISTRIES = {"norm": {}, "position": {}, "mixer": {}, "ffn": {}, "block": {}}
+
+
+@dataclass
+class Rotation:
+    """What a position part hands a mixer: `table` float [max_positions, dim] on the device, the cosines of
+    the pairs' angles in its first half and their sines in the second; the first `dim` channels of a head
+    (even, at most the head size) are rotated, the rest pass through; pair j is the channels
+    (j, j + dim / 2), or (2 j, 2 j + 1) when `interleaved`.  The extent and the pairing are the position
+    part's to decide; the attention part and its kernels take what they are given."""
+    table: object
+    dim: int
+    interleaved: bool = False
 
 
 @dataclass

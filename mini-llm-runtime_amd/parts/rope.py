@@ -1,14 +1,14 @@
 """Rotary position encoding over the whole head, split-half pairing (j, j + dim/2):
 freq_j = base^(-2j/dim), angle = position * freq_j held in 32-bit, as the reference computes it
 (src/minillm/runtime.cpp:231-241, table form src/minillm/cuda/storage.cpp:261-287).  The table
-[max_positions, dim] holds cos in its first half and sin in its second; the attention part's
-fused kernel reads it."""
+[max_positions, dim] holds cos in its first half and sin in its second.  The part hands the attention
+part a `Rotation`: this table, the rotated width (here the whole head) and the pairing (here split-half)."""
 from __future__ import annotations
 
 import numpy as np
 import torch
 
-from .registry import register_part
+from .registry import Rotation, register_part
 
 
 @register_part("position", "rope_split_half")
@@ -16,6 +16,10 @@ class RopeSplitHalf:
     def __init__(self, spec):
         self.dim, self.base = spec.dim, float(spec.base)
         self._tables = {}
+
+    def rotation(self, max_positions, device):
+        """The whole head in split-half pairs."""
+        return Rotation(self.rotation_table(max_positions, device), self.dim, interleaved=False)
 
     def rotation_table(self, max_positions, device):
         key = (max_positions, str(device))

@@ -303,6 +303,53 @@ def test_qk_norm_rope_kv(dtype, shape):
     assert torch.isnan(k2.float()).all()
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("case", [
+    # (q heads, kv heads, head_dim, channels turned, interleaved, rows)
+    (4, 2, 16, 8, True, 5), (4, 2, 16, 16, True, 70), (2, 1, 64, 32, False, 9), (2, 1, 64, 32, False, 130),
+    (3, 3, 48, 2, True, 4), (2, 2, 128, 64, True, 66), (1, 1, 20, 10, False, 3), (2, 1, 256, 128, False, 2)])
+def test_rotation_of_part_of_a_head_in_either_pairing(dtype, case):
+    """The rotation kernel takes the extent and the pairing from its caller: the first `turned` channels of a
+    head in pairs (j, j + turned / 2) or (2 j, 2 j + 1), the rest unrotated; the per-head norm spans the whole
+    head either way.  (70 and 130 rows: the vector kernel for many rows must not be taken for these.)"""
+    hq, hkv, d, turned, interleaved, rows = case
+    k = kernels(dtype)
+    page, eps = 16, 1e-5
+    width = (hq + 2 * hkv) * d
+    qkv = rnd((rows, width), dtype, 300)
+    qw, kw = rnd((d,), torch.float32, 301) + 1, rnd((d,), torch.float32, 302) + 1
+    n_pages = (rows + page - 1) // page + 1
+    table = torch.arange(n_pages, dtype=torch.int32).flip(0).view(1, -1).contiguous().cuda()
+    slots = torch.zeros(rows, dtype=torch.int32, device="cuda")
+    pos = torch.arange(rows, dtype=torch.int32, device="cuda")
+    angle = torch.arange(rows, dtype=torch.float64)[:, None] * (100.0 ** (-2.0 * torch.arange(turned // 2, dtype=torch.float64) / turned))[None, :]
+    rope = torch.cat([torch.cos(angle), torch.sin(angle)], dim=1).float().cuda()
+    k_pages = torch.full((n_pages, hkv, page, d), float("nan"), dtype=dtype, device="cuda")
+    v_pages = torch.full((n_pages, hkv, d, page), float("nan"), dtype=dtype, device="cuda")
+    q_out = torch.full((rows, hq * d), float("nan"), dtype=dtype, device="cuda")
+    k.qk_norm_rope_kv(qkv, q_out, k_pages, v_pages, table, slots, pos, qw, kw, eps, rope, hq, hkv, d, page,
+                      interleaved=interleaved)
+
+    def want(x, w):                                      # x [rows, heads, d] float64
+        x = x * torch.rsqrt((x * x).mean(-1, keepdim=True) + eps) * w.double().cpu()
+        c, s = torch.cos(angle)[:, None, :], torch.sin(angle)[:, None, :]
+        out = x.clone()
+        if interleaved:
+            a, b = x[..., 0:turned:2], x[..., 1:turned:2]
+            out[..., 0:turned:2], out[..., 1:turned:2] = a * c - b * s, a * s + b * c
+        else:
+            a, b = x[..., :turned // 2], x[..., turned // 2:turned]
+            out[..., :turned // 2], out[..., turned // 2:turned] = a * c - b * s, a * s + b * c
+        return out
+    x = qkv.double().cpu()
+    torch.testing.assert_close(q_out.double().cpu().view(rows, hq, d), want(x[:, :hq * d].view(rows, hq, d), qw), **tol(dtype))
+    k_want = want(x[:, hq * d:(hq + hkv) * d].view(rows, hkv, d), kw)
+    for r in range(rows):
+        pg = int(table[0, r // page])
+        torch.testing.assert_close(k_pages[pg, :, r % page].double().cpu(), k_want[r], **tol(dtype))
+        assert torch.equal(v_pages[pg, :, :, r % page].cpu(), qkv[r, (hq + hkv) * d:].view(hkv, d).cpu())
+
+
 def plain_attention(q, keys, values, scale, window):
     """One query row over its visible keys, float64.  q [Hq, D]; keys, values [L, Hkv, D]."""
     hq, hkv = q.shape[0], keys.shape[1]

@@ -84,19 +84,47 @@ def register_toys():
     @register_part("position", "toy_rotation_linear")
     class LinearRotation:
         """Split-half rotation by the angle (position + shift) / (1 + j) for the pair j: the framework's
-        attention only asks a position encoding for its table of cosines and sines."""
+        attention only asks a position encoding for its `Rotation` (table of cosines and sines, extent, pairing)."""
 
         def __init__(self, spec):
             self.dim, self.shift = spec.dim, spec.shift
             self._tables = {}
 
-        def rotation_table(self, max_positions, device):
+        def rotation(self, max_positions, device):
+            from mini_llm_runtime_amd.parts.registry import Rotation
             key = (max_positions, str(device))
             if key not in self._tables:
                 angle = linear_angles(np.arange(max_positions), self.dim, self.shift)
                 self._tables[key] = torch.from_numpy(np.concatenate([np.cos(angle), np.sin(angle)], axis=1)
                                                      .astype(np.float32)).to(device)
-            return self._tables[key]
+            return Rotation(self._tables[key], self.dim, interleaved=False)
+
+    @dataclass(frozen=True)
+    class PartialRotarySpec:
+        kind: str
+        dim: int            # the head size
+        turned: int         # how many channels of a head the part turns
+        interleaved: bool
+        base: float
+
+    @register_part("position", "toy_partial_rotary")
+    class PartialRotary:
+        """Only the first `turned` channels of a head are rotated, in pairs (2 j, 2 j + 1) or (j, j + turned / 2);
+        the rest pass through.  The extent and the pairing are this part's own: the attention part and its
+        kernels take them from the `Rotation` it hands over."""
+
+        def __init__(self, spec):
+            self.spec = spec
+            self._tables = {}
+
+        def rotation(self, max_positions, device):
+            from mini_llm_runtime_amd.parts.registry import Rotation
+            key = (max_positions, str(device))
+            if key not in self._tables:
+                angle = partial_angles(np.arange(max_positions), self.spec.turned, self.spec.base)
+                self._tables[key] = torch.from_numpy(np.concatenate([np.cos(angle), np.sin(angle)], axis=1)
+                                                     .astype(np.float32)).to(device)
+            return Rotation(self._tables[key], self.spec.turned, interleaved=self.spec.interleaved)
 
     @dataclass(frozen=True)
     class RoutedSpec:
@@ -221,12 +249,47 @@ def register_toys():
             return ModelSpec("ToyWindowForTests", self.vocab, self.hidden, (layer(1, None), layer(1, 24), layer(2, 10)),
                              (LayerRun(0, 0), LayerRun(1, 1), LayerRun(2, 2)), norm, False, 512)
 
+    @register_architecture("ToyPartialRotaryForTests")
+    class ToyPartialRotary(ToyBase):
+        """Layer 0 turns 8 of its heads' 16 channels in interleaved pairs, layer 1 (heads of 64 channels, the
+        size at which decoding would otherwise fold the rotation into the attention kernel) 32 of 64 in
+        split-half pairs."""
+
+        def model_spec(self):
+            norm = NormSpec("rmsnorm", self.hidden, 1e-5)
+            ffn = MlpSpec("swiglu", self.hidden, self.inter)
+            first = attention(self.hidden, 2, 1, 16, 1e-5, PartialRotarySpec("toy_partial_rotary", 16, 8, True, 100.0))
+            second = attention(self.hidden, 2, 2, 64, 1e-5, PartialRotarySpec("toy_partial_rotary", 64, 32, False, 1000.0))
+            return ModelSpec("ToyPartialRotaryForTests", self.vocab, self.hidden,
+                             (LayerSpec("prenorm", norm, first, norm, ffn), LayerSpec("prenorm", norm, second, norm, ffn)),
+                             (LayerRun(0, 0), LayerRun(1, 1)), norm, False, 512)
+
     return ToyState, ToyOrder, ToyRouted, ToyWindow
 
 
 def linear_angles(positions, dim, shift):
     j = np.arange(dim // 2, dtype=np.float64)
     return (np.asarray(positions, dtype=np.float64)[:, None] + shift) / (1.0 + j)[None, :]
+
+
+def partial_angles(positions, turned, base):
+    j = np.arange(turned // 2, dtype=np.float64)
+    return np.asarray(positions, dtype=np.float64)[:, None] * np.power(base, -2.0 * j / turned)[None, :]
+
+
+def partial_rotate(x, positions, turned, interleaved, base):
+    """x [T, heads, D]: the first `turned` channels of every head turned by the pairs' angles, the rest as they are."""
+    angle = partial_angles(positions, turned, base)
+    c, s = np.cos(angle)[:, None, :], np.sin(angle)[:, None, :]
+    out = x.copy()
+    if interleaved:
+        a, b = x[..., 0:turned:2], x[..., 1:turned:2]
+        out[..., 0:turned:2], out[..., 1:turned:2] = a * c - b * s, a * s + b * c
+    else:
+        half = turned // 2
+        a, b = x[..., :half], x[..., half:turned]
+        out[..., :half], out[..., half:turned] = a * c - b * s, a * s + b * c
+    return out
 
 
 _registered = []
@@ -478,3 +541,68 @@ def test_layers_with_and_without_a_window_in_one_model(tmp_path, dtype):
         assert groups[24] <= -(-24 // page) + 2 and groups[10] <= -(-10 // page) + 2, (done, groups)
     r.close_request(slot)
     assert all(r.cache.free_pages(g) == r.cache.num_pages for g in range(3))
+
+
+def plain_toy_partial_rotary(w, tokens):
+    pos = np.arange(len(tokens))
+    T = len(tokens)
+    h = P.embed(tokens, w["tok.weight"])
+    for i, (kv, d, turned, interleaved, base) in enumerate([(1, 16, 8, True, 100.0), (2, 64, 32, False, 1000.0)]):
+        lw = {k: w[f"layer{i}.mixer.{k}"] for k in ("q_proj", "k_proj", "v_proj", "o_proj")}
+        x = P.rms_norm(h, w[f"layer{i}.norm1.weight"], 1e-5)
+        q = P.rms_norm((x @ lw["q_proj"].T).reshape(T, 2, d), w[f"layer{i}.mixer.q_norm.weight"], 1e-5)
+        k = P.rms_norm((x @ lw["k_proj"].T).reshape(T, kv, d), w[f"layer{i}.mixer.k_norm.weight"], 1e-5)
+        v = (x @ lw["v_proj"].T).reshape(T, kv, d)
+        q, k = partial_rotate(q, pos, turned, interleaved, base), partial_rotate(k, pos, turned, interleaved, base)
+        h = h + P.causal_attention(q, k, v, pos, 1 / math.sqrt(d)).reshape(T, -1) @ lw["o_proj"].T
+        ffn = {k: w[f"layer{i}.ffn.{k}"] for k in ("gate_proj", "up_proj", "down_proj")}
+        h = h + P.swiglu_mlp(P.rms_norm(h, w[f"layer{i}.norm2.weight"], 1e-5), ffn)
+    return P.output_logits(h, w["out_norm.weight"], w["out.weight"], 1e-5)
+
+
+def test_the_plain_partial_rotation_is_a_rotation_of_the_turned_channels_only():
+    """Pins of the twin above: position 0 is the identity; the untouched channels stay; lengths of the pairs are
+    kept; with every channel turned in split-half pairs it is the plain implementation's own rotation."""
+    rng = np.random.default_rng(0)
+    x = rng.standard_normal((5, 2, 16))
+    pos = np.array([0, 1, 7, 100, 3])
+    for interleaved in (False, True):
+        y = partial_rotate(x, pos, 8, interleaved, 100.0)
+        np.testing.assert_allclose(y[0], x[0])
+        np.testing.assert_allclose(y[..., 8:], x[..., 8:])
+        np.testing.assert_allclose((y[..., :8] ** 2).sum(-1), (x[..., :8] ** 2).sum(-1))
+        assert np.abs(y[1:, :, :8] - x[1:, :, :8]).max() > 0.1
+    cos, sin = P.rope_cos_sin(pos, 16, 100.0)
+    # (the plain implementation holds its angles in 32-bit, as the reference does)
+    np.testing.assert_allclose(partial_rotate(x, pos, 16, False, 100.0), P.rope_rotate(x, cos, sin), atol=1e-4)
+    # interleaved pairs are the split-half ones under the permutation (2 j, 2 j + 1) <-> (j, j + half)
+    perm = np.concatenate([np.arange(0, 8, 2), np.arange(1, 8, 2)])
+    z = x.copy()
+    z[..., :8] = x[..., perm]
+    back = partial_rotate(z, pos, 8, False, 100.0)
+    np.testing.assert_allclose(partial_rotate(x, pos, 8, True, 100.0)[..., perm], back[..., :8])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_a_position_part_that_turns_part_of_a_head_in_its_own_pairs(tmp_path, dtype):
+    """A position part defined here turns half of a head's channels, in interleaved pairs in one layer and in
+    split-half pairs in the other: no file of the framework knows of it.  Whole, in portions, the last tokens
+    one by one (as captured graphs) and mixed, against the plain twin."""
+    from helpers import compare, last_one_by_one, make_requests, mixed, portions, run_steps, whole
+    from mini_llm_runtime_amd.engine import Runner
+    from mini_llm_runtime_amd.parts import DecoderModel
+    folder = write_folder(tmp_path, "ToyPartialRotaryForTests", seed=9)
+    model = DecoderModel.load(folder, dtype)
+    assert model.graph_safe()
+    w = plain_weights(folder)
+    reqs = make_requests(97, [50, 23, 70, 9, 31, 100], seed=14)
+    want = {(rid, p): row for rid, toks in reqs.items() for p, row in enumerate(plain_toy_partial_rotary(w, toks))}
+    name = "float32" if dtype == torch.float32 else "bfloat16"
+    r = Runner(model, max_tokens=128, max_slots=4, page_size=16)
+    for steps in (whole(reqs), portions(reqs), last_one_by_one(reqs)):
+        compare(run_steps(r, steps), want, name)
+    assert r.graph_failures == 0 and any(st["graph"] is not None for st in r._graphs.values())
+    steps, peak = mixed(reqs, seed=3)
+    r = Runner(model, max_tokens=peak, max_slots=4, page_size=16)
+    compare(run_steps(r, steps), want, name)
+    r.cache.check()
