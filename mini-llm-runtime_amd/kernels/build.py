@@ -25,6 +25,16 @@ ARCH = "gfx950"
 HIP_FLAGS = ["-O3", "-std=c++17", "-shared", "-fPIC", f"--offload-arch={ARCH}",
              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 HOST_FLAGS = ["-O2", "-std=c++17", "-shared", "-fPIC"]
+# MLR_HOST_SANITIZE=1 in the environment: the host library (page bookkeeping, batch forming) is built with the
+# address and undefined-behaviour sanitizers, as its own file, and loaded instead of the plain one.  The
+# process must then have the sanitizer's runtime loaded first (LD_PRELOAD=$(gcc -print-file-name=libasan.so)).
+# The reference runs its host tests the same way in CI (.github/workflows/ci.yml:60-71).  CPU code only.
+HOST_SANITIZE_FLAGS = ["-O1", "-g", "-fno-omit-frame-pointer", "-std=c++17", "-shared", "-fPIC",
+                       "-fsanitize=address,undefined", "-fno-sanitize-recover=all"]
+
+
+def host_sanitized():
+    return os.environ.get("MLR_HOST_SANITIZE", "") not in ("", "0")
 
 # name -> (sources relative to csrc/, headers it includes, depends on the element type[, extra link flags])
 HIP_LIBRARIES = {
@@ -92,9 +102,9 @@ def _plan(name, tag):
     """(output path, command, digest of everything the output depends on)."""
     if name in HOST_LIBRARIES:
         sources, headers = HOST_LIBRARIES[name]
-        out = os.path.join(_lib_dir(), f"libmlr_{name}.so")
-        cmd = [_find_cxx(), *HOST_FLAGS, "-o", out] + [os.path.join(CSRC, s) for s in sources]
-        flags = HOST_FLAGS
+        flags = HOST_SANITIZE_FLAGS if host_sanitized() else HOST_FLAGS
+        out = os.path.join(_lib_dir(), f"libmlr_{name}{'_sanitized' if host_sanitized() else ''}.so")
+        cmd = [_find_cxx(), *flags, "-o", out] + [os.path.join(CSRC, s) for s in sources]
     else:
         sources, headers, typed, *rest = HIP_LIBRARIES[name]
         link = rest[0] if rest else []
@@ -183,7 +193,7 @@ def load(name, dtype=None):
     """The ctypes library `name` for element type `dtype`, built first if need be."""
     typed = name in HIP_LIBRARIES and HIP_LIBRARIES[name][2]
     tag = dtype_tag(dtype) if typed else None
-    key = (name, tag)
+    key = (name, tag, host_sanitized() and name in HOST_LIBRARIES)
     if key in _loaded:
         return _loaded[key]
     ensure_built([name], dtype if typed else None)
@@ -193,6 +203,7 @@ def load(name, dtype=None):
     except OSError as err:
         raise BuildError(f"cannot load {out}: {err}") from None
     _loaded[key] = lib
+    lib._mlr_path = out
     return lib
 
 
