@@ -185,6 +185,7 @@ __device__ __forceinline__ void tile_group(const TileArgs& a, int grp, int kvh, 
         bf16x8 k[KN][2], v[VN][2];
         int tb;
         unsigned v_ok;               // bit i: pass i's page is mapped and its first key written
+        bool whole;                  // every key of the block is written and mapped: nothing to check or zero
     };
     // global -> registers.  No branch around a load (a load behind a branch makes the compiler wait for
     // every load in flight): addresses are clamped to valid memory, and what must read as zero is zeroed
@@ -195,6 +196,26 @@ __device__ __forceinline__ void tile_group(const TileArgs& a, int grp, int kvh, 
         st.tb = tb;
         const int pidx = (tb >> pshift) - first_page;
         const uint32_t inpage = big_page ? (tb & (P - 1)) : 0;
+        // (all blocks but a group's last, unless a window has given pages back: the same for every thread)
+        st.whole = a.window <= 0 && tb + BLOCK_KEYS <= ke;
+        if (st.whole) {
+#pragma unroll
+            for (int i = 0; i < KN; ++i) {
+                const int pg = page_lds[pidx + k_pageadd[i]];
+                const __bf16* kptr = a.k_pages + (__umul24(pg, page_stride) + inpage * D + k_off0[i]);
+                st.k[i][0] = *reinterpret_cast<const bf16x8*>(kptr);
+                st.k[i][1] = *reinterpret_cast<const bf16x8*>(kptr + 8);
+            }
+#pragma unroll
+            for (int i = 0; i < VN; ++i) {
+                const int pg = page_lds[pidx + v_pageadd[i]];
+                const __bf16* vptr = a.v_pages + (__umul24(pg, page_stride) + inpage + v_off0[i]);
+                st.v[i][0] = *reinterpret_cast<const bf16x8*>(vptr);
+                st.v[i][1] = *reinterpret_cast<const bf16x8*>(vptr + 8);
+            }
+            st.v_ok = ~0u;
+            return;
+        }
         unsigned ok = 0;
 #pragma unroll
         for (int i = 0; i < KN; ++i) {
@@ -233,7 +254,7 @@ __device__ __forceinline__ void tile_group(const TileArgs& a, int grp, int kvh, 
                 bf16x8 v0 = st.v[i][0], v1 = st.v[i][1];
                 const int key0 = st.tb + 16 * (v_m0 + VSTEP * i);
                 const bool ok = (st.v_ok >> i) & 1;
-                if (!(ok && key0 + 16 <= ke)) {
+                if (!st.whole && !(ok && key0 + 16 <= ke)) {
                     // values of keys that are not written yet, or of a page that was given back (behind a
                     // window), count as zero: their probability is zero, but zero times whatever the
                     // memory holds need not be
