@@ -8,10 +8,14 @@
 // block the wavefronts of parity 0 take keys 0..31 and those of parity 1 keys 32..63.  The two parities of
 // a column are merged through LDS at the end.
 //
-// On this GPU vector instructions run beside matrix instructions only to a small part (measured: about a
-// quarter of the shorter of the two), so the loop counts its vector instructions: offsets that do not
-// change are computed once, a thread stages 32 contiguous bytes per page lookup, the maximum of a tile
-// is taken three values at a time.
+// A wavefront's block is one chain of dependent steps (keys from LDS, eight products into one accumulator,
+// maximum, exponentials, sum, eight products more, staging), and a vector instruction that needs the result
+// of the one before it issues every 9 cycles, not every 4 (measured; 6 with eight independent chains).  A
+// group's time is therefore the length of that chain times its blocks, whatever else runs on the compute
+// unit (measured at 2 048 tokens: the last group alone on the GPU 36.6 us, the whole prompt 44.1), and the
+// loop counts its instructions: offsets that do not change are computed once, a thread stages 32 contiguous
+// bytes per page lookup, blocks whose keys are all written are staged without checks, the maximum of a
+// tile is taken three values at a time.
 //
 // Per tile of 32 keys, with v_mfma_f32_32x32x16_bf16:
 //   S^T[key][column]  = K[key][d] . Q^T[d][column]         A = 32 keys x 16 channels from LDS, B = Q (registers)
