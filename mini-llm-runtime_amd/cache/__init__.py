@@ -1,3 +1,5 @@
-from .manager import (CacheError, CacheFull, CacheManager, KvSpec, KvView, PageBook, StateSpec)
+from .manager import (PAGE, CacheError, CacheFull, CacheManager, KvSpec, KvView, PageBook, PagedSpec, PagedView,
+                      StateSpec)
 
-__all__ = ["CacheError", "CacheFull", "CacheManager", "KvSpec", "KvView", "PageBook", "StateSpec"]
+__all__ = ["PAGE", "CacheError", "CacheFull", "CacheManager", "KvSpec", "KvView", "PageBook", "PagedSpec", "PagedView",
+           "StateSpec"]

@@ -2,11 +2,13 @@
 fixed-size state per request.
 
 A model names its cache needs as one spec per cache entry (an entry is what one run of a layer
-reads and writes): `KvSpec` for a mixer that keeps keys and values, `StateSpec` for a mixer
-with state of fixed size, None for a layer without memory.  Entries with equal `KvSpec` form
-a group; a group has its own pool of pages (one page id is valid in every entry of the
-group), its own block tables and its own rule for giving pages back (all keys kept, or only a
-window).  The bookkeeping itself (free lists, tables, lengths, invariants) is native code in
+reads and writes): `PagedSpec` for a mixer that keeps something per token (`KvSpec`, keys and
+values, is the usual case of it), `StateSpec` for a mixer with state of fixed size, None for a
+layer without memory.  What a page holds is the mixer's business: the spec names the tensors
+and their shape within a page, the manager only multiplies them out.  Entries with equal specs
+form a group; a group has its own pool of pages (one page id is valid in every entry of the
+group), its own page size, its own block tables and its own rule for giving pages back (all
+tokens kept, or only a window).  The bookkeeping itself (free lists, tables, lengths, invariants) is native code in
 csrc/host/cache_manager.cpp; this module owns the device memory and keeps the device copies
 of the block tables current.
 
@@ -37,17 +39,68 @@ class CacheFull(CacheError):
     """Not enough free pages (or slots) for what was asked; nothing was changed."""
 
 
+PAGE = "page"          # stands for the page's tokens in a `PagedSpec` shape
+
+
+@dataclass(frozen=True)
+class PagedSpec:
+    """What a mixer keeps per token: named tensors, each given by its shape WITHIN a page, with `PAGE` where
+    the page's tokens go; the manager allocates [pages + 1, *shape] of each for every entry of the group.
+    `page_size` None: the engine's; `dtype` None: the engine's element type."""
+    tensors: Tuple[Tuple[str, Tuple], ...]
+    window: Optional[int] = None      # None: all tokens are kept
+    page_size: Optional[int] = None
+    dtype: Optional[torch.dtype] = None
+
+    def shape_of(self, name, page_size):
+        for n, shape in self.tensors:
+            if n == name:
+                return tuple(page_size if e == PAGE else int(e) for e in shape)
+        raise KeyError(name)
+
+    def elements_per_page(self, page_size):
+        total = 0
+        for name, _ in self.tensors:
+            count = 1
+            for e in self.shape_of(name, page_size):
+                count *= e
+            total += count
+        return total
+
+
 @dataclass(frozen=True)
 class KvSpec:
+    """Keys [kv_heads, page, head_dim] and values [kv_heads, head_dim, page]: transposed within the page,
+    so that the keys of one channel lie side by side for the matrix-core product of probabilities and
+    values."""
     kv_heads: int
     head_dim: int
     window: Optional[int] = None      # None: all keys are kept
+
+    def paged(self):
+        return PagedSpec((("k", (self.kv_heads, PAGE, self.head_dim)), ("v", (self.kv_heads, self.head_dim, PAGE))),
+                         self.window)
+
+
+def _as_paged(spec):
+    if isinstance(spec, KvSpec):
+        return spec.paged()
+    return spec if isinstance(spec, PagedSpec) else None
 
 
 @dataclass(frozen=True)
 class StateSpec:
     shape: Tuple[int, ...]
     dtype: torch.dtype = torch.float32
+
+
+@dataclass
+class PagedView:
+    tensors: dict                     # name -> [num_pages + 1, *shape within a page] (the last page: scratch)
+    block_table: torch.Tensor         # device int32 [max_slots + 1, max_blocks] (the last row: the scratch request)
+    page_size: int
+    window: Optional[int]
+    group: int
 
 
 @dataclass
@@ -214,24 +267,27 @@ class CacheManager:
     @staticmethod
     def plan(entry_specs, dtype, page_size, max_tokens, max_slots, max_length):
         """(bytes of pages, of block tables, of state slabs) that a manager with these sizes allocates:
-        per group of equal `KvSpec`s keys and values [entries, pages + 1, kv_heads, page_size, head_dim]
-        and a table [max_slots + 1, ceil(max_length / page_size)] of int32; per `StateSpec` two slabs
+        per group of equal specs every tensor of the spec as [entries, pages + 1, *shape within a page]
+        and a table [max_slots + 1, ceil(max_length / page size)] of int32; per `StateSpec` two slabs
         [max_slots + 1, *shape] (live and staged)."""
-        element = torch.empty((), dtype=dtype).element_size()
-        pages = (max_tokens + page_size - 1) // page_size + 1
-        blocks = (max_length + page_size - 1) // page_size
         groups = {}
         state = 0
         for spec in entry_specs:
-            if isinstance(spec, KvSpec):
-                groups[spec] = groups.get(spec, 0) + 1
+            paged = _as_paged(spec)
+            if paged is not None:
+                groups[paged] = groups.get(paged, 0) + 1
             elif isinstance(spec, StateSpec):
                 count = 2 * (max_slots + 1)          # live and staged rows, one more for the scratch request
                 for extent in spec.shape:
                     count *= int(extent)
                 state += count * torch.empty((), dtype=spec.dtype).element_size()
-        kv = sum(2 * n * pages * spec.kv_heads * page_size * spec.head_dim * element for spec, n in groups.items())
-        tables = len(groups) * (max_slots + 1) * blocks * 4
+        kv = tables = 0
+        for spec, n in groups.items():
+            size = spec.page_size or page_size
+            element = torch.empty((), dtype=spec.dtype or dtype).element_size()
+            pages = (max_tokens + size - 1) // size + 1
+            kv += n * pages * spec.elements_per_page(size) * element
+            tables += (max_slots + 1) * ((max_length + size - 1) // size) * 4
         return kv, tables, state
 
     def __init__(self, entry_specs, dtype, device, page_size, max_tokens, max_slots, max_length):
@@ -239,36 +295,45 @@ class CacheManager:
             raise CacheError("page_size and max_tokens must be positive")
         self.dtype, self.device, self.page_size = dtype, torch.device(device), page_size
         self.max_slots, self.max_length = max_slots, max_length
-        self.num_pages = (max_tokens + page_size - 1) // page_size
         self.book = PageBook(max_slots, max_length)
         self.entry_specs = list(entry_specs)
         self._group_of_spec = {}
         self._entry_place = {}            # cache id -> (group, index within the group)
         members = []
+        self.group_specs, self.group_page_size, self.group_pages = [], [], []
         for cid, spec in enumerate(self.entry_specs):
-            if isinstance(spec, KvSpec):
-                if spec not in self._group_of_spec:
-                    self._group_of_spec[spec] = self.book.add_group(page_size, self.num_pages, spec.window)
-                    members.append([])
-                g = self._group_of_spec[spec]
-                self._entry_place[cid] = (g, len(members[g]))
-                members[g].append(cid)
-        self.group_specs = [None] * len(members)
-        for spec, g in self._group_of_spec.items():
-            self.group_specs[g] = spec
+            paged = _as_paged(spec)
+            if paged is None:
+                continue
+            if paged not in self._group_of_spec:
+                size = paged.page_size or page_size
+                if size <= 0:
+                    raise CacheError("a group's page size must be positive")
+                pages = (max_tokens + size - 1) // size
+                self._group_of_spec[paged] = self.book.add_group(size, pages, paged.window)
+                members.append([])
+                self.group_specs.append(paged)
+                self.group_page_size.append(size)
+                self.group_pages.append(pages)
+            g = self._group_of_spec[paged]
+            self._entry_place[cid] = (g, len(members[g]))
+            members[g].append(cid)
+        self.num_pages = self.group_pages[0] if self.group_pages else (max_tokens + page_size - 1) // page_size
         # Beyond the pool and the slots of the bookkeeping, every group has one page more, every block
         # table one row more and every state slab one row more: a scratch request of one token (slot
         # `scratch_slot`, its only block mapped to that page), with which a step may fill a batch up to a
         # size it has a captured graph for.
         self.scratch_slot = max_slots
-        self._k, self._v, self._tables = [], [], []
+        self._paged, self._tables = [], []      # per group: {name: [entries, pages + 1, *shape]}, block table
         for g, spec in enumerate(self.group_specs):
-            shape = (len(members[g]), self.num_pages + 1, spec.kv_heads, page_size, spec.head_dim)
-            v_shape = (len(members[g]), self.num_pages + 1, spec.kv_heads, spec.head_dim, page_size)
-            self._k.append(torch.full(shape, float("nan"), dtype=dtype, device=self.device))
-            self._v.append(torch.full(v_shape, float("nan"), dtype=dtype, device=self.device))
+            size, pages = self.group_page_size[g], self.group_pages[g]
+            kind = spec.dtype or dtype
+            fill = float("nan") if kind.is_floating_point else 0
+            self._paged.append({name: torch.full((len(members[g]), pages + 1, *spec.shape_of(name, size)), fill,
+                                                 dtype=kind, device=self.device)
+                                for name, _ in spec.tensors})
             table = torch.full((max_slots + 1, self.book.max_blocks(g)), -1, dtype=torch.int32, device=self.device)
-            table[max_slots, 0] = self.num_pages
+            table[max_slots, 0] = pages
             self._tables.append(table)
         self._stages = {}                # group -> [pinned copy of its table, event of the last upload, in use]
         # State of fixed size: a live slab, which mixers read, and a staged one, into which they write the
@@ -281,10 +346,20 @@ class CacheManager:
                 self._staged[cid] = torch.zeros_like(self._states[cid])
 
     # -- views for the parts ---------------------------------------------------------------------
-    def kv_view(self, cache_id):
+    def paged_view(self, cache_id):
+        """What the entry keeps per token: its tensors [pages + 1, *shape within a page], the group's block
+        table, page size and window."""
         g, i = self._entry_place[cache_id]
         spec = self.group_specs[g]
-        return KvView(self._k[g][i], self._v[g][i], self._tables[g], self.page_size, spec.window, g)
+        return PagedView({name: t[i] for name, t in self._paged[g].items()}, self._tables[g],
+                         self.group_page_size[g], spec.window, g)
+
+    def kv_view(self, cache_id):
+        """The same for an entry of keys and values (`KvSpec`)."""
+        g, i = self._entry_place[cache_id]
+        spec = self.group_specs[g]
+        return KvView(self._paged[g]["k"][i], self._paged[g]["v"][i], self._tables[g], self.group_page_size[g],
+                      spec.window, g)
 
     def state_view(self, cache_id):
         """[max_slots + 1, *shape]: the requests' live state (row = slot); read it, do not write it."""
@@ -314,8 +389,17 @@ class CacheManager:
         for cid, saved in snapshot.items():
             self._states[cid].copy_(saved)
 
+    def reserve_unit(self):
+        """Tokens in which a request's whole life can be set aside so that every group has the pages for it:
+        the least common multiple of the groups' page sizes (with one group, its page size)."""
+        import math
+        unit = 1
+        for size in self.group_page_size or [self.page_size]:
+            unit = unit * size // math.gcd(unit, size)
+        return unit
+
     def kv_bytes(self):
-        return sum(t.numel() * t.element_size() for t in self._k + self._v)
+        return sum(t.numel() * t.element_size() for group in self._paged for t in group.values())
 
     def table_bytes(self):
         return sum(t.numel() * t.element_size() for t in self._tables)

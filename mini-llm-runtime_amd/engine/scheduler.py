@@ -151,7 +151,10 @@ class Engine:
                                        check_finite=check_finite, profile=profile)
         self.sampler = sampler or Sampler(self.runner.kernels, self.runner.device, max_rows=o.max_active)
         self.clock = clock
-        self.total_pages = o.context_tokens // o.block_size
+        # pages are set aside in units that every group of the cache can serve (its page size, when all
+        # groups have the same)
+        self._unit = max(o.block_size, self.runner.reserve_unit())
+        self.total_pages = o.context_tokens // self._unit
         self.free_credits = self.total_pages
         self.waiting: List[Request] = []
         self.active: List[Request] = []
@@ -238,7 +241,7 @@ class Engine:
         return events
 
     def _pages_for(self, tokens):
-        return (tokens + self.options.block_size - 1) // self.options.block_size
+        return (tokens + self._unit - 1) // self._unit
 
     # -- admission -------------------------------------------------------------------------------
     def _admit(self, req):

@@ -120,6 +120,10 @@ class Runner:
     def free_slots(self):
         return self.cache.book.free_slots()
 
+    def reserve_unit(self):
+        """Tokens in which a scheduler sets a request's pages aside (see `CacheManager.reserve_unit`)."""
+        return self.cache.reserve_unit()
+
     # -- steps as graphs -----------------------------------------------------------------------
     def _signature(self, entries):
         """What a captured step is fixed to: how many tokens every entry brings and where it wants logits."""

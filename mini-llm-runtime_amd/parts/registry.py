@@ -10,7 +10,7 @@ Interfaces (B = the tokens of a step, E = the model width, T = the engine's elem
                   write_h; out[r] = norm(x[rows[r] or r]) as T.
   position        rotation(max_positions, device) -> Rotation (the table of cosines and sines, how
                   many channels of a head it turns and how they pair up), or None for "no rotation".
-  mixer           weight_specs(), bind();  cache_spec() -> KvSpec | StateSpec | None;
+  mixer           weight_specs(), bind();  cache_spec() -> KvSpec | PagedSpec | StateSpec | None;
                   libraries() -> names of the kernel libraries it launches;
                   forward(ctx, x, cache_id, write_cache) -> T [B, E], x being the normed input.
   feed-forward    weight_specs(), bind(), libraries();  forward(ctx, x) -> T [B, E].
@@ -25,6 +25,10 @@ Interfaces (B = the tokens of a step, E = the model width, T = the engine's elem
   mixer           forward_handoff(ctx, hand, h, norm_after, cache_id, write_cache) -> Handoff | None:
                   the first projection takes `hand`, the last adds into h and prepares `norm_after`.
   feed-forward    forward_handoff(ctx, hand, h, norm_after) -> Handoff | None, likewise.
+
+A mixer that keeps something else than keys and values per token names it in a PagedSpec: tensors by their
+shape within a page, optionally a page size and an element type of its own; it finds them, with the group's
+block table, in ctx.cache.paged_view(cache_id).
 
 A mixer with state of fixed size (cache_spec() -> StateSpec) reads a request's live state from
 ctx.cache.state_view(cache_id)[slot] and leaves the state its step leads to in

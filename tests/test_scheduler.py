@@ -76,6 +76,9 @@ class FakeRunner:
     def free_slots(self):
         return self.book.free_slots()
 
+    def reserve_unit(self):
+        return self.book.groups[0][0]
+
     def open_request(self):
         s = self.book.acquire_slot()
         self.history[s] = []

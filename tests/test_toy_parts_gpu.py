@@ -70,6 +70,52 @@ def register_toys():
                     staged.index_copy_(0, slot, torch.cat([sums[-1], count[-1:]])[None])
             return out
 
+    @dataclass(frozen=True)
+    class LatentMeanSpec:
+        kind: str
+        hidden: int
+        rank: int
+        page: int
+
+    @register_part("mixer", "toy_latent_mean")
+    class LatentMean:
+        """Keeps one small vector per token, c_t = down . x_t, and gives out_t = up . mean(c_0 .. c_t).  What it
+        keeps is neither keys nor values: its spec names one tensor of its own shape, in 32-bit whatever the
+        engine's element type, in pages of its own size; the cache manager only multiplies the shape out and
+        gives the group its own pool and block tables."""
+        graph_safe = False       # slots and positions of the step's entries are read on the host
+
+        def __init__(self, spec):
+            self.spec = spec
+
+        def weight_specs(self):
+            return {"down": WeightSpec((self.spec.rank, self.spec.hidden)), "up": WeightSpec((self.spec.hidden, self.spec.rank))}
+
+        def bind(self, weights):
+            self.down, self.up = weights["down"].float(), weights["up"].float()
+
+        def cache_spec(self):
+            from mini_llm_runtime_amd.cache import PAGE, PagedSpec
+            return PagedSpec((("latent", (PAGE, self.spec.rank)),), page_size=self.spec.page, dtype=torch.float32)
+
+        def libraries(self):
+            return []
+
+        def forward(self, ctx, x, cache_id, write_cache=True):
+            view = ctx.cache.paged_view(cache_id)
+            pages, table, size = view.tensors["latent"], view.block_table, view.page_size
+            assert size == self.spec.page and pages.dtype == torch.float32
+            latent = x.float() @ self.down.t()
+            out = torch.empty_like(x)
+            for slot, first, n, pos0 in ctx.segments:
+                seen = torch.arange(0, pos0 + n, device=x.device)
+                ids = table[slot].index_select(0, seen // size).long()
+                if write_cache:
+                    pages[ids[pos0:], seen[pos0:] % size] = latent[first:first + n]
+                sums = torch.cumsum(pages[ids, seen % size], dim=0)[pos0:]
+                out[first:first + n] = ((sums / (seen[pos0:] + 1).float()[:, None]) @ self.up.t()).to(x.dtype)
+            return out
+
     def attention(hidden, heads, kv_heads, head_dim, eps, position=None):
         return AttentionSpec("gqa_attention", hidden, heads, kv_heads, head_dim, 1 / math.sqrt(head_dim),
                              NormSpec("rmsnorm", head_dim, eps),
@@ -263,6 +309,23 @@ def register_toys():
             return ModelSpec("ToyPartialRotaryForTests", self.vocab, self.hidden,
                              (LayerSpec("prenorm", norm, first, norm, ffn), LayerSpec("prenorm", norm, second, norm, ffn)),
                              (LayerRun(0, 0), LayerRun(1, 1)), norm, False, 512)
+
+    @register_architecture("ToyLatentForTests")
+    class ToyLatent(ToyBase):
+        """Layer 0: attention; layer 1: the mixer that keeps a vector of 6 numbers per token in pages of 4
+        tokens; layer 2: attention over the last 24 keys."""
+
+        def model_spec(self):
+            norm = NormSpec("rmsnorm", self.hidden, 1e-5)
+            ffn = MlpSpec("swiglu", self.hidden, self.inter)
+            full = attention(self.hidden, 2, 1, 16, 1e-5)
+            near = AttentionSpec(*[getattr(full, f) for f in (
+                "kind", "hidden", "q_heads", "kv_heads", "head_dim", "scale", "qk_norm", "position")], 24)
+            return ModelSpec("ToyLatentForTests", self.vocab, self.hidden,
+                             (LayerSpec("prenorm", norm, full, norm, ffn),
+                              LayerSpec("prenorm", norm, LatentMeanSpec("toy_latent_mean", self.hidden, 6, 4), norm, ffn),
+                              LayerSpec("prenorm", norm, near, norm, ffn)),
+                             (LayerRun(0, 0), LayerRun(1, 1), LayerRun(2, 2)), norm, False, 512)
 
     return ToyState, ToyOrder, ToyRouted, ToyWindow
 
@@ -606,3 +669,64 @@ def test_a_position_part_that_turns_part_of_a_head_in_its_own_pairs(tmp_path, dt
     r = Runner(model, max_tokens=peak, max_slots=4, page_size=16)
     compare(run_steps(r, steps), want, name)
     r.cache.check()
+
+
+def plain_toy_latent(w, tokens):
+    pos = np.arange(len(tokens))
+    h = P.embed(tokens, w["tok.weight"])
+    for i in range(3):
+        x = P.rms_norm(h, w[f"layer{i}.norm1.weight"], 1e-5)
+        if i == 1:
+            latent = x @ w["layer1.mixer.down"].T
+            mixed = (np.cumsum(latent, axis=0) / (pos + 1)[:, None]) @ w["layer1.mixer.up"].T
+        else:
+            mixed = P.attention_block(x, plain_layer_weights(w, i), dict(ATTN_CFG, num_key_value_heads=1), pos,
+                                      24 if i == 2 else None)
+        h = h + mixed
+        ffn = {k: w[f"layer{i}.ffn.{k}"] for k in ("gate_proj", "up_proj", "down_proj")}
+        h = h + P.swiglu_mlp(P.rms_norm(h, w[f"layer{i}.norm2.weight"], 1e-5), ffn)
+    return P.output_logits(h, w["out_norm.weight"], w["out.weight"], 1e-5)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_a_mixer_that_keeps_something_of_its_own_per_token_in_pages_of_its_own_size(tmp_path, dtype):
+    """What a page holds is the mixer's business: a spec that names one tensor of its own shape, element type
+    and page size gets a pool, block tables and views like keys and values do, without a change to the cache
+    manager; pages of every pool are counted, given back and used again."""
+    from helpers import compare, make_requests, mixed, portions, run_steps, whole
+    from mini_llm_runtime_amd.cache import CacheManager, KvSpec, PagedSpec
+    from mini_llm_runtime_amd.engine import Entry, Runner
+    from mini_llm_runtime_amd.parts import DecoderModel
+    folder = write_folder(tmp_path, "ToyLatentForTests", seed=11)
+    model = DecoderModel.load(folder, dtype)
+    assert [type(s) for s in model.cache_entry_specs] == [KvSpec, PagedSpec, KvSpec]
+    w = plain_weights(folder)
+    reqs = make_requests(97, [50, 23, 70, 9, 31], seed=12)
+    want = {(rid, p): row for rid, toks in reqs.items() for p, row in enumerate(plain_toy_latent(w, toks))}
+    name = "float32" if dtype == torch.float32 else "bfloat16"
+    r = Runner(model, max_tokens=128, max_slots=4, page_size=16)
+    cache = r.cache
+    assert cache.group_page_size == [16, 4, 16] and cache.group_pages == [8, 32, 8]
+    latent = cache.paged_view(1).tensors["latent"]
+    assert latent.shape == (33, 4, 6) and latent.dtype == torch.float32          # (one page more: the scratch request's)
+    assert cache.kv_view(0).k_pages.shape == (9, 1, 16, 16) and cache.kv_view(0).v_pages.shape == (9, 1, 16, 16)
+    # the plan counts what is allocated, tensor by tensor
+    kv, tables, state = CacheManager.plan(model.cache_entry_specs, dtype, 16, 128, 4, r.max_length)
+    assert (kv, tables, state) == (cache.kv_bytes(), cache.table_bytes(), 0)
+    compare(run_steps(r, whole(reqs)), want, name)
+    compare(run_steps(r, portions(reqs)), want, name)
+    steps, peak = mixed(reqs, seed=5)
+    r = Runner(model, max_tokens=peak, max_slots=4, page_size=16)
+    compare(run_steps(r, steps), want, name)
+    r.cache.check()
+    # one request in portions: every pool holds what its rule says, in pages of its own size
+    r = Runner(model, max_tokens=128, max_slots=4, page_size=16)
+    slot, toks = r.open_request(), reqs["r2"]
+    for at in range(0, len(toks), 13):
+        r.step([Entry(slot, toks[at:at + 13], [])])
+        done = min(at + 13, len(toks))
+        held = [r.cache.group_pages[g] - r.cache.free_pages(g) for g in range(3)]
+        assert held[0] == -(-done // 16) and held[1] == -(-done // 4) and held[2] <= -(-24 // 16) + 2, (done, held)
+    r.close_request(slot)
+    assert all(r.cache.free_pages(g) == r.cache.group_pages[g] for g in range(3))
+
