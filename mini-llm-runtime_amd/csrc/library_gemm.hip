@@ -7,8 +7,9 @@
 // its own estimate, and the first call of a shape runs each of them on the caller's operands and keeps the
 // fastest (the estimate is off by up to 2x at a few hundred rows and by 5-10 % on some large shapes); only
 // row counts that are likely to come again are timed, see below.  While the stream
-// is being captured nothing can be timed; then the library's first candidate is taken, and the choice is
-// made again by the next call outside a capture.  The caller brings the workspace (the same for every
+// is being captured nothing can be timed; a shape that is first met there keeps the library's first candidate
+// for good, so that a captured step and a later eager step of the same shape never use different algorithms
+// (the engine runs every shape eagerly before it captures it).  The caller brings the workspace (the same for every
 // call, so that calls on one stream may follow each other without clearing it).
 #include <hip/hip_runtime.h>
 #include <hipblaslt/hipblaslt.h>
@@ -145,6 +146,8 @@ extern "C" int mlr_library_gemm(const void* a, const void* w, void* out, int M, 
         hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
         if (hipStreamIsCapturing(stream, &capturing) == hipSuccess && capturing == hipStreamCaptureStatusNone)
             choose_by_time(p, a, w, out, workspace, workspace_bytes, stream);
+        else
+            p.timed = true;        // chosen: the first candidate, which the graph now holds
     }
     const float one = 1.0f, zero = 0.0f;
     const hipblasStatus_t st = hipblasLtMatmul(g_handle, p.desc, &one, w, p.a, a, p.b, &zero, out, p.c, out, p.c,
