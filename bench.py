@@ -93,7 +93,7 @@ class Bench:
         torch, c = self.torch, self.cfg
         if self.args.fill == "random":
             runner.cache.commit(slots, [tokens] * len(slots))
-            for slab in runner.cache._k + runner.cache._v:
+            for slab in runner.cache.paged_tensors():
                 slab.normal_()
             return
         for s in slots:

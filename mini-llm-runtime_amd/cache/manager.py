@@ -398,8 +398,13 @@ class CacheManager:
             unit = unit * size // math.gcd(unit, size)
         return unit
 
+    def paged_tensors(self):
+        """Every group's tensors, [entries, pages + 1, *shape within a page] each (a benchmark fills them with
+        noise instead of running a prompt)."""
+        return [t for group in self._paged for t in group.values()]
+
     def kv_bytes(self):
-        return sum(t.numel() * t.element_size() for group in self._paged for t in group.values())
+        return sum(t.numel() * t.element_size() for t in self.paged_tensors())
 
     def table_bytes(self):
         return sum(t.numel() * t.element_size() for t in self._tables)
