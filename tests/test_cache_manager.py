@@ -212,3 +212,39 @@ def test_commit_reports_first_positions():
         b.commit_first([s0, 2], [1, 1])
     assert (b.table() == before[0]).all() and (b.free_pages(), b.length(s0), b.length(s1)) == before[1:]
     b.check()
+
+
+def test_a_spec_names_what_a_page_holds_and_groups_have_page_sizes_of_their_own():
+    """What is allocated follows from the specs alone: every tensor of a spec as [entries, pages + 1, *shape
+    within a page], pages of the group's own size and element type; equal specs share a group.  (On the CPU:
+    the manager's memory is ordinary tensors there.)"""
+    import torch
+
+    from mini_llm_runtime_amd.cache import PAGE, CacheManager, KvSpec, PagedSpec, StateSpec
+    latent = PagedSpec((("latent", (PAGE, 6)), ("gate", (3, PAGE))), page_size=4, dtype=torch.float32)
+    specs = [KvSpec(2, 16), latent, KvSpec(2, 16), StateSpec((5,), torch.float32), KvSpec(2, 16, window=24), None, latent]
+    m = CacheManager(specs, torch.bfloat16, "cpu", page_size=16, max_tokens=100, max_slots=3, max_length=64)
+    assert m.group_page_size == [16, 4, 16] and m.group_pages == [7, 25, 7]
+    assert m.kv_view(0).k_pages.shape == (8, 2, 16, 16) and m.kv_view(2).v_pages.shape == (8, 2, 16, 16)
+    assert m.kv_view(0).group == m.kv_view(2).group != m.kv_view(4).group
+    first, second = m.paged_view(1), m.paged_view(6)
+    assert first.group == second.group and first.page_size == 4 and first.window is None
+    assert first.tensors["latent"].shape == (26, 4, 6) and first.tensors["gate"].shape == (26, 3, 4)
+    assert first.tensors["latent"].dtype == torch.float32 and m.kv_view(0).k_pages.dtype == torch.bfloat16
+    assert first.tensors["latent"].data_ptr() != second.tensors["latent"].data_ptr()
+    assert first.block_table.shape == (4, 16) and m.kv_view(0).block_table.shape == (4, 4)
+    assert torch.isnan(first.tensors["latent"]).all()                  # a never-written page shows
+    planned = CacheManager.plan(specs, torch.bfloat16, 16, 100, 3, 64)
+    assert planned == (m.kv_bytes(), m.table_bytes(), m.state_bytes())
+    assert m.kv_bytes() == 3 * 8 * 2 * (2 * 16 * 16) * 2 + 2 * 26 * (4 * 6 + 3 * 4) * 4
+    assert m.reserve_unit() == 16
+    # a request takes pages of every group, each in its own size, and gives them all back
+    slot = m.acquire_slot()
+    m.prepare([slot], [21])
+    m.commit([slot], [21])
+    assert [m.group_pages[g] - m.free_pages(g) for g in range(3)] == [2, 6, 2]
+    m.release_slot(slot)
+    assert [m.free_pages(g) for g in range(3)] == m.group_pages
+    m.check()
+    odd = CacheManager([KvSpec(1, 16), PagedSpec((("x", (PAGE,)),), page_size=24)], torch.float32, "cpu", 16, 96, 2, 96)
+    assert odd.reserve_unit() == 48
