@@ -206,14 +206,20 @@ struct SkinnyEpilogue {
     const float* next_w;      // [N] weights of the norm that follows, or null
     __bf16* x_out;            // [M][N]
     float* ss_out;            // [M][gridDim.x]
+    int cols;                 // PAIR: the output columns of a workgroup, 17..32 (otherwise 16, whatever this says)
 };
 
-template <int MT, bool OUT_FLOAT, bool GATED, int UMAX = 4, bool STAGE = false, int EPI = EPI_NONE>   // UMAX: the most groups of k a turn takes
+// PAIR: a workgroup owns `cols` (17..32) output columns, two strips side by side, the second one partly
+// used: for a number of columns that deals strips of 16 unevenly to the compute units (384 strips on 256
+// units take as long as 512), 24 columns a workgroup give every unit the same work.  The second strip
+// rides where GATED keeps its second matrix.
+template <int MT, bool OUT_FLOAT, bool GATED, int UMAX = 4, bool STAGE = false, int EPI = EPI_NONE, bool PAIR = false>   // UMAX: the most groups of k a turn takes
 __global__ __launch_bounds__(SKINNY_WAVES * 64) void gemm_skinny_kernel(const __bf16* __restrict__ a,
                                                                const __bf16* __restrict__ w,
                                                                void* __restrict__ out_raw, int M, int N, int K,
                                                                SkinnyEpilogue epi) {
-    constexpr int NW = GATED ? 2 : 1;
+    constexpr int NW = (GATED || PAIR) ? 2 : 1;
+    static_assert(!PAIR || (MT == 1 && !GATED && !STAGE && EPI != EPI_RESIDUAL), "two strips: a plain product of few rows");
     static_assert(!STAGE || MT == 1, "the activation is staged for at most 16 rows");
     static_assert(EPI == EPI_NONE || MT == 1, "the norm is handed over for at most 16 rows");
     static_assert(EPI != EPI_RESIDUAL || (!GATED && !OUT_FLOAT), "the residual sum follows a plain projection");
@@ -222,7 +228,11 @@ __global__ __launch_bounds__(SKINNY_WAVES * 64) void gemm_skinny_kernel(const __
     extern __shared__ __attribute__((aligned(16))) char staged[];   // [SKINNY_WAVES][M][pitch] when STAGE
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r16 = lane & 15, b = lane >> 4;
-    const int n0 = blockIdx.x * 16;
+    const int cols = PAIR ? epi.cols : 16;
+    const int n0 = blockIdx.x * cols;
+    const int last_row = PAIR ? min(N - 1, n0 + cols - 1) : N - 1;     // (PAIR: rows beyond the workgroup's columns read its last one)
+    // this lane's weight row for g = 0 and for g = 1 (GATED: the same row of the second matrix; PAIR: 16 rows on)
+    const int wrow_of[2] = {min(n0 + r16, N - 1), GATED ? N + min(n0 + r16, N - 1) : min(n0 + 16 + r16, last_row)};
     const bool vector_ok = (K % 8) == 0;
     const int steps = (K + 31) / 32;
     const int per_wave = (steps + SKINNY_WAVES - 1) / SKINNY_WAVES;
@@ -268,7 +278,9 @@ __global__ __launch_bounds__(SKINNY_WAVES * 64) void gemm_skinny_kernel(const __
         const int groups = steps / W;
         const int per_wave_g = (groups + SKINNY_WAVES - 1) / SKINNY_WAVES;
         const int g_begin = wave * per_wave_g, g_end = min(groups, g_begin + per_wave_g);
-        const __bf16* wrow = w + (size_t)min(n0 + r16, N - 1) * K + b * (8 * W);
+        const __bf16* wrow[NW];
+#pragma unroll
+        for (int g = 0; g < NW; ++g) wrow[g] = w + (size_t)wrow_of[g] * K + b * (8 * W);
         const __bf16* xrow[MT];
 #pragma unroll
         for (int i = 0; i < MT; ++i) xrow[i] = a + (size_t)min(16 * i + r16, M - 1) * K + b * (8 * W);
@@ -304,7 +316,7 @@ __global__ __launch_bounds__(SKINNY_WAVES * 64) void gemm_skinny_kernel(const __
                 for (int g = 0; g < NW; ++g)
 #pragma unroll
                     for (int c = 0; c < W; ++c)
-                        wf[g][u][c] = *reinterpret_cast<const bf16x8*>(wrow + (size_t)g * N * K + (g0 + u) * (32 * W) + 8 * c);
+                        wf[g][u][c] = *reinterpret_cast<const bf16x8*>(wrow[g] + (g0 + u) * (32 * W) + 8 * c);
             __builtin_amdgcn_sched_barrier(0);            // or the compiler spreads the loads among the products
             if constexpr (STAGE) {
                 // LDS serves a wavefront's accesses in their order: the reads below see these writes, and
@@ -343,7 +355,7 @@ __global__ __launch_bounds__(SKINNY_WAVES * 64) void gemm_skinny_kernel(const __
             const int k = s * 32 + b * 8;
             bf16x8 wf[NW];
 #pragma unroll
-            for (int g = 0; g < NW; ++g) wf[g] = load_k8(w + (size_t)g * N * K, n0 + r16, N, k, K, vector_ok);
+            for (int g = 0; g < NW; ++g) wf[g] = load_k8(w, wrow_of[g], GATED ? 2 * N : N, k, K, vector_ok);
 #pragma unroll
             for (int i = 0; i < MT; ++i) {
                 const bf16x8 xf = load_k8(a, 16 * i + r16, M, k, K, vector_ok);
@@ -390,6 +402,13 @@ __global__ __launch_bounds__(SKINNY_WAVES * 64) void gemm_skinny_kernel(const __
             float y = v[0];
             if (GATED) y = (v[0] / (1.0f + expf(-v[0]))) * v[NW - 1];
             y4[i][r] = y;
+            if constexpr (PAIR) {                         // the second strip's sum of this lane: column n0 + 16 + 4 b + r
+                const int n = n0 + 16 + 4 * b + r;
+                if (r16 < M && n <= last_row) {
+                    if (OUT_FLOAT) ((float*)out_raw)[(size_t)r16 * N + n] = v[1];
+                    else ((__bf16*)out_raw)[(size_t)r16 * N + n] = (__bf16)v[1];
+                }
+            }
         }
     }
     if constexpr (EPI == EPI_RESIDUAL) {
@@ -448,9 +467,41 @@ __global__ __launch_bounds__(SKINNY_WAVES * 64) void gemm_skinny_kernel(const __
     }
 }
 
+// Columns of a workgroup when two strips side by side deal the work out more evenly than strips of 16 do, else 0.
+// Only where the weight is long enough for the memory's rate to count (k from 2048).
+static int skinny_pair_columns(int N, int K) {
+    static int units = 0;
+    if (units == 0) {
+        int device = 0;
+        if (hipGetDevice(&device) != hipSuccess ||
+            hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || units <= 0)
+            units = -1;
+    }
+    if (units < 0 || K < 2048 || N % 4 != 0) return 0;
+    const int strips = (N + 15) / 16;
+    const int turns = (strips + units - 1) / units;       // strips of 16: the busiest unit's share, in strips
+    for (int j = 1; j <= 4; ++j) {
+        const int cols = (((N + units * j - 1) / (units * j)) + 3) / 4 * 4;
+        if (cols > 32) continue;
+        if (cols <= 16) break;
+        return (double)(j * cols) < 0.9 * 16.0 * turns ? cols : 0;
+    }
+    return 0;
+}
+
 template <int MT, bool OUT_FLOAT, bool GATED, int UMAX, bool STAGE, int EPI>
 static int launch_skinny_kernel(const void* a, const void* w, void* out, int M, int N, int K, size_t lds,
                                 const SkinnyEpilogue& epi, hipStream_t stream) {
+    if constexpr (MT == 1 && !GATED && !STAGE && EPI != EPI_RESIDUAL && UMAX == 4) {
+        const int cols = skinny_pair_columns(N, K);
+        if (cols > 0) {
+            SkinnyEpilogue e = epi;
+            e.cols = cols;
+            gemm_skinny_kernel<MT, OUT_FLOAT, false, 4, false, EPI, true>
+                <<<dim3((N + cols - 1) / cols), SKINNY_WAVES * 64, 0, stream>>>((const __bf16*)a, (const __bf16*)w, out, M, N, K, e);
+            return (int)hipGetLastError();
+        }
+    }
     auto* kernel = gemm_skinny_kernel<MT, OUT_FLOAT, GATED, UMAX, STAGE, EPI>;
     if (STAGE) {                                          // static and dynamic LDS together may pass 64 KB
         static const hipError_t allowed = hipFuncSetAttribute(
@@ -481,7 +532,8 @@ static int launch_skinny(const void* a, const void* w, void* out, int M, int N, 
         // extra step costs what it saves, and the gated variant, whose turns would have to shrink to stay
         // within the registers of two workgroups a compute unit, gains nothing.)
         const size_t lds = (size_t)SKINNY_WAVES * M * SKINNY_STAGE_PITCH(4);
-        if (M >= 2 && K % 64 == 0 && K > 2048 && lds <= SKINNY_STAGE_LDS)
+        const bool pair = EPI != EPI_RESIDUAL && skinny_pair_columns(N, K) > 0;     // (two strips: without the stage)
+        if (!pair && M >= 2 && K % 64 == 0 && K > 2048 && lds <= SKINNY_STAGE_LDS)
             return launch_skinny_as<MT, GATED, 4, true, EPI>(a, w, out, M, N, K, out_float, lds, epi, stream);
     }
     if (short_k) return launch_skinny_as<MT, GATED, 2, false, EPI>(a, w, out, M, N, K, out_float, 0, epi, stream);

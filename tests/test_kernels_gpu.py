@@ -137,6 +137,35 @@ def test_gemm(dtype, mnk):
             torch.testing.assert_close(out.double(), want, **t)
 
 
+@pytest.mark.parametrize("mnk", [(8, 6144, 2048), (3, 6100, 2048), (16, 5120, 2112), (1, 10240, 2048), (5, 4100, 4096)])
+def test_gemm_two_strips_a_workgroup(mnk):
+    """Few rows and numbers of columns that would deal strips of 16 unevenly to the compute units: a workgroup
+    then owns two strips side by side (24, 20, ... columns), the last workgroup fewer.  Plain and with the rows'
+    scale of a norm that was handed over; rows stay independent of the batch."""
+    m, n, kk = mnk
+    k = kernels(torch.bfloat16)
+    a = rnd((m, kk), torch.bfloat16, 17)
+    w = rnd((n, kk), torch.bfloat16, 18)
+    want = a.double() @ w.double().T
+    for out_dtype in (torch.bfloat16, torch.float32):
+        out = torch.full((m, n), float("nan"), dtype=out_dtype, device="cuda")
+        k.gemm(a, w, out)
+        t = dict(atol=1e-4 * math.sqrt(kk), rtol=1e-5) if out_dtype == torch.float32 else \
+            dict(atol=2e-2 * math.sqrt(kk) / 4, rtol=2e-2)
+        torch.testing.assert_close(out.double(), want, **t)
+    one = torch.empty((1, n), dtype=torch.bfloat16, device="cuda")
+    k.gemm(a[m - 1:].contiguous(), w, one)
+    assert torch.equal(one[0], out.to(torch.bfloat16)[m - 1]) or out_dtype != torch.bfloat16
+    full = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
+    k.gemm(a, w, full)
+    assert torch.equal(one[0], full[m - 1])
+    ss = (torch.rand((m, k.handoff_parts(kk)), device="cuda") + 0.5).float()
+    scaled = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    k.gemm_prenormed(a, ss, 1e-6, w, scaled)
+    scale = 1.0 / torch.sqrt(ss.double().sum(dim=1) / kk + 1e-6)
+    torch.testing.assert_close(scaled.double(), want * scale[:, None], atol=2e-2 * math.sqrt(kk) / 4, rtol=2e-2)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_gemm_rows_do_not_depend_on_the_batch(dtype):
     """A row's result is the same bits whatever rows stand beside it.  The float kernel has one order of
