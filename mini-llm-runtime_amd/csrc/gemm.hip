@@ -207,6 +207,7 @@ struct SkinnyEpilogue {
     __bf16* x_out;            // [M][N]
     float* ss_out;            // [M][gridDim.x]
     int cols;                 // PAIR: the output columns of a workgroup, 17..32 (otherwise 16, whatever this says)
+    int ss_stride;            // floats between the rows of ss_out (its capacity: a strip of 16 a part)
 };
 
 // PAIR: a workgroup owns `cols` (17..32) output columns, two strips side by side, the second one partly
@@ -219,7 +220,7 @@ __global__ __launch_bounds__(SKINNY_WAVES * 64) void gemm_skinny_kernel(const __
                                                                void* __restrict__ out_raw, int M, int N, int K,
                                                                SkinnyEpilogue epi) {
     constexpr int NW = (GATED || PAIR) ? 2 : 1;
-    static_assert(!PAIR || (MT == 1 && !GATED && !STAGE && EPI != EPI_RESIDUAL), "two strips: a plain product of few rows");
+    static_assert(!PAIR || (MT == 1 && !GATED && !STAGE), "two strips: a plain product of few rows");
     static_assert(!STAGE || MT == 1, "the activation is staged for at most 16 rows");
     static_assert(EPI == EPI_NONE || MT == 1, "the norm is handed over for at most 16 rows");
     static_assert(EPI != EPI_RESIDUAL || (!GATED && !OUT_FLOAT), "the residual sum follows a plain projection");
@@ -241,6 +242,7 @@ __global__ __launch_bounds__(SKINNY_WAVES * 64) void gemm_skinny_kernel(const __
     // (no branch around a load); only wavefront 0 uses it.
     float ss_mine = 0.f;                                   // EPI_SCALE: this lane's share of the row's partial sums
     float4 h4 = make_float4(0.f, 0.f, 0.f, 0.f), nw4 = h4;  // EPI_RESIDUAL: h and the next norm's weights at (row r16, columns n0 + 4 b ..)
+    float4 h4b = h4, nw4b = h4;                            // ... and, PAIR, at the second strip's columns n0 + 16 + 4 b ..
     if constexpr (EPI == EPI_SCALE) {
         // the row's partial sums are dealt out to the 32 (wavefront, lane block) pairs in runs of q; a run is
         // added in ascending order, the four runs of a wavefront as (0 + 1) + (2 + 3), the wavefronts in the
@@ -260,6 +262,11 @@ __global__ __launch_bounds__(SKINNY_WAVES * 64) void gemm_skinny_kernel(const __
         if ((N & 3) == 0) {
             h4 = *reinterpret_cast<const float4*>(epi.h + at);
             if (epi.next_w) nw4 = *reinterpret_cast<const float4*>(epi.next_w + n);
+            if constexpr (PAIR) {                         // (PAIR is only launched for N and cols that are multiples of 4)
+                const int n2 = min(n0 + 16 + 4 * b, N - 4);
+                h4b = *reinterpret_cast<const float4*>(epi.h + (size_t)min(r16, M - 1) * N + n2);
+                if (epi.next_w) nw4b = *reinterpret_cast<const float4*>(epi.next_w + n2);
+            }
         }
     }
     floatx4 acc[NW][MT];
@@ -388,6 +395,7 @@ __global__ __launch_bounds__(SKINNY_WAVES * 64) void gemm_skinny_kernel(const __
         row_scale = 1.0f / sqrtf(total * epi.inv_size + epi.eps);
     }
     float y4[MT][4];
+    float y4b[4] = {0.f, 0.f, 0.f, 0.f};                   // PAIR: the second strip's sums of this lane
 #pragma unroll
     for (int i = 0; i < MT; ++i) {
 #pragma unroll
@@ -402,7 +410,8 @@ __global__ __launch_bounds__(SKINNY_WAVES * 64) void gemm_skinny_kernel(const __
             float y = v[0];
             if (GATED) y = (v[0] / (1.0f + expf(-v[0]))) * v[NW - 1];
             y4[i][r] = y;
-            if constexpr (PAIR) {                         // the second strip's sum of this lane: column n0 + 16 + 4 b + r
+            if constexpr (PAIR) y4b[r] = v[1];
+            if constexpr (PAIR && EPI != EPI_RESIDUAL) {  // the second strip's sum of this lane: column n0 + 16 + 4 b + r
                 const int n = n0 + 16 + 4 * b + r;
                 if (r16 < M && n <= last_row) {
                     if (OUT_FLOAT) ((float*)out_raw)[(size_t)r16 * N + n] = v[1];
@@ -445,6 +454,40 @@ __global__ __launch_bounds__(SKINNY_WAVES * 64) void gemm_skinny_kernel(const __
                     if (epi.next_w) epi.x_out[at] = (__bf16)(x[r] * epi.next_w[n + r]);
                 }
             }
+        }
+        if constexpr (PAIR) {
+            // the second strip, whole groups of four columns: first its squares on their own, (0 + 1) + (2 + 3)
+            // like the first strip's, then added to them
+            const int n2 = n0 + 16 + 4 * b;
+            const bool ok = row_ok && n2 + 3 <= last_row;
+            const float hv[4] = {h4b.x, h4b.y, h4b.z, h4b.w}, wv[4] = {nw4b.x, nw4b.y, nw4b.z, nw4b.w};
+            float x2[4], sq2 = 0.f;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                x2[r] = ok ? hv[r] + y4b[r] : 0.f;
+                sq2 += x2[r] * x2[r];
+            }
+            if (ok) {
+                *reinterpret_cast<float4*>(epi.h + (size_t)r16 * N + n2) = make_float4(x2[0], x2[1], x2[2], x2[3]);
+                if (epi.next_w) {
+                    typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;
+                    *reinterpret_cast<bf16x4*>(epi.x_out + (size_t)r16 * N + n2) =
+                        bf16x4{(__bf16)(x2[0] * wv[0]), (__bf16)(x2[1] * wv[1]), (__bf16)(x2[2] * wv[2]), (__bf16)(x2[3] * wv[3])};
+                }
+            }
+            if (epi.next_w) {
+                sq += __shfl_xor(sq, 16, MLR_WAVE);
+                sq += __shfl_xor(sq, 32, MLR_WAVE);
+                sq2 += __shfl_xor(sq2, 16, MLR_WAVE);
+                sq2 += __shfl_xor(sq2, 32, MLR_WAVE);
+                if (b == 0 && row_ok) {
+                    // a workgroup a part; the parts beyond the workgroups, up to the buffer's capacity, are zero
+                    float* parts = epi.ss_out + (size_t)r16 * epi.ss_stride;
+                    parts[blockIdx.x] = sq + sq2;
+                    if ((int)(gridDim.x + blockIdx.x) < epi.ss_stride) parts[gridDim.x + blockIdx.x] = 0.f;
+                }
+            }
+            return;
         }
         if (epi.next_w) {
             sq += __shfl_xor(sq, 16, MLR_WAVE);            // (0 + 1) + (2 + 3) over the lane blocks: the strip's 16 columns
@@ -492,11 +535,13 @@ static int skinny_pair_columns(int N, int K) {
 template <int MT, bool OUT_FLOAT, bool GATED, int UMAX, bool STAGE, int EPI>
 static int launch_skinny_kernel(const void* a, const void* w, void* out, int M, int N, int K, size_t lds,
                                 const SkinnyEpilogue& epi, hipStream_t stream) {
-    if constexpr (MT == 1 && !GATED && !STAGE && EPI != EPI_RESIDUAL && UMAX == 4) {
+    if constexpr (MT == 1 && !GATED && !STAGE && UMAX == 4) {
         const int cols = skinny_pair_columns(N, K);
         if (cols > 0) {
             SkinnyEpilogue e = epi;
             e.cols = cols;
+            e.ss_stride = (N + 15) / 16;
+            // (the parts beyond the workgroups are zeroed by the workgroups themselves: there are at most as many)
             gemm_skinny_kernel<MT, OUT_FLOAT, false, 4, false, EPI, true>
                 <<<dim3((N + cols - 1) / cols), SKINNY_WAVES * 64, 0, stream>>>((const __bf16*)a, (const __bf16*)w, out, M, N, K, e);
             return (int)hipGetLastError();
@@ -532,7 +577,7 @@ static int launch_skinny(const void* a, const void* w, void* out, int M, int N, 
         // extra step costs what it saves, and the gated variant, whose turns would have to shrink to stay
         // within the registers of two workgroups a compute unit, gains nothing.)
         const size_t lds = (size_t)SKINNY_WAVES * M * SKINNY_STAGE_PITCH(4);
-        const bool pair = EPI != EPI_RESIDUAL && skinny_pair_columns(N, K) > 0;     // (two strips: without the stage)
+        const bool pair = skinny_pair_columns(N, K) > 0;     // (two strips: without the stage)
         if (!pair && M >= 2 && K % 64 == 0 && K > 2048 && lds <= SKINNY_STAGE_LDS)
             return launch_skinny_as<MT, GATED, 4, true, EPI>(a, w, out, M, N, K, out_float, lds, epi, stream);
     }
