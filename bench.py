@@ -243,12 +243,18 @@ class Bench:
             engine.run_until_done()
             torch.cuda.synchronize()
             return time.perf_counter() - t0
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        warmed = engine.warm_up() if a.warm_up else 0      # the decoding steps captured before the first request
+        torch.cuda.synchronize()
+        warm = time.perf_counter() - t0
         first = burst(requests)                 # a server's first minute: step shapes are met and captured
         before = dict(engine.stats)
         seconds = burst(requests)               # the same burst again: what a server that has run a while does
         return {"requests": requests, "slots": slots, "prompt_tokens": prompt, "output_tokens": output,
                 "seconds": round(seconds, 3), "generated_tok_s": round(requests * output / seconds, 1),
                 "total_tok_s": round(requests * (prompt + output) / seconds, 1), "first_burst_seconds": round(first, 3),
+                "warm_up_seconds": round(warm, 3), "warm_up_graphs": warmed,
                 "batches": engine.stats["batches"] - before["batches"],
                 "mixed_batches": engine.stats["mixed_batches"] - before["mixed_batches"]}
 
@@ -268,6 +274,8 @@ def main():
                     help="tuning aid: workgroups that the split of a token's keys aims for")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points, the prefill and the 8B block")
     ap.add_argument("--no-8b", action="store_true", help="skip the block of 8B measurements in the default run")
+    ap.add_argument("--warm-up", type=int, default=0,
+                    help="--only engine: 1 captures the decoding steps (Engine.warm_up) before the first burst")
     ap.add_argument("--only", default="all", choices=["all", "decode", "prefill", "engine", "mixed"],
                     help="profiling aid: run just the decode steps, just the prefill or just the mixed step; engine: the "
                          "scheduler over a burst of requests (3 x batch requests of 512 prompt and 128 output tokens, "

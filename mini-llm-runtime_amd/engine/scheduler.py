@@ -165,6 +165,13 @@ class Engine:
         self.stats = dict(batches=0, mixed_batches=0, prefill_tokens=0, decode_tokens=0, generated_tokens=0,
                           max_batch_tokens=0, max_batch_sequences=0, admission_waits=0, cancelled=0, timeouts=0)
 
+    def warm_up(self, batch_sizes=None, contexts=None):
+        """Captures the decoding steps ahead of the first requests (`Runner.warm_up`); to be called while the
+        engine is idle.  Returns the number of graphs captured."""
+        if self.active:
+            raise RuntimeError("warm_up: the engine has running requests")
+        return self.runner.warm_up(batch_sizes, contexts)
+
     # -- submit ----------------------------------------------------------------------------------
     def submit(self, prompt, max_tokens=64, temperature=0.0, seed=None, ignore_eos=False, priority=0,
                timeout_ms=None):

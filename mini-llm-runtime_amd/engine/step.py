@@ -289,6 +289,58 @@ class Runner:
         state["graph"], state["logits"] = graph, logits
         return logits
 
+    def warm_up(self, batch_sizes=None, contexts=None):
+        """Captures the decoding steps a server will meet before it meets them, so that no request waits for a
+        capture (about 20 ms a shape): for every number of single tokens that `_decode_fill` fills a batch up
+        to (at most `max_slots`, or those of `batch_sizes`) and every context bucket (512, 1024, ... up to
+        max_length, or those of `contexts`) whose requests fit the page pool, that many requests are opened at
+        a context of the bucket, stepped three times (eager, captured, replayed) and closed.  Their pages hold
+        zeros meanwhile and are filled with NaN again afterwards.  To be called while no request is open.
+        Returns the number of graphs captured."""
+        if not self.use_graphs or self.poisoned:
+            return 0
+        if self.free_slots() != self.cache.max_slots:
+            raise StepError("warm_up: close every request first")
+        limit = min(self.cache.max_slots, self.graph_max_batch)
+        if batch_sizes is None:
+            batch_sizes = [n for n in range(1, limit + 1)
+                           if n % (1 if n <= 8 else 2 if n <= 16 else 4 if n <= 64 else 8) == 0]
+        if contexts is None:
+            contexts, bucket = [], 512
+            while True:
+                contexts.append(min(bucket, self.max_length))
+                if bucket >= self.max_length:
+                    break
+                bucket *= 2
+        tensors = [t for t in self.cache.paged_tensors() if t.dtype.is_floating_point]
+        for t in tensors:
+            t.zero_()
+        before = sum(1 for st in self._graphs.values() if st["graph"] is not None)
+        try:
+            for context in contexts:
+                bucket = self._context_bucket(context)
+                start = max(1, min(bucket // 2 + 1, bucket - 4)) if bucket > 512 else 1
+                for n in sorted(set(int(b) for b in batch_sizes if 1 <= b <= limit), reverse=True):
+                    key = (((1, (0,)),) * n, bucket)
+                    if key in self._graphs and self._graphs[key]["graph"] is not None:
+                        continue
+                    if any(n * -(-(start + 4) // size) > pages for size, pages in zip(self.cache.group_page_size,
+                                                                                         self.cache.group_pages)):
+                        continue                          # that many requests of that length do not fit the pool
+                    slots = [self.open_request() for _ in range(n)]
+                    try:
+                        if start > 1:
+                            self.cache.commit(slots, [start - 1] * n)      # (their keys and values: the zeros)
+                        for _ in range(3):
+                            self.step([Entry(slot, [0], [0]) for slot in slots])
+                    finally:
+                        for slot in slots:
+                            self.close_request(slot)
+        finally:
+            for t in tensors:
+                t.fill_(float("nan"))
+        return sum(1 for st in self._graphs.values() if st["graph"] is not None) - before
+
     # -- the step ------------------------------------------------------------------------------
     def _validate(self, entries):
         if self.poisoned:

@@ -244,3 +244,33 @@ def test_command_line_through_the_scheduler(model_folders, plain_models, tmp_pat
                         "exceed")]:
         bad = run_cli(args)
         assert bad.returncode == 1 and text in bad.stderr, (args, bad.stderr)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_warm_up_captures_the_decoding_steps_ahead_of_the_requests(model_folders, plain_models, dtype):
+    """`Engine.warm_up`: the decoding steps of every batch size (and of the context buckets that fit) are
+    captured while the engine is idle; the requests that follow find their graphs, meet no capture, read no
+    leftover of the warm-up (the pages are NaN again) and get the plain greedy tokens."""
+    import torch
+    from mini_llm_runtime_amd.api import parse_dtype
+    from mini_llm_runtime_amd.engine import Engine, EngineOptions
+    from mini_llm_runtime_amd.parts import DecoderModel
+    model = DecoderModel.load(model_folders["A"], parse_dtype(dtype), "cuda:0")
+    eng = Engine(model, EngineOptions(context_tokens=4096, max_model_len=1024, max_active=6, batch_tokens=64,
+                                      prefill_chunk=32, block_size=PAGE_SIZE["A"]))
+    captured = eng.warm_up()
+    runner = eng.runner
+    one = (1, (0,))
+    assert captured == 12 and all(runner._graphs[((one,) * n, b)]["graph"] is not None
+                                  for n in range(1, 7) for b in (512, 1024))
+    assert runner.graph_failures == 0 and runner.free_slots() == 6 and runner.cache.free_pages() == runner.cache.num_pages
+    assert all(bool(torch.isnan(t).all()) for t in runner.cache.paged_tensors())
+    assert eng.warm_up() == 0                                       # nothing left to capture
+    prompts = prompts_for("A", (7, 13, 5, 1, 30, 9))
+    ids = [eng.submit(p, max_tokens=12, ignore_eos=True) for p in prompts]
+    eng.run_until_done()
+    for rid, prompt in zip(ids, prompts):
+        check_greedy(plain_models["A"], prompt, eng.finished[rid].generated, dtype)
+    decode_graphs = [key for key, st in runner._graphs.items() if all(e == one for e in key[0]) and st["graph"] is not None]
+    assert len(decode_graphs) == 12 and runner.graph_failures == 0
+    assert runner.cache.free_pages() == runner.cache.num_pages
