@@ -295,8 +295,9 @@ class Runner:
         to (at most `max_slots`, or those of `batch_sizes`) and every context bucket (512, 1024, ... up to
         max_length, or those of `contexts`) whose requests fit the page pool, that many requests are opened at
         a context of the bucket, stepped three times (eager, captured, replayed) and closed.  Their pages hold
-        zeros meanwhile and are filled with NaN again afterwards.  To be called while no request is open.
-        Returns the number of graphs captured."""
+        zeros meanwhile and are filled with NaN again afterwards.  Short contexts come first, and it stops when
+        the runner holds `max_graphs` shapes (one more would push the oldest out again).  To be called while no
+        request is open.  Returns the number of graphs captured."""
         if not self.use_graphs or self.poisoned:
             return 0
         if self.free_slots() != self.cache.max_slots:
@@ -324,6 +325,8 @@ class Runner:
                     key = (((1, (0,)),) * n, bucket)
                     if key in self._graphs and self._graphs[key]["graph"] is not None:
                         continue
+                    if key not in self._graphs and len(self._graphs) >= self.max_graphs:
+                        break
                     if any(n * -(-(start + 4) // size) > pages for size, pages in zip(self.cache.group_page_size,
                                                                                          self.cache.group_pages)):
                         continue                          # that many requests of that length do not fit the pool

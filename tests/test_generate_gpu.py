@@ -247,6 +247,21 @@ def test_command_line_through_the_scheduler(model_folders, plain_models, tmp_pat
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_warm_up_stops_at_the_number_of_graphs_the_runner_keeps(model_folders, dtype):
+    """A runner that keeps three captured shapes: the warm-up captures three (the shortest contexts' first)
+    and stops, instead of pushing out what it has just captured."""
+    from mini_llm_runtime_amd.api import parse_dtype
+    from mini_llm_runtime_amd.engine import Runner
+    from mini_llm_runtime_amd.parts import DecoderModel
+    model = DecoderModel.load(model_folders["A"], parse_dtype(dtype), "cuda:0")
+    r = Runner(model, max_tokens=4096, max_slots=4, max_length=1024, page_size=PAGE_SIZE["A"], max_graphs=3)
+    assert r.warm_up() == 3 and len(r._graphs) == 3
+    assert all(st["graph"] is not None and key[1] == 512 for key, st in r._graphs.items())
+    assert r.warm_up() == 0 and r.graph_failures == 0
+    assert r.free_slots() == 4 and r.cache.free_pages() == r.cache.num_pages
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_warm_up_captures_the_decoding_steps_ahead_of_the_requests(model_folders, plain_models, dtype):
     """`Engine.warm_up`: the decoding steps of every batch size (and of the context buckets that fit) are
     captured while the engine is idle; the requests that follow find their graphs, meet no capture, read no
