@@ -3,6 +3,7 @@
     llm = LLM("path/to/folder", dtype="bfloat16")
     tokens = llm.generate([1, 2, 3], max_tokens=16)                     # one prompt -> one list
     many = llm.generate([[1, 2, 3], [4, 5]], max_tokens=8, temperature=0.8, seed=7)
+    text = llm.generate("The capital of France is", max_tokens=16)      # needs tokenizer.json in the folder
 
 Generation goes through the scheduler (continuous batching over the step function); `runner`
 gives direct access to the step function for tests and tools.
@@ -33,6 +34,8 @@ class LLM:
         fields of EngineOptions (context_tokens, max_model_len, max_active, batch_tokens,
         prefill_chunk, block_size, policy, ...)."""
         self.dtype = parse_dtype(dtype)
+        self.folder = model
+        self._tokenizer = None
         self.model = DecoderModel.load(model, self.dtype, device)
         opts = options or EngineOptions()
         for key, value in overrides.items():
@@ -46,10 +49,27 @@ class LLM:
     def runner(self):
         return self.engine.runner
 
+    @property
+    def tokenizer(self):
+        """The vocabulary of the model folder's tokenizer.json (read when text is first asked for)."""
+        if self._tokenizer is None:
+            from .tokenizer import Tokenizer
+            self._tokenizer = Tokenizer(self.folder, self.model.spec.vocab_size, self.model.spec.eos_token_ids)
+        return self._tokenizer
+
     def generate(self, prompts, max_tokens=32, temperature=0.0, seed=None, ignore_eos=False, timeout_ms=None):
-        """`prompts`: one list of token ids or a list of such lists.  Returns the generated ids
-        (without the prompt), in the same shape.  A request that runs out of `timeout_ms` returns what it
-        has generated until then."""
+        """`prompts`: one list of token ids or a list of such lists; or one text or a list of texts (the
+        model folder must hold a tokenizer.json then).  Returns the generated ids (without the prompt), in
+        the same shape; for text, the generated text (the token that ended it left out).  A request that
+        runs out of `timeout_ms` returns what it has generated until then."""
+        as_text = isinstance(prompts, str) or (len(prompts) > 0 and all(isinstance(p, str) for p in prompts))
+        if as_text:
+            one = isinstance(prompts, str)
+            ids = self.generate([self.tokenizer.tokenize(p) for p in ([prompts] if one else prompts)], max_tokens,
+                                temperature, seed, ignore_eos, timeout_ms)
+            eos = set() if ignore_eos else set(self.model.spec.eos_token_ids)
+            texts = [self.tokenizer.text([t for t in row if t not in eos]) for row in ids]
+            return texts[0] if one else texts
         single = len(prompts) > 0 and not isinstance(prompts[0], (list, tuple))
         batch = [prompts] if single else list(prompts)
         ids = []

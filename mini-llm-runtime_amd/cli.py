@@ -1,13 +1,14 @@
 """`mini-llm`: generate from token ids on one MI355X.  Options keep the names and meanings of the
-reference's CLIs (apps/mini_main.cpp:19-83, apps/cuda_main.cpp:18-54) where it has them.  There is no
-tokenizer here: prompts are given as ids.
+reference's CLIs (apps/mini_main.cpp:19-83, apps/cuda_main.cpp:18-54) where it has them.  Prompts are
+token ids, or text when the model folder (or --tokenizer) holds a tokenizer.json.
 
 Two ways to run:
 
-  * `--prompt-ids 1,2,3`: one sequence straight on the step function, as the reference's CLIs run theirs:
-    the prompt in portions of --chunk tokens with logits asked for at its last token only, then one token
-    per step; the last generated token is never fed back, so the cache must hold prompt + tokens - 1
-    positions.
+  * `--prompt-ids 1,2,3` or `--prompt TEXT`: one sequence straight on the step function, as the reference's
+    CLIs run theirs: the prompt in portions of --chunk tokens with logits asked for at its last token only,
+    then one token per step; the last generated token is never fed back, so the cache must hold prompt +
+    tokens - 1 positions.  With a tokenizer the report holds the generated `text` as well, and without any
+    prompt option the reference's default prompt is taken ("The capital of France is").
   * `--prompts-file FILE` (one comma-separated prompt a line): every prompt becomes a request of the
     scheduler (`Engine`): admission, portions under the token budget, continuous batching over
     --sequences slots, --policy mixed or prefill_first.
@@ -22,7 +23,8 @@ import time
 
 from .options import Option, OptionError, parse
 
-USAGE = """mini-llm (--model DIR | --random-weights CONFIG.json [--seed 0]) (--prompt-ids 1,2,3 | --prompts-file FILE)
+USAGE = """mini-llm (--model DIR | --random-weights CONFIG.json [--seed 0])
+         (--prompt-ids 1,2,3 | --prompt TEXT | --prompts-file FILE) [--tokenizer tokenizer.json|DIR]
          [--tokens 32] [--context 2048] [--batch 128] [--chunk 128] [--sequences 4]
          [--dtype bfloat16|float32] [--temperature 0] [--sample-seed 0] [--page-size 16]
          [--policy mixed|prefill_first] [--device 0] [--device-budget-bytes 0] [--ignore-eos]
@@ -35,6 +37,7 @@ TABLE = [
     Option("--help", "switch"), Option("--inspect", "switch"), Option("--ignore-eos", "switch"),
     Option("--device-time", "switch"), Option("--profile", "switch"), Option("--check-finite", "switch"),
     Option("--model"), Option("--random-weights"), Option("--output"), Option("--prompts-file"),
+    Option("--prompt"), Option("--tokenizer"),
     Option("--dtype", default="bfloat16"), Option("--policy", default="mixed"),
     Option("--cuda-precision"), Option("--kv-layout", default="paged"),
     Option("--prompt-ids", "ints", default=[]),
@@ -95,7 +98,10 @@ def read_prompts(path, vocab):
     return prompts
 
 
-def one_sequence(opts, model, runner, sampler, prompt, count, chunk):
+DEFAULT_PROMPT = "The capital of France is"        # apps/cuda_main.cpp:53, apps/mini_main.cpp:85
+
+
+def one_sequence(opts, model, runner, sampler, prompt, count, chunk, tokenizer=None):
     """The reference CLI's loop (apps/cuda_main.cpp:91-119): portions, then one token per step."""
     import torch
     from .engine import Entry
@@ -144,7 +150,9 @@ def one_sequence(opts, model, runner, sampler, prompt, count, chunk):
     elapsed = time.perf_counter() - started
     pages_before = runner.cache.num_pages - runner.cache.free_pages()
     runner.close_request(slot)
-    return {"input_token_ids": prompt, "token_ids": generated, "prompt_tokens": len(prompt),
+    text = {} if tokenizer is None else \
+        {"text": tokenizer.text([t for t in generated if opts["--ignore-eos"] or t not in eos])}
+    return {"input_token_ids": prompt, "token_ids": generated, **text, "prompt_tokens": len(prompt),
             "completion_tokens": len(generated), "ttft_ms": prefill_s * 1e3, "elapsed_s": elapsed,
             "output_tokens_per_second": len(generated) / elapsed if elapsed > 0 else None,
             "used_kv_pages_before_release": pages_before,
@@ -152,7 +160,7 @@ def one_sequence(opts, model, runner, sampler, prompt, count, chunk):
             "forwards": forwards}
 
 
-def many_requests(opts, engine, prompts, count):
+def many_requests(opts, engine, prompts, count, tokenizer=None):
     """Every prompt a request of the scheduler; the report lists them in the order of the file."""
     started = time.perf_counter()
     ids = [engine.submit(p, max_tokens=count, temperature=opts["--temperature"], seed=opts["--sample-seed"] + i,
@@ -166,6 +174,9 @@ def many_requests(opts, engine, prompts, count):
     requests = [{"input_token_ids": p, "token_ids": list(engine.finished[rid].generated),
                  "finish_reason": engine.finished[rid].finish_reason, "ttft_ms": first.get(rid, 0.0) * 1e3}
                 for rid, p in zip(ids, prompts)]
+    if tokenizer is not None:
+        for r in requests:
+            r["text"] = tokenizer.text(r["token_ids"])
     generated = sum(len(r["token_ids"]) for r in requests)
     return {"requests": requests, "prompt_tokens": sum(len(p) for p in prompts), "completion_tokens": generated,
             "elapsed_s": elapsed, "output_tokens_per_second": generated / elapsed if elapsed > 0 else None,
@@ -187,8 +198,17 @@ def main(argv=None):
         output = opts["--output"]
         if opts.given("--output") and (not output or os.path.exists(output)):
             raise OptionError("--output must be a new file")
-        if opts.given("--prompt-ids") == opts.given("--prompts-file"):
-            raise OptionError("give --prompt-ids or --prompts-file (one of them)")
+        ways = [name for name in ("--prompt-ids", "--prompt", "--prompts-file") if opts.given(name)]
+        if len(ways) > 1:
+            raise OptionError(f"give --prompt-ids, --prompt or --prompts-file (one of them), not {' and '.join(ways)}")
+        if not ways or ways == ["--prompt"] or opts.given("--tokenizer"):
+            # text needs a vocabulary: looked for now, before the weights are read
+            from .tokenizer import tokenizer_file
+            where = opts["--tokenizer"] if opts.given("--tokenizer") else opts["--model"]
+            if not where or tokenizer_file(where) is None:
+                raise OptionError("no tokenizer.json in the model folder or under --tokenizer: give --prompt-ids "
+                                  "or --prompts-file" if not opts.given("--tokenizer") else
+                                  f"--tokenizer {where}: no tokenizer.json there")
         context, batch, sequences = opts["--context"], opts["--batch"], opts["--sequences"]
         chunk = opts["--chunk"] if opts.given("--chunk") else batch
         if chunk > batch:
@@ -228,6 +248,14 @@ def main(argv=None):
         except MemoryBudgetError as error:
             raise OptionError(str(error)) from None
         vocab = model.spec.vocab_size
+        tokenizer = None
+        if opts.given("--tokenizer") or not (opts.given("--prompt-ids") or opts.given("--prompts-file")):
+            from .tokenizer import Tokenizer, TokenizerError
+            try:
+                tokenizer = Tokenizer(opts["--tokenizer"] if opts.given("--tokenizer") else folder, vocab,
+                                      model.spec.eos_token_ids)
+            except TokenizerError as error:
+                raise OptionError(str(error)) from None
         limit = min(context, model.spec.max_positions)
         pool = sequences * ((limit + page - 1) // page) * page
         common = {"backend": "mini-llm-runtime_amd", "dtype": str(dtype).replace("torch.", "")}
@@ -242,18 +270,23 @@ def main(argv=None):
                     prefill_chunk=min(chunk, max(batch, sequences)), block_size=page, policy=opts["--policy"]),
                     device_budget_bytes=budget, check_finite=opts["--check-finite"], profile=opts["--profile"])
                 runner = engine.runner
-                report = many_requests(opts, engine, prompts, count)
+                report = many_requests(opts, engine, prompts, count, tokenizer)
             else:
-                prompt = opts["--prompt-ids"]
-                if not prompt or any(t < 0 or t >= vocab for t in prompt):
-                    raise OptionError("--prompt-ids must name at least one token id inside the vocabulary")
+                if opts.given("--prompt-ids"):
+                    prompt = opts["--prompt-ids"]
+                    if not prompt or any(t < 0 or t >= vocab for t in prompt):
+                        raise OptionError("--prompt-ids must name at least one token id inside the vocabulary")
+                else:
+                    prompt = tokenizer.tokenize(opts["--prompt"] if opts.given("--prompt") else DEFAULT_PROMPT)
+                    if not prompt:
+                        raise OptionError("--prompt: the text gives no token")
                 if len(prompt) > limit or count - 1 > limit - len(prompt):
                     raise OptionError("prompt and the output tokens written to the cache exceed the context")
                 runner = Runner(model, max_tokens=pool, max_slots=sequences, max_length=limit, max_batch_tokens=batch,
                                 page_size=page, device_budget_bytes=budget, check_finite=opts["--check-finite"],
                                 profile=opts["--profile"])
                 sampler = Sampler(runner.kernels, runner.device, max_rows=1)
-                report = one_sequence(opts, model, runner, sampler, prompt, count, chunk)
+                report = one_sequence(opts, model, runner, sampler, prompt, count, chunk, tokenizer)
         except MemoryBudgetError as error:
             raise OptionError(str(error)) from None
         report = {**common, **report,

@@ -289,3 +289,37 @@ def test_warm_up_captures_the_decoding_steps_ahead_of_the_requests(model_folders
     decode_graphs = [key for key, st in runner._graphs.items() if all(e == one for e in key[0]) and st["graph"] is not None]
     assert len(decode_graphs) == 12 and runner.graph_failures == 0
     assert runner.cache.free_pages() == runner.cache.num_pages
+
+
+def test_text_prompts_through_the_command_line_and_the_entry_point(model_folders, plain_models, tmp_path):
+    """A model folder that holds a tokenizer.json: --prompt TEXT (and no prompt option at all: the reference's
+    default prompt, apps/cuda_main.cpp:53) runs the same tokens as --prompt-ids, the report holds the generated
+    text, and `LLM.generate` takes and returns text."""
+    import shutil
+    pytest.importorskip("tokenizers")
+    from test_tokenizer import WORDS, write_tokenizer
+    from mini_llm_runtime_amd.api import LLM
+    folder = str(tmp_path / "model")
+    shutil.copytree(model_folders["A"], folder)
+    write_tokenizer(os.path.join(folder, "tokenizer.json"))
+    prompt = [2, 3, 4, 5, 6]                                           # "The capital of France is"
+    expect = plain_models["A"].greedy(prompt, 6)
+    common = ["--tokens", "6", "--dtype", "float32", "--context", "64", "--sequences", "1", "--ignore-eos"]
+    by_ids = run_cli(["--model", folder, "--prompt-ids", "2,3,4,5,6"] + common)
+    by_text = run_cli(["--model", folder, "--prompt", "The capital of France is"] + common)
+    by_default = run_cli(["--model", folder] + common)
+    elsewhere = run_cli(["--model", model_folders["A"], "--tokenizer", os.path.join(folder, "tokenizer.json"),
+                         "--prompt", "the capital of france is"] + common)
+    for done in (by_ids, by_text, by_default, elsewhere):
+        assert done.returncode == 0, done.stderr
+    reports = [json.loads(done.stdout) for done in (by_ids, by_text, by_default, elsewhere)]
+    assert all(r["input_token_ids"] == prompt and r["token_ids"] == expect for r in reports)
+    assert "text" not in reports[0]
+    words = lambda ids: " ".join(WORDS[t] for t in ids if t < len(WORDS) and WORDS[t] != "<eos>")
+    assert all(r["text"] == words(expect) for r in reports[1:])
+    llm = LLM(folder, dtype="float32", context_tokens=256, max_model_len=64, max_active=2, block_size=PAGE_SIZE["A"])
+    assert llm.generate("The capital of France is", max_tokens=6, ignore_eos=True) == words(expect)
+    both = llm.generate(["the capital", "paris is a city"], max_tokens=4, ignore_eos=True)
+    assert both == [words(plain_models["A"].greedy([2, 3], 4)), words(plain_models["A"].greedy([7, 6, 8, 9], 4))]
+    bad = run_cli(["--model", folder, "--prompt", ""] + common)
+    assert bad.returncode == 1 and "no token" in bad.stderr
