@@ -84,7 +84,8 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(AttnArgs a) {
             const int kp = t0 + threadIdx.x;
             long long off = -1, voff = -1;
             if (kp >= kbegin && kp < kend) {
-                const int page = table[kp / a.page_size];
+                const int block = kp / a.page_size;
+                const int page = block < a.max_blocks ? table[block] : -1;     // (beyond the table's row: no page)
                 if (page >= 0) {
                     off = (((long long)page * a.kv_heads + kvh) * a.page_size + kp % a.page_size) * D;
                     voff = ((long long)page * a.kv_heads + kvh) * D * a.page_size + kp % a.page_size;
@@ -361,7 +362,9 @@ __global__ __launch_bounds__(256, (NCH <= 4 ? 2 : 1)) void attention_mfma_kernel
     const int first_page = t_begin * MFMA_TILE_KEYS / P;
     {
         const int n_pages = min(DECODE_PAGE_CACHE, (hi + P - 1) / P - first_page);
-        for (int i = threadIdx.x; i < n_pages; i += 256) page_lds[i] = table[first_page + i];
+        // (an entry beyond the request's row of the table is no page, like an entry of -1)
+        for (int i = threadIdx.x; i < n_pages; i += 256)
+            page_lds[i] = first_page + i < a.max_blocks ? table[first_page + i] : -1;
     }
 
     // The queries.  FUSED: the raw query of this lane's column, its norm weights and its rotation row are
@@ -697,7 +700,8 @@ __device__ __forceinline__ void prefill_group(const AttnArgs& a, const int32_t* 
     const int first_page = (lo / MFMA_TILE_KEYS) * MFMA_TILE_KEYS / P;
     {
         const int n_pages = min(PAGE_CACHE, (ke + P - 1) / P - first_page);
-        for (int i = threadIdx.x; i < n_pages; i += 256) page_lds[i] = table[first_page + i];
+        for (int i = threadIdx.x; i < n_pages; i += 256)
+            page_lds[i] = first_page + i < a.max_blocks ? table[first_page + i] : -1;
         __syncthreads();
     }
     const int kchunks = 4 * D;                         // 32 keys x D / 8 chunks of 16 bytes; as many for V
@@ -996,7 +1000,8 @@ __global__ __launch_bounds__(64) void attention_combine_fused_kernel(AttnArgs a,
         co[i] = cs[j];
         si[i] = cs[rotated ? j + half : 0];
     }
-    const int page = a.block_table[(size_t)slot * a.max_blocks + pos / P];
+    const int page_read = a.block_table[(size_t)slot * a.max_blocks + min(pos / P, a.max_blocks - 1)];
+    const int page = pos / P < a.max_blocks ? page_read : -1;    // (beyond the request's row of the table: no page)
     const int glo = a.window > 0 ? max(0, pos + 1 - a.window) : 0;
     const int first = a.max_splits > 1 ? glo / a.split_keys : 0;
     const int last = a.max_splits > 1 ? min(a.max_splits - 1, max(pos - 1, 0) / a.split_keys) : 0;

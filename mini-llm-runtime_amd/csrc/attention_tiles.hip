@@ -156,10 +156,17 @@ __device__ __forceinline__ void tile_group(const TileArgs& a, int grp, int kvh, 
     const int blk_begin = lo_s / BLOCK_KEYS, blk_end = (ke_s + BLOCK_KEYS - 1) / BLOCK_KEYS;
     const int first_page = (blk_begin * BLOCK_KEYS) >> pshift;
     const int32_t* table = a.block_table + (size_t)slot * a.max_blocks;
+    bool all_mapped;                                  // every page of the key range is there (none given back, none missing)
     {
         const int n_pages = min(PAGE_IDS, ((ke_s + P - 1) >> pshift) - first_page);
-        for (int i = threadIdx.x; i < n_pages; i += THREADS) page_lds[i] = table[first_page + i];
-        __syncthreads();
+        // (an entry beyond the request's row of the table is no page, like an entry of -1)
+        int mine_mapped = 1;
+        for (int i = threadIdx.x; i < n_pages; i += THREADS) {
+            const int id = first_page + i < a.max_blocks ? table[first_page + i] : -1;
+            page_lds[i] = id;
+            mine_mapped &= id >= 0 ? 1 : 0;
+        }
+        all_mapped = __syncthreads_and(mine_mapped) != 0;
     }
 
     // What a thread stages per block and pass: 32 bytes of the keys (16 channels of one key) and 32 bytes of
@@ -202,7 +209,7 @@ __device__ __forceinline__ void tile_group(const TileArgs& a, int grp, int kvh, 
         const int pidx = (tb >> pshift) - first_page;
         const uint32_t inpage = big_page ? (tb & (P - 1)) : 0;
         // (all blocks but a group's last, unless a window has given pages back: the same for every thread)
-        st.whole = a.window <= 0 && tb + BLOCK_KEYS <= ke;
+        st.whole = all_mapped && a.window <= 0 && tb + BLOCK_KEYS <= ke;
         if (st.whole) {
 #pragma unroll
             for (int i = 0; i < KN; ++i) {

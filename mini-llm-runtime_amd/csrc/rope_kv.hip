@@ -51,7 +51,9 @@ __global__ void qk_norm_rope_kv_kernel(
     size_t cache_row = 0, cache_page = 0;
     bool cache_ok = false;
     if (write_cache) {
-        const int page = block_table[(size_t)slot * max_blocks + pos / page_size];
+        // (a position beyond the request's row of the table has no page, like an entry of -1)
+        const int block = pos / page_size;
+        const int page = block < max_blocks ? block_table[(size_t)slot * max_blocks + block] : -1;
         cache_ok = page >= 0;
         cache_page = (size_t)(page < 0 ? 0 : page) * kv_heads;
         cache_row = cache_page * page_size + (pos % page_size);
@@ -160,7 +162,8 @@ __device__ __forceinline__ void write_values_transposed(
         int in_page = 0;
         if (r < rows) {
             const int pos = positions[r];
-            const int page = block_table[(size_t)slots[r] * max_blocks + pos / page_size];
+            const int block = pos / page_size;
+            const int page = block < max_blocks ? block_table[(size_t)slots[r] * max_blocks + block] : -1;
             if (page >= 0) base = ((long long)page * kv_heads + kvh) * head_dim * page_size;
             in_page = pos % page_size;
         }
@@ -232,7 +235,9 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kv_vec_kernel(
     }
     // what needs the position: the page (entry 0 of the request's row when nothing is written) and the
     // rotation row
-    const int page = block_table[(size_t)slot * max_blocks + (write_cache ? pos / page_size : 0)];
+    const int block = write_cache ? pos / page_size : 0;       // (beyond the request's row of the table: no page)
+    const int page_read = block_table[(size_t)slot * max_blocks + min(block, max_blocks - 1)];
+    const int page = block < max_blocks ? page_read : -1;
     float co[8], si[8];
     if (HAS_ROPE) {
         const float* cs = rope + (size_t)pos * head_dim;

@@ -1014,3 +1014,36 @@ def test_bfloat16_widening_and_rounding():
             out = torch.empty((rows, 8), dtype=torch.bfloat16, device="cuda")
             engine.gemm(a[:rows].to(torch.bfloat16).cuda(), w, out)
             assert torch.equal(out.float().cpu(), want[:rows, None].expand(rows, 8)), rows
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows", [3, 96])
+def test_a_position_beyond_the_block_table_has_no_page(dtype, rows):
+    """The engine never asks for it (the cache manager bounds a request's length by its row of the table); a
+    caller of the kernels that does gets what a missing page gives: the query is normed and rotated, nothing
+    is cached, and no kernel reads past the table's row.  Few rows (the general kernel) and many (the vector
+    kernel and its transposing value writer)."""
+    hq, hkv, d, page, max_blocks = 4, 2, 64, 16, 2
+    k = kernels(dtype)
+    inside = max_blocks * page                                         # 32 positions have a page
+    positions = torch.tensor([30 + 3 * (i // 2) for i in range(rows)], dtype=torch.int32)      # 30, 30, 33, 33, ...
+    slots = torch.tensor([i % 2 for i in range(rows)], dtype=torch.int32)
+    seen = {(int(slots[i]), int(positions[i])): i for i in range(rows)}         # (every position of a slot once)
+    assert len(seen) == rows
+    table = torch.tensor([[3, 0], [1, 2]], dtype=torch.int32)
+    qkv = rnd((rows, (hq + 2 * hkv) * d), dtype, 70)
+    qw, kw = rnd((d,), torch.float32, 71) + 1, rnd((d,), torch.float32, 72) + 1
+    rope = rope_table(256, d, 10000.0)
+    k_pages = torch.full((4, hkv, page, d), float("nan"), dtype=dtype, device="cuda")
+    v_pages = torch.full((4, hkv, d, page), float("nan"), dtype=dtype, device="cuda")
+    q_out = torch.full((rows, hq * d), float("nan"), dtype=dtype, device="cuda")
+    k.qk_norm_rope_kv(qkv, q_out, k_pages, v_pages, table.cuda(), slots.cuda(), positions.cuda(), qw, kw, 1e-6, rope,
+                      hq, hkv, d, page)
+    assert bool(torch.isfinite(q_out.float()).all())
+    cached = sum(1 for (s, p) in seen if p < inside)
+    kp, vp = k_pages.cpu().float(), v_pages.cpu().float()
+    assert int((~torch.isnan(kp)).sum()) == cached * hkv * d and int((~torch.isnan(vp)).sum()) == cached * hkv * d
+    for (s, p), i in seen.items():
+        if p < inside:
+            assert torch.equal(v_pages[int(table[s, p // page]), :, :, p % page].cpu(),
+                               qkv[i, (hq + hkv) * d:].view(hkv, d).cpu())
