@@ -135,7 +135,7 @@ __global__ __launch_bounds__(THREADS) void pick_kernel(const float* __restrict__
                                                        int32_t* __restrict__ tokens) {
     __shared__ float scan[CHUNKS];
     __shared__ float vals[THREADS];
-    __shared__ int chosen_chunk, chosen;
+    __shared__ int chosen_chunk, chosen, last_thread;
     __shared__ float chunk_lo;
     const int r = blockIdx.x, t = threadIdx.x;
     const float temp = temperature[r];
@@ -144,15 +144,21 @@ __global__ __launch_bounds__(THREADS) void pick_kernel(const float* __restrict__
         float c = 0.f;
         for (int i = 0; i < CHUNKS; ++i) { c += csum[r * CHUNKS + i]; scan[i] = c; }
         const float target = uniform[r] * c;
-        int pick = -1;
-        for (int i = 0; i < CHUNKS; ++i)
-            if (target < scan[i] && csum[r * CHUNKS + i] > 0.f) { pick = i; break; }
+        // the first chunk whose running sum passes the target; when rounding has pushed the target to the
+        // total itself (u within 2^-23 of 1), the last chunk that holds any probability
+        int pick = -1, last = -1;
+        for (int i = 0; i < CHUNKS; ++i) {
+            if (!(csum[r * CHUNKS + i] > 0.f)) continue;
+            last = i;
+            if (target < scan[i]) { pick = i; break; }
+        }
+        if (pick < 0) pick = last;
         chosen_chunk = pick;
         chunk_lo = pick > 0 ? scan[pick - 1] : 0.f;
         chosen = -1;
     }
     __syncthreads();
-    if (chosen_chunk < 0) return;                   // rounding pushed the target past the end: keep the argmax
+    if (chosen_chunk < 0) return;                   // (no chunk holds any probability: cannot happen; the argmax stays)
     const float target = uniform[r] * scan[CHUNKS - 1];
     const float* row = logits + (size_t)r * vocab;
     int cb, ce;
@@ -166,18 +172,31 @@ __global__ __launch_bounds__(THREADS) void pick_kernel(const float* __restrict__
     __syncthreads();
     if (t == 0) {
         float c = chunk_lo;
-        for (int i = 0; i < THREADS; ++i) { c += vals[i]; vals[i] = c; }
+        int last = -1;                              // the last thread whose tokens hold any probability
+        for (int i = 0; i < THREADS; ++i) {
+            if (vals[i] > 0.f) last = i;
+            c += vals[i];
+            vals[i] = c;
+        }
+        last_thread = last;
     }
     __syncthreads();
     const float lo = t ? vals[t - 1] : chunk_lo, hi = vals[t];
-    if (target >= lo && target < hi && end > begin) {
+    // The thread whose stretch of the running sum holds the target.  The sums within the chunk are added in
+    // another order than the chunk's own sum was, so the target may come to lie at or past their end by a
+    // rounding: then the last thread that holds any probability takes it, and gives its last such token.
+    const bool mine = target >= lo && target < hi && end > begin;
+    const bool past_the_end = t == last_thread && target >= vals[THREADS - 1];
+    if (mine || past_the_end) {
         float c = lo;
-        int pick = end - 1;
+        int pick = -1, last = end - 1;
         for (int i = begin; i < end; ++i) {
-            c += expf((row[i] - row_max) * inv_t);
+            const float e = expf((row[i] - row_max) * inv_t);
+            if (e > 0.f) last = i;
+            c += e;
             if (c > target) { pick = i; break; }
         }
-        chosen = pick;
+        chosen = pick >= 0 ? pick : last;
     }
     __syncthreads();
     if (t == 0 && chosen >= 0) tokens[r] = chosen;

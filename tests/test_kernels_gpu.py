@@ -590,9 +590,11 @@ def test_sample_greedy(vocab):
         assert got[1] == vocab // 2 and got[2] == 0
 
 
-@pytest.mark.parametrize("vocab", [5, 311, 4099, 151936])
+@pytest.mark.parametrize("vocab", [5, 311, 4099, 151936, 1859, 2680, 2769, 146254, 236821])
 def test_sample_temperature(vocab):
-    """The drawn token's slice of the CDF of softmax(logits / T) (float64) holds u."""
+    """The drawn token's slice of the CDF of softmax(logits / T) (float64) holds u.  Row 1 draws u = 1 - 2^-23:
+    in 32-bit its target is the total itself or a rounding below it, and the token must still come from the
+    CDF's end (the last five sizes are ones at which the running sums, added in another order, end below it)."""
     from plain.qwen3_plain import temperature_cdf
     k = kernels(torch.float32)
     g = torch.Generator().manual_seed(vocab + 1)
