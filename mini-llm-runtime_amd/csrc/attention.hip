@@ -432,8 +432,8 @@ __global__ __launch_bounds__(256, (NCH <= 4 ? 2 : 1)) void attention_mfma_kernel
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
                     const float lo_v = x[c][e], hi_v = x[c + HC][e];
-                    x[c][e] = lo_v * co[e] - hi_v * si[e];
-                    x[c + HC][e] = lo_v * si[e] + hi_v * co[e];
+                    x[c][e] = turn_x(lo_v, hi_v, co[e], si[e]);
+                    x[c + HC][e] = turn_y(lo_v, hi_v, co[e], si[e]);
                 }
             }
         }
@@ -1024,8 +1024,8 @@ __global__ __launch_bounds__(64) void attention_combine_fused_kernel(AttnArgs a,
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
         if (lane + 64 * i >= half) qa[i] = qb[i] = ka[i] = kb[i] = 0.f;
-        qsum += qa[i] * qa[i] + qb[i] * qb[i];
-        ksum += ka[i] * ka[i] + kb[i] * kb[i];
+        qsum += squares(qa[i], qb[i]);
+        ksum += squares(ka[i], kb[i]);
     }
     if (normed) {
         qsum = wave_sum(qsum);
@@ -1045,10 +1045,10 @@ __global__ __launch_bounds__(64) void attention_combine_fused_kernel(AttnArgs a,
     for (int i = 0; i < 2; ++i) {
         float qx = qa[i], qy = qb[i], kx = ka[i], ky = kb[i];
         if (rotated) {
-            qx = qa[i] * co[i] - qb[i] * si[i];
-            qy = qa[i] * si[i] + qb[i] * co[i];
-            kx = ka[i] * co[i] - kb[i] * si[i];
-            ky = ka[i] * si[i] + kb[i] * co[i];
+            qx = turn_x(qa[i], qb[i], co[i], si[i]);
+            qy = turn_y(qa[i], qb[i], co[i], si[i]);
+            kx = turn_x(ka[i], kb[i], co[i], si[i]);
+            ky = turn_y(ka[i], kb[i], co[i], si[i]);
         }
         k_lo[i] = (__bf16)kx;
         k_hi[i] = (__bf16)ky;

@@ -49,6 +49,20 @@ __device__ __forceinline__ void store_vec(elem_t* p, const float* in) {
     *reinterpret_cast<vec16*>(p) = *reinterpret_cast<const vec16*>(tmp);
 }
 
+// The same bits whatever fused operations the compiler would choose: a token's key is written by one of three
+// kernels (the general and the vector kernel of rope_kv.hip, the decode merge of attention.hip) and should not
+// depend on which.  An empty asm makes an intermediate opaque, so that a product cannot be drawn into the
+// sum that follows it; the fused multiply-adds that are meant are written out.
+__device__ __forceinline__ float opaque(float v) {
+    asm("" : "+v"(v));
+    return v;
+}
+// (x, y) = (a, b) turned by the angle with cosine c and sine s
+__device__ __forceinline__ float turn_x(float a, float b, float c, float s) { return __builtin_fmaf(a, c, -opaque(b * s)); }
+__device__ __forceinline__ float turn_y(float a, float b, float c, float s) { return __builtin_fmaf(a, s, opaque(b * c)); }
+// a^2 + b^2, to be added to a running sum
+__device__ __forceinline__ float squares(float a, float b) { return opaque(__builtin_fmaf(a, a, opaque(b * b))); }
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, MLR_WAVE);

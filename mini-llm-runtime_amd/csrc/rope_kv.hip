@@ -84,7 +84,7 @@ __global__ void qk_norm_rope_kv_kernel(
                 pair_of(j, ia, ib, turned);
                 a[i] = to_float(src[ia]);
                 b[i] = to_float(src[ib]);
-                sum += a[i] * a[i] + b[i] * b[i];
+                sum += squares(a[i], b[i]);
             }
         }
         if (w) {
@@ -119,8 +119,8 @@ __global__ void qk_norm_rope_kv_kernel(
                 float x = a[i], y = b[i];
                 if (cs && turned) {
                     const float c = cs[j], s = cs[j + rot_half];
-                    x = a[i] * c - b[i] * s;
-                    y = a[i] * s + b[i] * c;
+                    x = turn_x(a[i], b[i], c, s);
+                    y = turn_y(a[i], b[i], c, s);
                 }
                 dst[ia] = from_float<elem_t>(x);
                 dst[ib] = from_float<elem_t>(y);
@@ -253,7 +253,7 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kv_vec_kernel(
     for (int e = 0; e < 8; ++e) {
         a[e] = (float)lo8[e];
         b[e] = (float)hi8[e];
-        sum += a[e] * a[e] + b[e] * b[e];
+        sum += squares(a[e], b[e]);
     }
     for (int off = 1; off < lph; off <<= 1) sum += __shfl_xor(sum, off, MLR_WAVE);
     if (!active) return;
@@ -281,8 +281,8 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kv_vec_kernel(
     if (HAS_ROPE) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-            const float x = a[e] * co[e] - b[e] * si[e];
-            const float y = a[e] * si[e] + b[e] * co[e];
+            const float x = turn_x(a[e], b[e], co[e], si[e]);
+            const float y = turn_y(a[e], b[e], co[e], si[e]);
             a[e] = x;
             b[e] = y;
         }

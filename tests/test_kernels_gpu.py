@@ -918,6 +918,11 @@ def test_prompt_portion_beyond_the_page_cache_of_a_workgroup():
     (6, 1, 192, 16, [1, 70], None, 0, False, True),
     (2, 1, 256, 16, [129, 1], 1, 64, True, False),
     (32, 8, 128, 64, [513, 512, 511], 512, 256, True, True),
+    # (heads above 128 channels, where a lane holds two rotation pairs: cases in which the two ways once differed
+    # in a key's last bit, the compiler having fused the products and sums of the two kernels differently)
+    (10, 5, 256, 32, [2078, 867, 853, 202], 441, 0, True, True),
+    (15, 3, 192, 128, [1, 246, 75, 83, 345, 236, 609], None, 64, True, True),
+    (64, 8, 256, 16, [2270, 123, 1915, 575, 687], None, 0, False, True),
 ])
 def test_decode_attention_that_norms_rotates_and_caches_itself(case):
     """Every request brings one new token.  The fused pair of launches against the separate ones (per-head
