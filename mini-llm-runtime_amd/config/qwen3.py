@@ -80,10 +80,25 @@ class Qwen3Config:
                                         scaling.get("rope_type", scaling.get("type")) in
                                         (None, "none", "default")):
             raise ConfigError("config.json: rope_scaling is not supported")
-        if data.get("attention_bias", False):
+        for key in ("attention_bias", "use_sliding_window"):
+            if data.get(key) is not None and not isinstance(data[key], bool):
+                raise ConfigError(f"config.json: `{key}` must be true or false")
+        if data.get("attention_bias"):
             raise ConfigError("config.json: attention_bias is not supported (Qwen3 dense has no biases)")
-        if data.get("use_sliding_window", False):
+        if data.get("use_sliding_window"):
             raise ConfigError("config.json: use_sliding_window is not supported (full causal attention)")
+        # (a list that names the kind of attention of every layer: anything but full attention everywhere would
+        # be computed wrongly here, so it is refused rather than passed over)
+        kinds = data.get("layer_types")
+        if kinds is not None:
+            layers = _integer(data, "num_hidden_layers")
+            if not isinstance(kinds, list) or len(kinds) != layers or any(not isinstance(k, str) for k in kinds):
+                raise ConfigError("config.json: `layer_types` must name the attention of each of the "
+                                  f"{layers} layers")
+            if any(k != "full_attention" for k in kinds):
+                raise ConfigError("config.json: layer_types other than full_attention are not supported")
+        if data.get("model_type") is not None and data["model_type"] != "qwen3":
+            raise ConfigError(f"config.json: model_type {data['model_type']!r} does not go with {cls.architecture}")
         act = data.get("hidden_act", "silu")
         if act != "silu":
             raise ConfigError(f"config.json: hidden_act {act!r} is not supported (silu)")

@@ -59,6 +59,9 @@ def test_head_dim_is_its_own_key():
     {"use_sliding_window": True}, {"attention_bias": True}, {"hidden_act": "gelu"},
     {"vocab_size": "many"}, {"tie_word_embeddings": "yes"}, {"intermediate_size": 1.5},
     {"eos_token_id": 10_000}, {"eos_token_id": "x"}, {"num_hidden_layers": True},
+    {"use_sliding_window": "no"}, {"attention_bias": 0}, {"model_type": "qwen2"}, {"model_type": 3},
+    {"layer_types": ["sliding_attention", "full_attention"]}, {"layer_types": ["full_attention"]},
+    {"layer_types": "full_attention"}, {"layer_types": [1, 2]},
 ])
 def test_rejects(change):
     raw = copy.deepcopy(TINY["A"])
@@ -104,6 +107,8 @@ def test_load_config_from_folder(tmp_path):
     # keys that other tools write are ignored
     (tmp_path / "config.json").write_text(json.dumps(dict(TINY["C"], torch_dtype="bfloat16", model_type="qwen3",
                                                           sliding_window=None, max_window_layers=2,
+                                                          use_sliding_window=False, attention_bias=False,
+                                                          layer_types=["full_attention"] * 2,
                                                           use_cache=True, bos_token_id=1)))
     assert load_config(str(tmp_path)).vocab_size == 517
 
