@@ -84,6 +84,25 @@ class LLM:
         return out[0] if single else out
 
 
+    def stream(self, prompts, max_tokens=32, temperature=0.0, seed=None, ignore_eos=False, timeout_ms=None):
+        """As `generate` for token ids, but a generator: yields (index of the prompt, token id or None, finish
+        reason or None) as soon as a step of the scheduler has produced it; a request's last event carries its
+        reason ("stop", "length", "timeout", "cancelled")."""
+        single = len(prompts) > 0 and not isinstance(prompts[0], (list, tuple))
+        index = {}
+        for i, prompt in enumerate([prompts] if single else list(prompts)):
+            rid = self.engine.submit(prompt, max_tokens=max_tokens, temperature=temperature,
+                                     seed=None if seed is None else seed + i, ignore_eos=ignore_eos,
+                                     timeout_ms=timeout_ms)
+            index[rid] = i
+        while any(rid in index for rid in [r.id for r in self.engine.waiting + self.engine.active]):
+            for rid, token, reason in self.engine.step():
+                if rid in index:
+                    yield index[rid], token, reason
+        for rid in index:
+            self.engine.finished.pop(rid, None)
+
+
 def generate(model, prompts, max_tokens=32, temperature=0.0, seed=None, dtype="bfloat16", **engine_options):
     """One call: load the model folder, generate, return the token ids."""
     return LLM(model, dtype=dtype, **engine_options).generate(prompts, max_tokens, temperature, seed)

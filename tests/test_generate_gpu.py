@@ -323,3 +323,25 @@ def test_text_prompts_through_the_command_line_and_the_entry_point(model_folders
     assert both == [words(plain_models["A"].greedy([2, 3], 4)), words(plain_models["A"].greedy([7, 6, 8, 9], 4))]
     bad = run_cli(["--model", folder, "--prompt", ""] + common)
     assert bad.returncode == 1 and "no token" in bad.stderr
+
+
+def test_tokens_as_they_come(model_folders, plain_models):
+    """`LLM.stream`: the same tokens as `generate`, handed out step by step, each request's last event with its reason."""
+    from mini_llm_runtime_amd.api import LLM
+    llm = LLM(model_folders["A"], dtype="float32", context_tokens=256, max_model_len=64, max_active=2,
+              block_size=PAGE_SIZE["A"], batch_tokens=16, prefill_chunk=8)
+    prompts = prompts_for("A", (7, 13, 5))
+    got, reasons, order = {i: [] for i in range(3)}, {}, []
+    for i, token, reason in llm.stream(prompts, max_tokens=5, ignore_eos=True):
+        assert i not in reasons                                         # nothing after a request's last event
+        if token is not None:
+            got[i].append(token)
+            order.append(i)
+        if reason is not None:
+            reasons[i] = reason
+    assert reasons == {0: "length", 1: "length", 2: "length"}
+    for i, prompt in enumerate(prompts):
+        assert got[i] == plain_models["A"].greedy(prompt, 5)
+    assert order != sorted(order)                                       # two slots: the requests' tokens come interleaved
+    assert not llm.engine.finished and llm.runner.cache.free_pages() == llm.runner.cache.num_pages
+    assert llm.generate(prompts[0], max_tokens=5, ignore_eos=True) == got[0]      # the engine goes on as before
