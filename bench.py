@@ -111,6 +111,9 @@ class Bench:
         sampler = Sampler(runner.kernels, runner.device, max_rows=batch)
         fill = a.context - steps - warmup
         assert fill >= 1
+        # (part of the set-up, like compiling: the decoding step of this batch and context is captured before the
+        # requests exist, so that the timed steps are replays whatever --warmup is)
+        runner.warm_up(batch_sizes=[batch], contexts=[a.context])
         slots = [runner.open_request() for _ in range(batch)]
         self.fill(runner, slots, fill)
         tokens = torch.randint(0, c.vocab_size, (batch,), generator=self.g).tolist()
