@@ -16,6 +16,7 @@ class Workspace:
         self._arena = None
         self.planned_bytes = 0
         self._unplanned = {}          # (name, dtype) -> bytes allocated outside the plan
+        self._views = {}              # (name, dtype, shape) -> the view handed out for it
 
     @staticmethod
     def plan_bytes(plan):
@@ -37,6 +38,11 @@ class Workspace:
         return sum(self._unplanned.values())
 
     def get(self, name, shape, dtype):
+        # (a step asks for the same few shapes again and again: the views are kept, a steady step makes none)
+        shape = tuple(shape)
+        view = self._views.get((name, dtype, shape))
+        if view is not None:
+            return view
         count = 1
         for extent in shape:
             count *= int(extent)
@@ -46,7 +52,13 @@ class Workspace:
             buf = torch.empty(max(count, 1), dtype=dtype, device=self.device)
             self._buffers[key] = buf
             self._unplanned[key] = buf.numel() * buf.element_size()
-        return buf[:count].view(shape)
+            for stale in [k for k in self._views if k[0] == name and k[1] == dtype]:
+                del self._views[stale]                     # (views of the buffer that this one replaces)
+        view = buf[:count].view(shape)
+        if len(self._views) >= 4096:
+            self._views.clear()
+        self._views[(name, dtype, shape)] = view
+        return view
 
     def bytes(self):
         return self.planned_bytes + self.unplanned_bytes()
