@@ -45,10 +45,13 @@ except AttributeError:                                         # pragma: no cove
     _raw_stream = None
 
 
+_device_index = getattr(torch._C, "_cuda_getDevice", None)    # (the current device's index without torch.cuda's wrapper)
+
+
 def _stream():
     """Handle of torch's current stream on the current device."""
     if _raw_stream is not None:
-        return _ptr(_raw_stream(torch.cuda.current_device()))
+        return _ptr(_raw_stream(_device_index() if _device_index is not None else torch.cuda.current_device()))
     return _ptr(torch.cuda.current_stream().cuda_stream)
 
 
@@ -60,9 +63,12 @@ def _need(cond, message):
 
 def _tensor(t, name, dtype, shape=None, ndim=None):
     # one cheap test on the way that every launch takes; the message is only put together on failure
-    if (isinstance(t, torch.Tensor) and t.is_cuda and t.dtype == dtype and t.is_contiguous()
-            and (ndim is None or t.dim() == ndim) and (shape is None or t.shape == tuple(shape))):
-        return t
+    try:
+        if (t.is_cuda and t.dtype is dtype and t.is_contiguous() and (ndim is None or t.dim() == ndim)
+                and (shape is None or t.shape == shape or t.shape == tuple(shape))):
+            return t
+    except AttributeError:                                # (no tensor: said below)
+        pass
     _need(isinstance(t, torch.Tensor), f"{name}: expected a tensor")
     _need(t.is_cuda, f"{name}: must lie on the GPU (there is no CPU path)")
     _need(t.dtype == dtype, f"{name}: expected {dtype}, got {t.dtype}")
