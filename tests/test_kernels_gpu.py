@@ -137,7 +137,8 @@ def test_gemm(dtype, mnk):
             torch.testing.assert_close(out.double(), want, **t)
 
 
-@pytest.mark.parametrize("mnk", [(8, 6144, 2048), (3, 6100, 2048), (16, 5120, 2112), (1, 10240, 2048), (5, 4100, 4096)])
+@pytest.mark.parametrize("mnk", [(8, 6144, 2048), (3, 6100, 2048), (16, 5120, 2112), (1, 10240, 2048), (5, 4100, 4096),
+                                 (8, 6144, 4096), (2, 5120, 8192)])
 def test_gemm_two_strips_a_workgroup(mnk):
     """Few rows and numbers of columns that would deal strips of 16 unevenly to the compute units: a workgroup
     then owns two strips side by side (24, 20, ... columns), the last workgroup fewer.  Plain and with the rows'
