@@ -84,4 +84,48 @@ int mlr_schedule_batch(const MlrScheduleItem* items, int n, int64_t batch_tokens
     return written;
 }
 
+// Which waiting requests start now: a pure function of the queue, the pages that are not set aside and the
+// free request slots (the reference's admission, src/engine.cpp:295-355).  The queue is walked by aged
+// priority, higher first, earlier arrival first among equals; a request starts when the pages of its whole
+// life (prompt and every token it may generate) are free and a slot is; one that does not fit is passed over,
+// unless it has waited `reserve_ms` or longer: then nothing behind it starts, so that what is given back goes
+// to it.  `sorted` receives the queue's order of the walk (all n indices), `admitted` the indices that start,
+// in that order; `waits` counts the requests that did not fit.  Returns the number admitted, -1 on bad arguments.
+struct MlrWaiting {
+    int64_t pages;
+    int32_t priority;
+    int64_t waited_ms;
+    uint64_t order;
+};
+
+int mlr_admit(const MlrWaiting* items, int n, int64_t free_pages, int free_slots, int aging_ms, int64_t reserve_ms,
+              int32_t* sorted, int32_t* admitted, int64_t* waits) {
+    if (n < 0 || aging_ms <= 0 || reserve_ms < 0 || free_pages < 0) return -1;
+    std::vector<int64_t> rank(n);
+    for (int i = 0; i < n; ++i) rank[i] = mlr_effective_priority(items[i].priority, items[i].waited_ms, aging_ms);
+    std::vector<int32_t> walk(n);
+    std::iota(walk.begin(), walk.end(), 0);
+    std::sort(walk.begin(), walk.end(), [&](int a, int b) {
+        if (rank[a] != rank[b]) return rank[a] > rank[b];
+        if (items[a].order != items[b].order) return items[a].order < items[b].order;
+        return a < b;
+    });
+    int started = 0;
+    *waits = 0;
+    for (int at = 0; at < n; ++at) {
+        const int i = walk[at];
+        sorted[at] = i;
+        if (free_slots <= 0) continue;                   // (the rest of the walk only writes the order down)
+        if (items[i].pages <= free_pages) {
+            admitted[started++] = i;
+            free_pages -= items[i].pages;
+            free_slots -= 1;
+        } else {
+            *waits += 1;
+            if (items[i].waited_ms >= reserve_ms) free_slots = 0;      // the pool is kept for this one
+        }
+    }
+    return started;
+}
+
 }  // extern "C"

@@ -37,6 +37,11 @@ class _Slice(ctypes.Structure):
     _fields_ = [("key", ctypes.c_int64), ("tokens", ctypes.c_int64), ("prefill", ctypes.c_int32)]
 
 
+class _Waiting(ctypes.Structure):
+    _fields_ = [("pages", ctypes.c_int64), ("priority", ctypes.c_int32), ("waited_ms", ctypes.c_int64),
+                ("order", ctypes.c_uint64)]
+
+
 POLICIES = {"mixed": 0, "prefill_first": 1}
 
 
@@ -47,12 +52,31 @@ def _lib():
                                            ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.POINTER(_Slice)]
         lib.mlr_effective_priority.argtypes = [ctypes.c_int, ctypes.c_int64, ctypes.c_int]
         lib.mlr_effective_priority.restype = ctypes.c_int64
+        lib.mlr_admit.argtypes = [ctypes.POINTER(_Waiting), ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
+                                  ctypes.c_int64, ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_int32),
+                                  ctypes.POINTER(ctypes.c_int64)]
         lib._mlr_sched_typed = True
     return lib
 
 
 def effective_priority(priority, wait_ms, aging_ms):
     return _lib().mlr_effective_priority(priority, int(wait_ms), aging_ms)
+
+
+def admit(items, free_pages, free_slots, aging_ms=250, reserve_ms=2000):
+    """items: (pages of the request's whole life, priority, waited_ms, order) of every waiting request.  Returns
+    (the queue's indices in the order of the walk, the indices that start now in that order, how many did not
+    fit): see `mlr_admit`."""
+    n = len(items)
+    arr = (_Waiting * max(n, 1))()
+    for i, (pages, priority, waited_ms, order) in enumerate(items):
+        arr[i] = _Waiting(pages, priority, int(waited_ms), order)
+    walk, started = (ctypes.c_int32 * max(n, 1))(), (ctypes.c_int32 * max(n, 1))()
+    waits = ctypes.c_int64(0)
+    count = _lib().mlr_admit(arr, n, free_pages, free_slots, aging_ms, reserve_ms, walk, started, ctypes.byref(waits))
+    if count < 0:
+        raise ValueError("aging_ms must be positive, reserve_ms and free_pages not negative")
+    return list(walk[:n]), list(started[:count]), waits.value
 
 
 def schedule_batch(items, batch_tokens, prefill_chunk, policy="mixed", aging_ms=250, portion_step=0):
@@ -251,32 +275,27 @@ class Engine:
         return (tokens + self._unit - 1) // self._unit
 
     # -- admission -------------------------------------------------------------------------------
-    def _admit(self, req):
-        pages = self._pages_for(len(req.prompt) + req.max_tokens)
-        if pages > self.free_credits or self.runner.free_slots() == 0:
-            return False
-        req.slot = self.runner.open_request()
-        req.pages = pages
-        self.free_credits -= pages
-        self.active.append(req)
-        return True
-
     def _admit_waiting(self):
+        """The decision is `admit`'s (native, a pure function of the queue); here it is carried out: a slot and
+        the pages of its whole life for every request that starts, the queue left in the order of the walk."""
+        if not self.waiting:
+            return
         o = self.options
         now = self.clock()
-        ms = lambda t: int((now - t) * 1000)
-        self.waiting.sort(key=lambda r: (-effective_priority(r.priority, ms(r.created), o.aging_ms), r.order))
-        i = 0
-        while i < len(self.waiting) and self.runner.free_slots() > 0:
+        items = [(self._pages_for(len(r.prompt) + r.max_tokens), r.priority, int((now - r.created) * 1000), r.order)
+                 for r in self.waiting]
+        walk, started, waits = admit(items, self.free_credits, self.runner.free_slots(), o.aging_ms,
+                                     o.admission_reserve_ms)
+        self.stats["admission_waits"] += waits
+        queue = [self.waiting[i] for i in walk]
+        for i in started:
             req = self.waiting[i]
-            if self._admit(req):
-                self.waiting.pop(i)
-            elif ms(req.created) >= o.admission_reserve_ms:
-                self.stats["admission_waits"] += 1
-                break
-            else:
-                self.stats["admission_waits"] += 1
-                i += 1
+            req.slot = self.runner.open_request()
+            req.pages = items[i][0]
+            self.free_credits -= req.pages
+            self.active.append(req)
+        going = set(started)
+        self.waiting = [r for i, r in zip(walk, queue) if i not in going]
 
     def _finish(self, req, reason):
         req.finish_reason = reason

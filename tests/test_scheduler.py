@@ -382,3 +382,28 @@ def test_portions_that_do_not_end_a_prompt_are_multiples_of_the_step():
     assert schedule_batch(items, 8, 8, portion_step=32) == [(0, 1, False), (2, 7, True)]
     with pytest.raises(ValueError):
         schedule_batch(items, 8, 8, portion_step=-1)
+
+
+def test_admission_is_a_pure_function_of_the_queue():
+    """`admit` (native): the walk by aged priority, what fits starts, what does not is passed over until it has
+    waited the reserve time, and then holds everything behind it back (src/engine.cpp:295-355)."""
+    from mini_llm_runtime_amd.engine import admit
+    # (pages of the whole life, priority, waited ms, order)
+    queue = [(4, 0, 0, 0), (10, 0, 0, 1), (2, 0, 0, 2)]
+    assert admit(queue, free_pages=6, free_slots=3) == ([0, 1, 2], [0, 2], 1)          # the second is passed over
+    assert admit(queue, free_pages=16, free_slots=3) == ([0, 1, 2], [0, 1, 2], 0)
+    assert admit(queue, free_pages=16, free_slots=1) == ([0, 1, 2], [0], 0)            # no slot: no wait counted
+    assert admit(queue, free_pages=1, free_slots=3) == ([0, 1, 2], [], 3)
+    assert admit([], free_pages=5, free_slots=2) == ([], [], 0)
+    # one that has waited the reserve time walks first (eight aging intervals) and, not fitting, holds the rest back
+    held = [(4, 0, 0, 0), (10, 0, 2000, 1), (2, 0, 0, 2)]
+    assert admit(held, free_pages=6, free_slots=3) == ([1, 0, 2], [], 1)
+    assert admit(held, free_pages=6, free_slots=3, reserve_ms=2001) == ([1, 0, 2], [0, 2], 1)
+    assert admit(held, free_pages=12, free_slots=3) == ([1, 0, 2], [1, 2], 1)          # it starts; the first no longer fits
+    # priority first, then waiting (an aging interval is worth one level), then arrival
+    ranked = [(1, 0, 0, 0), (1, 3, 0, 1), (1, 1, 600, 2), (1, 3, 0, 3), (1, 2, 250, 4)]
+    assert admit(ranked, free_pages=2, free_slots=5)[:2] == ([1, 2, 3, 4, 0], [1, 2])
+    assert admit(ranked, free_pages=2, free_slots=5, aging_ms=1000)[0] == [1, 3, 4, 2, 0]
+    for bad in (dict(aging_ms=0), dict(reserve_ms=-1), dict(free_pages=-1)):
+        with pytest.raises(ValueError):
+            admit(queue, **{"free_pages": 6, "free_slots": 3, **bad})
