@@ -1,6 +1,7 @@
 """What a part may see of the running step, and the scratch memory it may use."""
 from __future__ import annotations
 
+import numpy as np
 import torch
 
 
@@ -80,7 +81,7 @@ class Uploader:
         self._busy = False
 
     def send(self, values, dst):
-        """values: list of ints; dst: device int32 vector of at least that many elements."""
+        """values: a list of ints or an int32 numpy vector; dst: device int32 vector of at least that many elements."""
         n = len(values)
         if n > self._host.numel():
             if self._busy:
@@ -89,7 +90,10 @@ class Uploader:
             self._host = torch.empty(max(n, 2 * self._host.numel()), dtype=torch.int32).pin_memory()
         if self._busy:
             self._event.synchronize()
-        self._host[:n] = torch.tensor(values, dtype=torch.int32)
+        if isinstance(values, np.ndarray):
+            self._host.numpy()[:n] = values               # (a view of the pinned buffer: one copy, no tensor made)
+        else:
+            self._host[:n] = torch.tensor(values, dtype=torch.int32)
         dst[:n].copy_(self._host[:n], non_blocking=True)
         self._event.record()
         self._busy = True

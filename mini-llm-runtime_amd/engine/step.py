@@ -10,6 +10,7 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 from typing import List, Sequence
 
+import numpy as np
 import torch
 
 from ..cache.manager import CacheManager
@@ -193,7 +194,7 @@ class Runner:
                 return False
         return True
 
-    def _graph_step(self, entries, first, total, sig, fill=0, fill_first=False):
+    def _graph_step(self, entries, arrays, first, total, sig, fill=0, fill_first=False):
         """The same kernels as any step, launched from a captured graph.  The graph's buffers are fixed:
         token ids, positions and slots live in a vector of their own per shape (the wanted rows and the
         token groups, which depend on the shape only, are written there once), key splits are laid out
@@ -222,26 +223,10 @@ class Runner:
         else:
             self._graphs[sig] = self._graphs.pop(sig)        # most recently used last
         meta = state["meta"]
-        ids, pos, slot_of, segments = [], [], [], []
-
-        def scratch_rows():                               # rows of the scratch request: token 0 at position 0
-            for _ in range(fill):
-                segments.append((self.cache.scratch_slot, len(ids), 1, 0))
-                ids.append(0)
-                pos.append(0)
-                slot_of.append(self.cache.scratch_slot)
-        if fill_first:
-            scratch_rows()
-        for e, p0 in zip(entries, first):
-            n = len(e.tokens)
-            segments.append((e.slot, len(ids), n, p0))
-            ids.extend(int(t) for t in e.tokens)
-            pos.extend(range(p0, p0 + n))
-            slot_of.extend([e.slot] * n)
-        if not fill_first:
-            scratch_rows()
+        rows_of, segments = self._rows(entries, arrays, first, fill, fill_first)
         n_seg = len(segments)
-        state["upload"].send(ids + pos + slot_of + [seg[0] for seg in segments], meta)
+        state["upload"].send(np.concatenate([rows_of.ravel(), np.fromiter((seg[0] for seg in segments), np.int32, n_seg)]),
+                             meta)
         if state["graph"] is not None:
             state["graph"].replay()
             return state["logits"]
@@ -352,32 +337,109 @@ class Runner:
             raise StepError("empty batch")
         vocab = self.model.spec.vocab_size
         total = 0
+        arrays, wanted = [], []
         for e in entries:
             n = len(e.tokens)
             if n == 0:
                 raise StepError("a batch entry must bring at least one token")
             total += n
-            for t in e.tokens:
-                if not 0 <= int(t) < vocab:
-                    raise StepError(f"token id {t} is outside the vocabulary [0, {vocab})")
-            for w in e.want:
-                if not 0 <= int(w) < n:
-                    raise StepError(f"wanted place {w} is outside the entry's {n} tokens")
-            if len(set(int(w) for w in e.want)) != len(e.want):
-                # (a place named once bounds the wanted rows by the step's tokens, which the metadata
-                # vector is sized for)
-                raise StepError("a wanted place is named twice in one entry")
+            arrays.append(self._token_ids(e.tokens, vocab))
+            places = len(e.want)
+            if places <= 16:                              # (few places: plain comparisons cost less than vectors)
+                for w in e.want:
+                    if not 0 <= int(w) < n:
+                        raise StepError(f"wanted place {w} is outside the entry's {n} tokens")
+                if places > 1 and len(set(int(w) for w in e.want)) != places:
+                    raise StepError("a wanted place is named twice in one entry")
+                want = [int(w) for w in e.want]
+            else:
+                want = np.asarray(e.want, dtype=np.int64).reshape(-1)
+                if want.min() < 0 or want.max() >= n:
+                    bad = want[(want < 0) | (want >= n)][0]
+                    raise StepError(f"wanted place {bad} is outside the entry's {n} tokens")
+                if np.unique(want).size != want.size:
+                    # (a place named once bounds the wanted rows by the step's tokens, which the metadata
+                    # vector is sized for)
+                    raise StepError("a wanted place is named twice in one entry")
+            wanted.append(want)
         if total > self.max_batch_tokens:
             raise StepError(f"{total} tokens exceed the step's limit of {self.max_batch_tokens}")
-        wanted = sum(len(e.want) for e in entries)
-        if wanted > self.max_logits_rows:
-            raise StepError(f"{wanted} wanted places exceed the step's limit of {self.max_logits_rows}")
-        return total
+        rows = sum(len(w) for w in wanted)
+        if rows > self.max_logits_rows:
+            raise StepError(f"{rows} wanted places exceed the step's limit of {self.max_logits_rows}")
+        return total, arrays, wanted
+
+    @staticmethod
+    def _token_ids(tokens, vocab):
+        """An entry's tokens, checked (as they came when they are few, else as an int32 vector); refused when they
+        are no whole numbers of the vocabulary."""
+        if len(tokens) <= 16:                             # (few tokens: plain comparisons cost less than vectors)
+            for t in tokens:
+                try:
+                    inside = 0 <= t < vocab and int(t) == t
+                except (TypeError, ValueError):
+                    raise StepError("token ids must be whole numbers") from None
+                if not inside:
+                    raise StepError(f"token id {t} is outside the vocabulary [0, {vocab})" if isinstance(t, (int, np.integer))
+                                    else "token ids must be whole numbers")
+            return tokens                                 # (as they came: `_rows` puts them into its vector)
+        ids = np.asarray(tokens)
+        if ids.ndim != 1 or ids.dtype.kind not in "iub":
+            try:                                          # (numbers too large for a machine word, or no numbers)
+                ids = np.asarray([int(t) for t in tokens], dtype=object)
+            except (TypeError, ValueError):
+                raise StepError("token ids must be whole numbers") from None
+            if any(t != u for t, u in zip(ids, tokens)):
+                raise StepError("token ids must be whole numbers")
+        outside = (ids < 0) | (ids >= vocab)
+        if outside.any():
+            raise StepError(f"token id {ids[outside][0]} is outside the vocabulary [0, {vocab})")
+        return ids.astype(np.int32)
+
+    def _rows(self, entries, arrays, first, fill=0, fill_first=False):
+        """(token ids | positions | slots of the step's rows as int32 [3, rows], the segments (slot, first row,
+        tokens, first position)); `fill` rows of the scratch request (token 0 at position 0) in front or behind."""
+        total = sum(len(a) for a in arrays) + fill
+        scratch = self.cache.scratch_slot
+        if total <= 4 * (len(entries) + fill):
+            # mostly single tokens (a decoding step): three short lists and one conversion cost less than
+            # a few vector operations for every entry
+            ids, pos, slot_of, segments = [], [], [], []
+            if fill and fill_first:
+                segments = [(scratch, i, 1, 0) for i in range(fill)]
+                ids, pos, slot_of = [0] * fill, [0] * fill, [scratch] * fill
+            for e, tokens, p0 in zip(entries, arrays, first):
+                n = len(tokens)
+                segments.append((e.slot, len(ids), n, p0))
+                ids.extend(tokens)
+                pos.extend(range(p0, p0 + n))
+                slot_of.extend([e.slot] * n)
+            if fill and not fill_first:
+                segments += [(scratch, len(ids) + i, 1, 0) for i in range(fill)]
+                ids, pos, slot_of = ids + [0] * fill, pos + [0] * fill, slot_of + [scratch] * fill
+            return np.array([ids, pos, slot_of], dtype=np.int32), segments
+        rows = np.empty((3, total), dtype=np.int32)
+        segments, at = [], 0
+        if fill and fill_first:
+            rows[0:2, :fill], rows[2, :fill] = 0, scratch
+            segments += [(scratch, i, 1, 0) for i in range(fill)]
+            at = fill
+        for e, ids, p0 in zip(entries, arrays, first):
+            n = len(ids)
+            rows[0, at:at + n] = ids
+            rows[1, at:at + n] = np.arange(p0, p0 + n, dtype=np.int32)
+            rows[2, at:at + n] = e.slot
+            segments.append((e.slot, at, n, p0))
+            at += n
+        if fill and not fill_first:
+            rows[0:2, at:], rows[2, at:] = 0, scratch
+            segments += [(scratch, at + i, 1, 0) for i in range(fill)]
+        return rows, segments
 
     def step(self, entries: List[Entry]):
         """Returns float logits [R, V] on the device (R = wanted places, in the order of the
         entries and of their `want`), or None when nothing is wanted."""
-        total = self._validate(entries)
+        total, arrays, wanted = self._validate(entries)
         slots = [e.slot for e in entries]
         counts = [len(e.tokens) for e in entries]
         first = self.cache.commit_first(slots, counts)    # raises with nothing changed, else takes the pages
@@ -389,26 +451,25 @@ class Runner:
             if sig is not None:                           # a captured step is keyed by its shape and its context bucket
                 sig = (sig, self._context_bucket(max(p0 + n for p0, n in zip(first, counts))))
             if sig is not None and self._graph_wanted(entries, total + fill, sig):
-                logits = self._graph_step(entries, first, total + fill, sig, fill, fill_first)
+                logits = self._graph_step(entries, arrays, first, total + fill, sig, fill, fill_first)
                 self.cache.retire(slots)
                 self.steps += 1
                 self._raise_if_not_finite()
                 if fill and logits is not None:           # the scratch rows' logits are dropped
                     return logits[fill:] if fill_first else logits[:len(entries)]
                 return logits
-            ids, pos, slot_of, rows = [], [], [], []
-            segments = []
-            for e, p0 in zip(entries, first):
-                base = len(ids)
-                n = len(e.tokens)
-                segments.append((e.slot, base, n, p0))
-                ids.extend(int(t) for t in e.tokens)
-                pos.extend(range(p0, p0 + n))
-                slot_of.extend([e.slot] * n)
-                rows.extend(base + int(w) for w in e.want)
-            r = len(rows)
+            rows_of, segments = self._rows(entries, arrays, first)
+            if all(type(w) is list for w in wanted):       # (few places each: one short list)
+                rows = np.array([seg[1] + w for seg, places in zip(segments, wanted) for w in places], dtype=np.int32)
+            else:
+                rows = np.concatenate([seg[1] + np.asarray(w, dtype=np.int64) for seg, w in zip(segments, wanted)]
+                                      ).astype(np.int32)
+            r = rows.size
             stateful = self.cache.has_state()
-            self._upload.send(ids + pos + slot_of + rows + ([seg[0] for seg in segments] if stateful else []), self._meta)
+            parts = [rows_of.ravel(), rows]
+            if stateful:
+                parts.append(np.fromiter((seg[0] for seg in segments), np.int32, len(segments)))
+            self._upload.send(np.concatenate(parts), self._meta)
             ctx = self.ctx
             ctx.begin_step()
             ctx.n_tokens = total
