@@ -8,14 +8,17 @@
 // block the wavefronts of parity 0 take keys 0..31 and those of parity 1 keys 32..63.  The two parities of
 // a column are merged through LDS at the end.
 //
-// A wavefront's block is one chain of dependent steps (keys from LDS, eight products into one accumulator,
-// maximum, exponentials, sum, eight products more, staging), and a vector instruction that needs the result
-// of the one before it issues every 9 cycles, not every 4 (measured; 6 with eight independent chains).  A
-// group's time is therefore the length of that chain times its blocks, whatever else runs on the compute
-// unit (measured at 2 048 tokens: the last group alone on the GPU 36.6 us, the whole prompt 44.1), and the
-// loop counts its instructions: offsets that do not change are computed once, a thread stages 32 contiguous
-// bytes per page lookup, blocks whose keys are all written are staged without checks, the maximum of a
-// tile is taken three values at a time.
+// What a tile costs (measured): about 2 000 cycles of its SIMD, whether one wavefront or two share the SIMD: the
+// last group of a 2 048-token prompt alone on the GPU (one wavefront a SIMD) takes 36.6 us for its 32 blocks, the
+// whole prompt 42-44 (two a SIMD most of the time), a prompt of 8 192 tokens 0.95 us a tile and SIMD; and a
+// workgroup of eight wavefronts that shares blocks of 128 keys between four key parities (half as many turns
+// for a group) takes as long as this one.  Counted per tile at long contexts: 128 vector instructions (a
+// dependent one issues every 9 cycles, independent ones every 6, an exponential every 10-13), 16 matrix
+// instructions (512 cycles), 47 scalar ones, 16 reads and 8 writes of 16 bytes a lane through the LDS (24 KB;
+// a wavefront's read takes 31 cycles) -- which add up rather than overlap.  So the loop counts its
+// instructions: offsets that do not change are computed once, a thread stages 32 contiguous bytes per page
+// lookup, blocks whose keys are all written are staged without checks, the maximum of a tile is taken three
+// values at a time.
 //
 // Per tile of 32 keys, with v_mfma_f32_32x32x16_bf16:
 //   S^T[key][column]  = K[key][d] . Q^T[d][column]         A = 32 keys x 16 channels from LDS, B = Q (registers)
