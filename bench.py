@@ -178,6 +178,38 @@ class Bench:
         torch.cuda.empty_cache()
         return out
 
+    def prompt(self, portion=PREFILL_TOKENS, reps=2):
+        """One prompt of --context tokens, run in portions of `portion` tokens (the last one wants its logits):
+        tokens a second over the whole prompt and the time of every portion, whose attention reads all the keys
+        before it."""
+        from mini_llm_runtime_amd.engine import Entry
+        torch, a, c = self.torch, self.args, self.cfg
+        total = a.context
+        runner = self.runner(1, total, total, portion, graph_max_tokens=portion if a.prefill_graph else 512)
+        ids = torch.randint(0, c.vocab_size, (total,), generator=self.g).tolist()
+        best = None
+        for _ in range(reps):
+            s = runner.open_request()
+            times = []
+            for at in range(0, total, portion):
+                part = ids[at:at + portion]
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                runner.step([Entry(s, part, [len(part) - 1] if at + portion >= total else [])])
+                torch.cuda.synchronize()
+                times.append(time.perf_counter() - t0)
+            runner.close_request(s)
+            best = times if best is None or sum(times) < sum(best) else best
+        seconds = sum(best)
+        flops = 2.0 * total * self.layers * self.layer_params \
+            + 2.0 * total * total * c.num_attention_heads * c.head_dim * self.layers \
+            + 2.0 * c.vocab_size * c.hidden_size
+        del runner
+        torch.cuda.empty_cache()
+        return dict(value=round(total / seconds, 1), tokens=total, portion=portion, ms=round(seconds * 1e3, 2),
+                    frac=round(flops / seconds / MFMA_PEAK[self.tag], 5),
+                    first_portion_ms=round(best[0] * 1e3, 2), last_portion_ms=round(best[-1] * 1e3, 2))
+
     def mixed(self, decoding=64, reps=6):
         """ONE step that holds `decoding` single tokens of requests at the context length beside a portion of
         2048 tokens of another request's prompt (the reference's mixed workload,
@@ -279,8 +311,9 @@ def main():
     ap.add_argument("--no-8b", action="store_true", help="skip the block of 8B measurements in the default run")
     ap.add_argument("--warm-up", type=int, default=0,
                     help="--only engine: 1 captures the decoding steps (Engine.warm_up) before the first burst")
-    ap.add_argument("--only", default="all", choices=["all", "decode", "prefill", "engine", "mixed"],
-                    help="profiling aid: run just the decode steps, just the prefill or just the mixed step; engine: the "
+    ap.add_argument("--only", default="all", choices=["all", "decode", "prefill", "prompt", "engine", "mixed"],
+                    help="profiling aid: run just the decode steps, just the prefill or just the mixed step; prompt: one "
+                         "prompt of --context tokens in portions of 2048; engine: the "
                          "scheduler over a burst of requests (3 x batch requests of 512 prompt and 128 output tokens, "
                          "batch slots), printed as one line of its own")
     ap.add_argument("--library", type=int, default=1,
@@ -309,6 +342,9 @@ def main():
     c = bench.cfg
     if args.only == "prefill":
         print(json.dumps({"prefill": bench.prefill()}))
+        return 0
+    if args.only == "prompt":
+        print(json.dumps({"prompt": dict(bench.prompt(), model=f"Qwen3-{args.size.upper()} sizes", layers=bench.layers)}))
         return 0
     if args.only == "engine":
         print(json.dumps({"engine": bench.engine_burst()}))

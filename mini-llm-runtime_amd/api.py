@@ -71,36 +71,56 @@ class LLM:
             texts = [self.tokenizer.text([t for t in row if t not in eos]) for row in ids]
             return texts[0] if one else texts
         single = len(prompts) > 0 and not isinstance(prompts[0], (list, tuple))
-        batch = [prompts] if single else list(prompts)
-        ids = []
-        for i, prompt in enumerate(batch):
-            ids.append(self.engine.submit(prompt, max_tokens=max_tokens, temperature=temperature,
-                                          seed=None if seed is None else seed + i, ignore_eos=ignore_eos,
-                                          timeout_ms=timeout_ms))
+        ids = self._submit_all([prompts] if single else list(prompts), max_tokens, temperature, seed, ignore_eos,
+                               timeout_ms)
         done = self.engine.run_until_done()
         out = [done[i] for i in ids]
         for i in ids:
             self.engine.finished.pop(i, None)      # handed over: a long-lived engine keeps no record of them
         return out[0] if single else out
 
-
     def stream(self, prompts, max_tokens=32, temperature=0.0, seed=None, ignore_eos=False, timeout_ms=None):
         """As `generate` for token ids, but a generator: yields (index of the prompt, token id or None, finish
         reason or None) as soon as a step of the scheduler has produced it; a request's last event carries its
-        reason ("stop", "length", "timeout", "cancelled")."""
+        reason ("stop", "length", "timeout", "cancelled").  A caller that stops reading early (closes the
+        generator) cancels what still runs: nothing of it is left in the engine."""
         single = len(prompts) > 0 and not isinstance(prompts[0], (list, tuple))
-        index = {}
-        for i, prompt in enumerate([prompts] if single else list(prompts)):
-            rid = self.engine.submit(prompt, max_tokens=max_tokens, temperature=temperature,
-                                     seed=None if seed is None else seed + i, ignore_eos=ignore_eos,
-                                     timeout_ms=timeout_ms)
-            index[rid] = i
-        while any(rid in index for rid in [r.id for r in self.engine.waiting + self.engine.active]):
-            for rid, token, reason in self.engine.step():
-                if rid in index:
-                    yield index[rid], token, reason
-        for rid in index:
-            self.engine.finished.pop(rid, None)
+        ids = self._submit_all([prompts] if single else list(prompts), max_tokens, temperature, seed, ignore_eos,
+                               timeout_ms)
+        index = {rid: i for i, rid in enumerate(ids)}
+        live = set(ids)
+        try:
+            while live:
+                for rid, token, reason in self.engine.step():
+                    if rid in index:
+                        if reason is not None:
+                            live.discard(rid)
+                        yield index[rid], token, reason
+        finally:
+            self._withdraw(live)
+            for rid in ids:
+                self.engine.finished.pop(rid, None)
+
+    def _submit_all(self, batch, max_tokens, temperature, seed, ignore_eos, timeout_ms):
+        """Queues every prompt or none: when one is refused, those queued before it are taken back."""
+        ids = []
+        try:
+            for i, prompt in enumerate(batch):
+                ids.append(self.engine.submit(prompt, max_tokens=max_tokens, temperature=temperature,
+                                              seed=None if seed is None else seed + i, ignore_eos=ignore_eos,
+                                              timeout_ms=timeout_ms))
+        except Exception:
+            self._withdraw(ids)
+            for rid in ids:
+                self.engine.finished.pop(rid, None)
+            raise
+        return ids
+
+    def _withdraw(self, ids):
+        if ids and not self.engine.failed:
+            for rid in ids:
+                self.engine.cancel(rid)
+            self.engine.expire()
 
 
 def generate(model, prompts, max_tokens=32, temperature=0.0, seed=None, dtype="bfloat16", **engine_options):

@@ -250,13 +250,14 @@ class Engine:
         (src/engine.cpp:637).  Returns the events."""
         for req in self.waiting + self.active:
             req.cancelled = True
-        events = self._expire()
+        events = self.expire()
         self.failed = True
         return events
 
-    def _expire(self):
-        """Ends what was cancelled or has run out of time, before the next batch is formed: a waiting request
-        leaves the queue, a running one gives back its slot, its pages and its reservation."""
+    def expire(self):
+        """Ends what was cancelled or has run out of time (every `step` begins with it, before the next batch
+        is formed): a waiting request leaves the queue, a running one gives back its slot, its pages and its
+        reservation.  Returns the events."""
         now = self.clock()
         events = []
         for req in [r for r in self.waiting + self.active if r.cancelled or (r.deadline is not None and now >= r.deadline)]:
@@ -312,7 +313,7 @@ class Engine:
         if self.failed:
             raise RuntimeError("the engine stopped after a failed step")
         o = self.options
-        expired = self._expire()
+        expired = self.expire()
         self._admit_waiting()
         if not self.active:
             if self.waiting:

@@ -345,3 +345,36 @@ def test_tokens_as_they_come(model_folders, plain_models):
     assert order != sorted(order)                                       # two slots: the requests' tokens come interleaved
     assert not llm.engine.finished and llm.runner.cache.free_pages() == llm.runner.cache.num_pages
     assert llm.generate(prompts[0], max_tokens=5, ignore_eos=True) == got[0]      # the engine goes on as before
+
+
+def test_nothing_is_left_behind(model_folders, plain_models):
+    """A batch with a prompt that is refused queues none of its prompts, and a stream that its reader closes
+    early cancels what still runs: afterwards the engine is idle, every page and slot is free, and the next
+    call answers as a fresh engine would."""
+    from mini_llm_runtime_amd.api import LLM
+    llm = LLM(model_folders["A"], dtype="float32", context_tokens=256, max_model_len=64, max_active=2,
+              block_size=PAGE_SIZE["A"], batch_tokens=16, prefill_chunk=8)
+    prompts = prompts_for("A", (7, 13, 5))
+
+    def idle():
+        return (not llm.engine.has_work() and not llm.engine.finished
+                and llm.runner.cache.free_pages() == llm.runner.cache.num_pages
+                and llm.runner.free_slots() == 2 and llm.engine.free_credits == llm.engine.total_pages)
+
+    vocab = llm.model.spec.vocab_size
+    with pytest.raises(ValueError, match="outside the vocabulary"):
+        llm.generate([prompts[0], prompts[1], [1, vocab]], max_tokens=5)
+    assert idle()
+    with pytest.raises(ValueError, match="exceed max_model_len"):
+        next(llm.stream([prompts[0], list(range(70))], max_tokens=5))
+    assert idle()
+
+    withdrawn = llm.engine.stats["cancelled"]               # (the prompts queued before the refused ones)
+    assert withdrawn == 3
+    events = llm.stream(prompts, max_tokens=20, ignore_eos=True)
+    seen = [next(events) for _ in range(4)]                 # the first two requests run, the third still waits
+    assert all(reason is None for _, _, reason in seen)
+    events.close()
+    assert idle() and llm.engine.stats["cancelled"] == withdrawn + 3
+    assert llm.generate(prompts[2], max_tokens=6, ignore_eos=True) == plain_models["A"].greedy(prompts[2], 6)
+    assert idle()
