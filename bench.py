@@ -178,13 +178,15 @@ class Bench:
         torch.cuda.empty_cache()
         return out
 
-    def prompt(self, portion=PREFILL_TOKENS, reps=2):
+    def prompt(self, portion=PREFILL_TOKENS):
         """One prompt of --context tokens, run in portions of `portion` tokens (the last one wants its logits):
         tokens a second over the whole prompt and the time of every portion, whose attention reads all the keys
-        before it."""
+        before it.  The fastest of several runs counts; a short prompt is run often enough for its step to be
+        captured and replayed, as on a server that has met the shape before."""
         from mini_llm_runtime_amd.engine import Entry
         torch, a, c = self.torch, self.args, self.cfg
         total = a.context
+        reps = 10 if total <= 2 * portion else 2
         runner = self.runner(1, total, total, portion, graph_max_tokens=portion if a.prefill_graph else 512)
         ids = torch.randint(0, c.vocab_size, (total,), generator=self.g).tolist()
         best = None
