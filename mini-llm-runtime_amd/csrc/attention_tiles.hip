@@ -71,6 +71,7 @@ struct TileArgs {
     int groups, max_blocks, q_heads, kv_heads, head_dim, page_size, page_shift, window, split_keys, max_splits;
     float scale;
     int all_resident;            // the grid fits the GPU at once (two workgroups of 64 columns a compute unit)
+    int single;                  // host: the caller's `pairing`; kernel: 1 every workgroup takes one group, 0 two (group i and group groups - 1 - i)
 };
 
 template <int ND, int NQ>
@@ -476,7 +477,9 @@ __global__ __launch_bounds__(256) void tiles_combine_kernel(TileArgs a) {
 
 // Workgroups of 128 columns take two groups, one after the other: group i and group (groups - 1 - i).
 // Within a long prompt the groups' key ranges grow with their position, so every workgroup gets about the
-// same work.  Workgroups of 64 columns take one group each, the later (longer) groups first, and two of
+// same work -- unless the pairs would be fewer than the compute units: then every group gets a workgroup of
+// its own (a 2 048-token portion of the 0.6B sizes behind 30 000 tokens of context: 20.4 ms for 23.7 with
+// workgroups of 64 columns, which load and stage every key twice as often a column).  Workgroups of 64 columns take one group each, the later (longer) groups first, and two of
 // them share a compute unit.  When all of them fit the GPU at once, the order is: the later half of the
 // groups, longest first, then the earlier half, shortest first, so that the longest group shares its compute
 // unit with the shortest (measured at 2 048 tokens: 42.4 us for 44.1; with more workgroups than places the
@@ -491,7 +494,7 @@ __global__ __launch_bounds__(128 * NQ, NQ == 2 ? 2 : 1) void attention_tiles_ker
     if (total % 8 == 0) lin = (lin % 8) * (total / 8) + lin / 8;
     const int first = lin % per_head, kvh = lin / per_head;
     const int second = a.groups - 1 - first;
-    if (NQ == 2 || a.max_splits > 1) {                  // one group a workgroup, the later ones first
+    if (a.single) {                                     // one group a workgroup, the later ones first
         // (with splits: split by split, so that the workgroups under way at a time walk the same keys.
         // Measured at 2048 tokens in two splits: 53 us; a group's splits side by side: 60; no split: 44)
         const int half = (a.groups + 1) / 2;
@@ -516,8 +519,6 @@ static int launch_tiles(const TileArgs& a, hipStream_t stream) {
         if (e != hipSuccess) return (int)e;
         prepared = true;
     }
-    const bool single = NQ == 2 || a.max_splits > 1;
-    dim3 grid(single ? a.groups : (a.groups + 1) / 2, a.kv_heads, a.max_splits);
     static int compute_units = 0;
     if (compute_units == 0) {
         int device = 0;
@@ -525,7 +526,12 @@ static int launch_tiles(const TileArgs& a, hipStream_t stream) {
             hipDeviceGetAttribute(&compute_units, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess)
             compute_units = -1;
     }
+    // (pairs that would leave compute units idle are no gain: then every group gets a workgroup of its own)
+    const bool few_pairs = (long)((a.groups + 1) / 2) * a.kv_heads < compute_units;
+    const bool single = NQ == 2 || a.max_splits > 1 || a.single == 1 || (a.single == 0 && few_pairs);
+    dim3 grid(single ? a.groups : (a.groups + 1) / 2, a.kv_heads, a.max_splits);
     TileArgs b = a;
+    b.single = single ? 1 : 0;
     b.all_resident = NQ == 2 && compute_units > 0 && (long)a.groups * a.kv_heads * a.max_splits <= 2L * compute_units;
     attention_tiles_kernel<ND, NQ><<<grid, 128 * NQ, lds, stream>>>(b);
     int err = (int)hipGetLastError();
@@ -551,16 +557,19 @@ static int launch_tiles_dim(const TileArgs& a, hipStream_t stream) {
 // Groups: group_row0[i] = first batch row of group i, group_ntok[i] = its tokens (consecutive rows of one
 // request, at most columns / (q_heads / kv_heads); columns = 128 or 64).  A group's keys must span at most
 // PAGE_IDS pages (per key split, with splits).  The cache of num_pages pages must hold fewer than 2^32 elements.
-// With max_splits > 1, `partial` holds M * q_heads * max_splits * (head_dim + 4) floats, 16-byte aligned, M the batch's rows.  Returns 0, a HIP error
+// With max_splits > 1, `partial` holds M * q_heads * max_splits * (head_dim + 4) floats, 16-byte aligned, M the batch's rows.
+// `pairing` (workgroups of 128 columns without splits): 0 two groups a workgroup unless that would leave compute
+// units idle, 1 always one group a workgroup, 2 always two.  Returns 0, a HIP error
 // code, or a negative number for sizes this kernel does not take.
 extern "C" int mlr_attention_tiles(
     const void* q, const void* k_pages, const void* v_pages, const int32_t* block_table, int max_blocks,
     const int32_t* slots, const int32_t* positions, void* out, const int32_t* group_row0,
     const int32_t* group_ntok, int groups, int columns, int q_heads, int kv_heads, int head_dim, int page_size,
-    int num_pages, int window, float scale, int split_keys, int max_splits, float* partial, hipStream_t stream) {
+    int num_pages, int window, float scale, int split_keys, int max_splits, float* partial, int pairing,
+    hipStream_t stream) {
     if (groups <= 0) return 0;
     if (head_dim % 16 != 0 || head_dim < 16 || head_dim > 128 || q_heads % kv_heads != 0 ||
-        (columns != 128 && columns != 64) || q_heads / kv_heads > columns) return -1;
+        (columns != 128 && columns != 64) || q_heads / kv_heads > columns || pairing < 0 || pairing > 2) return -1;
     if (page_size < 16 || (page_size & (page_size - 1)) != 0) return -2;
     if (max_splits < 1) max_splits = 1;
     if (max_splits > 1 && (partial == nullptr || split_keys <= 0 || split_keys % BLOCK_KEYS != 0 ||
@@ -572,6 +581,6 @@ extern "C" int mlr_attention_tiles(
     while ((1 << shift) < page_size) ++shift;
     TileArgs a{(const __bf16*)q, (const __bf16*)k_pages, (const __bf16*)v_pages, block_table, slots, positions,
                (__bf16*)out, group_row0, group_ntok, partial, groups, max_blocks, q_heads, kv_heads, head_dim,
-               page_size, shift, window, split_keys, max_splits, scale, 0};
+               page_size, shift, window, split_keys, max_splits, scale, 0, pairing};
     return columns == 128 ? launch_tiles_dim<4>(a, stream) : launch_tiles_dim<2>(a, stream);
 }

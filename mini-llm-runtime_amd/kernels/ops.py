@@ -27,6 +27,7 @@ LIBRARY_GEMM_WORKSPACE = 128 << 20   # bytes of scratch memory that the library 
 PREFILL_MAX_PAGES = 2048      # page ids of one group that the prompt-portion attention kernel keeps in LDS
 TILES_MAX_HEAD_DIM = 128      # the 32x32-tile kernel for prompt portions keeps two sets of accumulators per lane
 TILES_COLUMNS = (128, 64)     # (token, head) columns of one of its workgroups: the usual and the small one
+TILES_PAIRING = {"auto": 0, "single": 1, "pairs": 2}
 MFMA_MAX_PAGES = 4096         # page ids of one key range that the single-token attention kernel keeps in LDS
 MAX_KEY_SPLITS = 1024         # the merge of key splits keeps one weight per split in LDS
 
@@ -601,14 +602,17 @@ class Kernels:
     @timed("attention")
     def attention_tiles(self, q, k_pages, v_pages, block_table, slots, positions, out, group_row0, group_ntok,
                         groups, q_heads, kv_heads, head_dim, page_size, scale, window=None, max_context=None,
-                        columns=TILES_COLUMNS[0], split_keys=0, max_splits=1, partial=None):
+                        columns=TILES_COLUMNS[0], split_keys=0, max_splits=1, partial=None, pairing="auto"):
         """Attention for prompt portions: groups of up to columns // (q_heads // kv_heads) consecutive rows
         of one request each (columns = 128, or 64 for batches that would not fill the GPU with the larger
         workgroups); keys and values of a group are staged once through LDS in blocks of 64.  With
         max_splits > 1 a group's keys are split over workgroups in ranges of split_keys (a multiple of 64)
-        and merged through `partial`.  The caller vouches for the groups (consecutive rows of one request,
+        and merged through `partial`.  `pairing`: whether a workgroup of 128 columns (without splits) takes two
+        groups, an early and a late one of a prompt, which evens out their key ranges: "auto" unless that would
+        leave compute units idle, "single" never, "pairs" always.  The caller vouches for the groups (consecutive rows of one request,
         no more tokens than `tiles_group_tokens`)."""
         _need(columns in TILES_COLUMNS, lambda: f"attention_tiles: columns must be one of {TILES_COLUMNS}")
+        _need(pairing in TILES_PAIRING, lambda: f"attention_tiles: pairing must be one of {sorted(TILES_PAIRING)}")
         _need(self.tiles_attention_supported(q_heads, kv_heads, head_dim, page_size, num_pages=k_pages.shape[0]),
               "attention_tiles: sizes not supported")
         _tensor(q, "q", self.dtype, ndim=2)
@@ -640,7 +644,7 @@ class Kernels:
                _p(positions), _p(out), _p(group_row0), _p(group_ntok), _c_int(groups), _c_int(columns),
                _c_int(q_heads), _c_int(kv_heads), _c_int(head_dim), _c_int(page_size), _c_int(k_pages.shape[0]),
                _c_int(window or 0), _c_float(scale), _c_int(split_keys), _c_int(max_splits), _p(partial),
-               _stream()), "attention_tiles")
+               _c_int(TILES_PAIRING[pairing]), _stream()), "attention_tiles")
 
     # -- sampling ----------------------------------------------------------------------------
     def sample_scratch(self, rows):

@@ -216,9 +216,9 @@ class GqaAttention:
             # (with key splits the 32x32-tile kernel takes any context length)
             tiles = k.tiles_attention_supported(*sizes, max_context=ctx.max_context, num_pages=view.k_pages.shape[0],
                                                 split_keys=ctx.split_keys)
-            # workgroups of 128 columns (launched in pairs) unless they would leave half of the compute
-            # units idle: then of 64
-            columns = 128 if m * s.q_heads > 128 * ctx.compute_units else 64
+            # workgroups of 128 columns (half the loads and LDS writes a column of those of 64) when the batch
+            # brings at least one of them for every compute unit: else of 64
+            columns = 128 if m * s.q_heads >= 128 * ctx.compute_units else 64
             big_factor = (columns // 16 if tiles
                           else 4 if k.prefill_attention_supported(*sizes, ctx.max_context) else 0)
             small, big, small_rows = ctx.token_groups(tq, big_factor)

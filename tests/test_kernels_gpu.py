@@ -499,9 +499,11 @@ def test_paged_attention(dtype, case):
         return
     # the 32x32-tile kernel for prompt portions, with both sizes of workgroup: groups of as many tokens as a
     # workgroup takes, and of fewer
-    for columns, big, split in ((128, k.tiles_group_tokens(hq, hkv, 128), 0), (128, 8 * tq, 0),
-                                (64, k.tiles_group_tokens(hq, hkv, 64), 0), (64, 3 * tq, 0),
-                                (128, k.tiles_group_tokens(hq, hkv, 128), 64), (64, 3 * tq, 128)):
+    # (workgroups of 128 columns that take two groups each, and one: small batches would only meet the latter)
+    for columns, big, split, pairing in ((128, k.tiles_group_tokens(hq, hkv, 128), 0, "pairs"), (128, 8 * tq, 0, "pairs"),
+                                         (128, 8 * tq, 0, "single"),
+                                         (64, k.tiles_group_tokens(hq, hkv, 64), 0, "auto"), (64, 3 * tq, 0, "auto"),
+                                         (128, k.tiles_group_tokens(hq, hkv, 128), 64, "auto"), (64, 3 * tq, 128, "auto")):
         first = list(range(0, lengths[0], big))
         count = [min(big, lengths[0] - r) for r in first]
         out4 = torch.full((m, hq * d), float("nan"), dtype=dtype, device="cuda")
@@ -512,7 +514,7 @@ def test_paged_attention(dtype, case):
         k.attention_tiles(q.view(m, hq * d).cuda(), k_pages.cuda(), v_pages.cuda(), table.cuda(), slots, pos, out4,
                           torch.tensor(first, dtype=torch.int32).cuda(), torch.tensor(count, dtype=torch.int32).cuda(),
                           len(first), hq, hkv, d, page, scale, window=window, columns=columns,
-                          split_keys=split, max_splits=splits, partial=part)
+                          split_keys=split, max_splits=splits, partial=part, pairing=pairing)
         got = out4.double().cpu().view(m, hq, d)
         for i in range(lengths[0]):
             torch.testing.assert_close(got[i], wants[i], **tol(dtype))
