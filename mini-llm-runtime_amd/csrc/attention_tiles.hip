@@ -15,7 +15,8 @@
 // for a group) takes as long as this one.  Counted per tile at long contexts: 128 vector instructions (a
 // dependent one issues every 9 cycles, independent ones every 6, an exponential every 10-13), 16 matrix
 // instructions (512 cycles), 47 scalar ones, 16 reads and 8 writes of 16 bytes a lane through the LDS (24 KB;
-// a wavefront's read takes 31 cycles) -- which add up rather than overlap.  So the loop counts its
+// a wavefront's read takes 31 cycles) -- which add up rather than overlap (taking the softmax, the matrix
+// instructions or the staging out of the kernel shortens it by each one's own time).  So the loop counts its
 // instructions: offsets that do not change are computed once, a thread stages 32 contiguous bytes per page
 // lookup, blocks whose keys are all written are staged without checks, the maximum of a tile is taken three
 // values at a time.
