@@ -37,6 +37,8 @@
 // end does not depend on the reference): raising it means rescaling 64 accumulators, and with 32 columns
 // in a wavefront some column would need it in nearly every tile otherwise.  The decision is taken per
 // column from the column's own scores, so a column's arithmetic does not depend on its neighbours.
+// The sum of a column's probabilities is taken over their bfloat16 roundings, the values that the second
+// product multiplies.
 //
 // Key splits (max_splits > 1), for a step whose groups alone would not fill the GPU (a short portion of a
 // long context): workgroup (group, kv head, split s) takes the keys [s * split_keys, (s + 1) * split_keys),
@@ -50,6 +52,7 @@
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;
+typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
 
 #define BLOCK_KEYS 64
@@ -316,15 +319,18 @@ __device__ __forceinline__ void tile_group(const TileArgs& a, int grp, int kvh, 
             }
         }
         const float m_use = fmaxf(m_ref, -1e30f);       // a column with no key yet: exp2(-inf - finite) = 0, not NaN
+        // (the sum is taken over the probabilities as the second product sees them, rounded to bfloat16, two
+        // at a time: v_dot2c_f32_bf16 with a pair of ones, half the instructions of single additions)
+        const bf16x2 ones = {(__bf16)1.0f, (__bf16)1.0f};
         float psum = 0.f;
 #pragma unroll
-        for (int m = 0; m < 2; ++m)
+        for (int m = 0; m < 2; ++m) {
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const float p = __builtin_amdgcn_exp2f(fmaf(sc[8 * m + e], c2, -m_use));
-                psum += p;
-                pf[m][e] = (__bf16)p;
-            }
+            for (int e = 0; e < 8; ++e) pf[m][e] = (__bf16)__builtin_amdgcn_exp2f(fmaf(sc[8 * m + e], c2, -m_use));
+#pragma unroll
+            for (int e = 0; e < 8; e += 2)
+                psum = __builtin_amdgcn_fdot2_f32_bf16(bf16x2{pf[m][e], pf[m][e + 1]}, ones, psum, false);
+        }
         l_run += psum;
     };
 
