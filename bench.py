@@ -4,14 +4,19 @@
 
 A "step" is one decode step of the whole batch: one token per request through the engine's step function
 and the greedy sampler.  Requests are first filled by real prefill (portions of 2048 tokens) so that the
-timed steps end at the context length.  One JSON line is printed:
+timed steps end at the context length.  The model of the default size is a random-weights model folder that is
+written and loaded like any other (the larger ones are drawn on the GPU: the same tensors without a file of
+many gigabytes).  Every runner is built with the product's own defaults.  One JSON line is printed:
 
   * value / ms_per_step / roofline: decode at --batch (8) of the --size (0.6b) model, with the step's share of
     the HBM roofline (bytes it has to read: every weight once and the live requests' cache; 8 TB/s);
-  * points: the same at batch 1 and 64;  prefill: 2048 tokens in one step, with its share of the MFMA peak;
-  * with the default size, a block "8b": decode at batch 1, 8 and 64, prefill and a mixed step (64 decoding
-    requests beside a 2048-token prompt portion in ONE step) at the Qwen3-8B sizes, each with its share of
-    its roofline.  `--size 32b --only mixed` measures the mixed step at the 32B sizes.
+  * points: the same at batch 1 and 64, and at batch 8 behind contexts of 1024, 8192 and 32768 tokens;
+    prefill: 2048 tokens in one step (the median of several; the fastest beside it), with its share of the
+    MFMA peak;
+  * with the default size, a block "8b" and a block "32b": decode at batch 64, 8 and 1, the prefill and a mixed
+    step (64 decoding requests beside a 2048-token prompt portion in ONE step) at those sizes, each with its
+    share of its roofline; the 64 requests of a block are filled once and serve all of its measurements.
+    `--size 32b --only mixed` measures the mixed step alone.
   * --profile: time per kernel class (event pairs around every launch, steps run eagerly) beside the line.
 """
 import argparse
@@ -55,19 +60,31 @@ class Bench:
         self.full_layers, sizes = SIZES[size]
         self.layers = layers if layers > 0 else self.full_layers
         self.cfg = c = config_from_dict(dict(sizes, architectures=["Qwen3ForCausalLM"], num_hidden_layers=self.layers))
-        # Random weights N(0, 0.02) (norm weights 1 + N(0, 0.1)) drawn on the GPU: the same tensors that the
-        # random-weights mode would write to a model folder, without the trip through a file of many gigabytes.
-        torch.manual_seed(0)
-        weights = {}
-        for name, spec in expected_tensors(c).items():
-            if spec.optional:
-                continue
-            if spec.keep_float32:
-                weights[name] = 1.0 + 0.1 * torch.randn(spec.shape, device="cuda", dtype=torch.float32)
-            else:
-                weights[name] = torch.randn(spec.shape, device="cuda", dtype=self.dtype).mul_(0.02)
-        self.model = DecoderModel(c, weights, self.dtype, "cuda:0")
-        del weights
+        if args.weights == "folder" or (args.weights == "auto" and size == "0.6b"):
+            # the product's way: a random-weights model folder (N(0, 0.02), norm weights 1 + N(0, 0.1)), written
+            # and loaded like any model folder, through the planned arena and its budget gate
+            import shutil
+            import tempfile
+            from mini_llm_runtime_amd.weights import write_random_model
+            base = "/dev/shm" if os.path.isdir("/dev/shm") and shutil.disk_usage("/dev/shm").free > (8 << 30) else None
+            with tempfile.TemporaryDirectory(prefix="mlr-bench-", dir=base) as folder:
+                write_random_model(folder, c, seed=0)
+                self.model = DecoderModel.load(folder, self.dtype, "cuda:0", device_budget_bytes=0)
+            self.weights_from = "model folder"
+        else:
+            # the same tensors drawn on the GPU, without the trip through a file of many gigabytes
+            torch.manual_seed(0)
+            weights = {}
+            for name, spec in expected_tensors(c).items():
+                if spec.optional:
+                    continue
+                if spec.keep_float32:
+                    weights[name] = 1.0 + 0.1 * torch.randn(spec.shape, device="cuda", dtype=torch.float32)
+                else:
+                    weights[name] = torch.randn(spec.shape, device="cuda", dtype=self.dtype).mul_(0.02)
+            self.model = DecoderModel(c, weights, self.dtype, "cuda:0")
+            del weights
+            self.weights_from = "drawn on the GPU"
         self.layer_params = c.hidden_size * (c.num_attention_heads + 2 * c.num_key_value_heads) * c.head_dim \
             + c.num_attention_heads * c.head_dim * c.hidden_size + 3 * c.hidden_size * c.intermediate_size
         self.elem = 2 if self.dtype == torch.bfloat16 else 4
@@ -101,19 +118,20 @@ class Bench:
             for at in range(0, tokens, PREFILL_TOKENS):
                 runner.step([Entry(s, ids[at:at + PREFILL_TOKENS], [])])
 
-    def decode(self, batch, steps, warmup):
+    def decode(self, batch, steps, warmup, context=None):
         """Fill `batch` requests so that warmup + steps decode steps end at the context length; time `steps`.
         Returns (seconds, mean context, profile report or None)."""
         from mini_llm_runtime_amd.engine import Entry
         from mini_llm_runtime_amd.sampling import Sampler
         torch, a, c = self.torch, self.args, self.cfg
-        runner = self.runner(batch, batch * (-(-a.context // 64) * 64), a.context, max(PREFILL_TOKENS, batch))
+        context = context or a.context
+        runner = self.runner(batch, batch * (-(-context // 64) * 64), context, max(PREFILL_TOKENS, batch))
         sampler = Sampler(runner.kernels, runner.device, max_rows=batch)
-        fill = a.context - steps - warmup
+        fill = context - steps - warmup
         assert fill >= 1
         # (part of the set-up, like compiling: the decoding step of this batch and context is captured before the
         # requests exist, so that the timed steps are replays whatever --warmup is)
-        runner.warm_up(batch_sizes=[batch], contexts=[a.context])
+        runner.warm_up(batch_sizes=[batch], contexts=[context])
         slots = [runner.open_request() for _ in range(batch)]
         self.fill(runner, slots, fill)
         tokens = torch.randint(0, c.vocab_size, (batch,), generator=self.g).tolist()
@@ -136,11 +154,11 @@ class Bench:
             runner.close_request(s)
         del runner, sampler
         torch.cuda.empty_cache()
-        return seconds, a.context - steps / 2.0, report
+        return seconds, context - steps / 2.0, report
 
-    def decode_point(self, batch, steps, warmup):
+    def decode_point(self, batch, steps, warmup, context=None):
         """{tok_s, ms, frac}: decoded tokens a second, milliseconds a step, share of the HBM roofline."""
-        seconds, mean_context, report = self.decode(batch, steps, warmup)
+        seconds, mean_context, report = self.decode(batch, steps, warmup, context)
         step_bytes = self.weight_bytes + batch * mean_context * self.kv_bytes_per_token
         out = dict(tok_s=round(batch * steps / seconds, 1), ms=round(seconds / steps * 1e3, 4),
                    frac=round(step_bytes / (seconds / steps) / HBM_PEAK, 5))
@@ -149,8 +167,9 @@ class Bench:
     def prefill(self):
         from mini_llm_runtime_amd.engine import Entry
         torch, a, c = self.torch, self.args, self.cfg
-        runner = self.runner(1, PREFILL_TOKENS, PREFILL_TOKENS, PREFILL_TOKENS,
-                             graph_max_tokens=PREFILL_TOKENS if a.prefill_graph and not a.profile else 512)
+        # (the product's defaults: a step of this many tokens is not captured as a graph unless --prefill-graph 1)
+        extra = dict(graph_max_tokens=PREFILL_TOKENS) if a.prefill_graph and not a.profile else {}
+        runner = self.runner(1, PREFILL_TOKENS, PREFILL_TOKENS, PREFILL_TOKENS, **extra)
         ids = torch.randint(0, c.vocab_size, (PREFILL_TOKENS,), generator=self.g).tolist()
         times = []
         for i in range(a.prefill_reps):
@@ -163,13 +182,13 @@ class Bench:
             torch.cuda.synchronize()
             times.append(time.perf_counter() - t0)
             runner.close_request(s)
-        seconds = min(times[1:])
+        seconds = statistics.median(times[1:])         # what a request meets; the fastest run beside it
         t = PREFILL_TOKENS
         flops = 2.0 * t * self.layers * self.layer_params \
             + 2.0 * t * t * c.num_attention_heads * c.head_dim * self.layers \
             + 2.0 * c.vocab_size * c.hidden_size
         out = dict(value=round(t / seconds, 1), tokens=t, ms=round(seconds * 1e3, 3),
-                   ms_median=round(statistics.median(times[1:]) * 1e3, 3),
+                   ms_best=round(min(times[1:]) * 1e3, 3),
                    frac=round(flops / seconds / MFMA_PEAK[self.tag], 5))
         report = runner.profile_report()
         if report is not None:
@@ -187,7 +206,7 @@ class Bench:
         torch, a, c = self.torch, self.args, self.cfg
         total = a.context
         reps = 10 if total <= 2 * portion else 2
-        runner = self.runner(1, total, total, portion, graph_max_tokens=portion if a.prefill_graph else 512)
+        runner = self.runner(1, total, total, portion, **(dict(graph_max_tokens=portion) if a.prefill_graph else {}))
         ids = torch.randint(0, c.vocab_size, (total,), generator=self.g).tolist()
         best = None
         for _ in range(reps):
@@ -262,6 +281,77 @@ class Bench:
         torch.cuda.empty_cache()
         return out
 
+    def block(self, steps, warmup, reps=6):
+        """Decode at batch 64, 8 and 1 and the mixed step on ONE runner whose 64 requests are filled once, by real
+        prefill, and serve every measurement (a large model's prompts are its longest set-up).  Each decode
+        point: tokens a second, milliseconds a step and the share of the HBM roofline at the contexts its
+        requests had meanwhile."""
+        from mini_llm_runtime_amd.engine import Entry
+        from mini_llm_runtime_amd.sampling import Sampler
+        torch, a, c = self.torch, self.args, self.cfg
+        decoding = 64
+        ctx_tokens = -(-a.context // 64) * 64
+        runner = self.runner(decoding + 1, decoding * ctx_tokens + PREFILL_TOKENS, a.context, PREFILL_TOKENS + decoding)
+        sampler = Sampler(runner.kernels, runner.device, max_rows=decoding)
+        runner.warm_up(batch_sizes=[1, 8, decoding], contexts=[a.context])
+        slots = [runner.open_request() for _ in range(decoding)]
+        fill = a.context - 3 * (steps + warmup) - (reps + 1)     # the first request decodes in every measurement
+        assert fill >= 1
+        self.fill(runner, slots, fill)
+        out = {"layers": self.layers}
+        for batch in (decoding, 8, 1):
+            live = slots[:batch]
+            tokens = torch.randint(0, c.vocab_size, (batch,), generator=self.g).tolist()
+            zeros = [0.0] * batch
+
+            def one(tokens):
+                logits = runner.step([Entry(s, [t], [0]) for s, t in zip(live, tokens)])
+                return sampler.sample(logits, zeros, zeros)
+            for _ in range(warmup):
+                tokens = one(tokens)
+            before = sum(runner.length(s) for s in live) / batch
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                tokens = one(tokens)
+            torch.cuda.synchronize()
+            seconds = time.perf_counter() - t0
+            step_bytes = self.weight_bytes + batch * (before + steps / 2.0) * self.kv_bytes_per_token
+            out[f"decode_b{batch}"] = round(batch * steps / seconds, 1)
+            out[f"ms_b{batch}"] = round(seconds / steps * 1e3, 4)
+            out[f"frac_b{batch}"] = round(step_bytes / (seconds / steps) / HBM_PEAK, 5)
+        # the mixed step: every request brings one token, beside them a portion of 2048 tokens of a new prompt
+        ids = torch.randint(0, c.vocab_size, (PREFILL_TOKENS,), generator=self.g).tolist()
+        tokens = torch.randint(0, c.vocab_size, (decoding,), generator=self.g).tolist()
+        zeros = [0.0] * decoding
+        times = []
+        context = sum(runner.length(s) for s in slots) / decoding
+        for i in range(reps + 1):
+            prompt = runner.open_request()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            logits = runner.step([Entry(s, [t], [0]) for s, t in zip(slots, tokens)] + [Entry(prompt, ids, [])])
+            tokens = sampler.sample(logits, zeros, zeros)
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t0)
+            runner.close_request(prompt)
+        times = times[1:]
+        t, hq, d = PREFILL_TOKENS, c.num_attention_heads, c.head_dim
+        context += (reps + 1) / 2.0
+        step_bytes = self.weight_bytes + (decoding * context + t) * self.kv_bytes_per_token
+        flops = 2.0 * (t + decoding) * self.layers * self.layer_params \
+            + (2.0 * t * t + 4.0 * decoding * context) * hq * d * self.layers + 2.0 * decoding * c.vocab_size * c.hidden_size
+        floor = max(step_bytes / HBM_PEAK, flops / MFMA_PEAK[self.tag])
+        seconds = statistics.median(times)
+        out.update(mixed_ms=round(seconds * 1e3, 3), mixed_floor_ms=round(floor * 1e3, 3), mixed_frac=round(floor / seconds, 5),
+                   mixed_bound="mfma" if flops / MFMA_PEAK[self.tag] > step_bytes / HBM_PEAK else "hbm",
+                   mixed_tok_s=round((t + decoding) / seconds, 1))
+        for s in slots:
+            runner.close_request(s)
+        del runner, sampler
+        torch.cuda.empty_cache()
+        return out
+
     def engine_burst(self):
         from mini_llm_runtime_amd.engine import Engine, EngineOptions
         torch, a, c = self.torch, self.args, self.cfg
@@ -311,6 +401,10 @@ def main():
                     help="tuning aid: workgroups that the split of a token's keys aims for")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points, the prefill and the 8B block")
     ap.add_argument("--no-8b", action="store_true", help="skip the block of 8B measurements in the default run")
+    ap.add_argument("--no-32b", action="store_true", help="skip the block of 32B measurements in the default run")
+    ap.add_argument("--weights", default="auto", choices=["auto", "folder", "gpu"],
+                    help="folder: a random-weights model folder, written and loaded like any other; gpu: the same "
+                         "tensors drawn on the GPU; auto: folder for the 0.6B sizes, gpu for the larger ones")
     ap.add_argument("--warm-up", type=int, default=0,
                     help="--only engine: 1 captures the decoding steps (Engine.warm_up) before the first burst")
     ap.add_argument("--only", default="all", choices=["all", "decode", "prefill", "prompt", "engine", "mixed"],
@@ -323,9 +417,10 @@ def main():
     ap.add_argument("--split-keys", type=int, default=256, help="the smallest range of keys of one attention workgroup")
     ap.add_argument("--tune", type=int, default=1,
                     help="0: the vendor library's first candidate for every shape, none timed (the engine's default is 1)")
-    ap.add_argument("--prefill-graph", type=int, default=1,
-                    help="1: the prefill step may be captured as a graph once its shape has come often enough")
-    ap.add_argument("--prefill-reps", type=int, default=10, help="prefill steps; the fastest but the first counts")
+    ap.add_argument("--prefill-graph", type=int, default=0,
+                    help="1: the prefill step may be captured as a graph once its shape has come often enough (the "
+                         "product's default keeps steps of more than 512 tokens eager)")
+    ap.add_argument("--prefill-reps", type=int, default=10, help="prefill steps; the median of all but the first counts")
     ap.add_argument("--fill", default="prefill", choices=["prefill", "random"],
                     help="how the requests' caches are filled before the timed steps: by real prefill "
                          "(default) or, as a profiling aid, with random keys and values")
@@ -372,34 +467,38 @@ def main():
                    "sampling": "greedy", "parallelism": "single GPU"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                      "frac": round(achieved * 1e9 / HBM_PEAK, 5)},
-        "library_tuning": bool(args.tune),
+        "library_tuning": bool(args.tune), "weights": bench.weights_from,
     }
     if report is not None:
         line["profile"] = report
     if not args.no_points and args.only == "all":
         line["prefill"] = bench.prefill()
         points = {}
+        few = (max(8, args.steps // 2), max(2, args.warmup // 2))
         for batch in (1, 64):
-            p, _, _ = bench.decode_point(batch, max(8, args.steps // 2), max(2, args.warmup // 2))
+            p, _, _ = bench.decode_point(batch, *few)
             points[f"decode_b{batch}"] = p["tok_s"]
             points[f"frac_b{batch}"] = p["frac"]
+        for context in (1024, 8192, 32768):              # the same batch behind shorter and longer contexts
+            if context <= c.max_position_embeddings:
+                p, _, _ = bench.decode_point(args.batch, *few, context=context)
+                points[f"decode_b{args.batch}_ctx{context}"] = p["tok_s"]
+                points[f"frac_b{args.batch}_ctx{context}"] = p["frac"]
         line["points"] = points
-        if args.size == "0.6b" and not args.no_8b and args.layers <= 0:
-            # the other half of the headline metric: the same measurements at the Qwen3-8B sizes (all 36 layers)
+        if args.size == "0.6b" and args.layers <= 0:
+            # the other sizes the metric names: the same measurements at the Qwen3-8B and the Qwen3-32B sizes
+            # (all 36 and all 64 layers)
             bench.close()
-            big = Bench("8b", 0, args)
-            block = {"layers": big.layers}
-            for batch in (1, 8, 64):
-                p, _, _ = big.decode_point(batch, max(8, args.steps // 2), max(2, args.warmup // 2))
-                block[f"decode_b{batch}"] = p["tok_s"]
-                block[f"ms_b{batch}"] = p["ms"]
-                block[f"frac_b{batch}"] = p["frac"]
-            pre = big.prefill()
-            block.update(prefill_tok_s=pre["value"], prefill_ms=pre["ms"], prefill_frac=pre["frac"])
-            mixed = big.mixed()
-            block.update(mixed_ms=mixed["ms"], mixed_floor_ms=mixed["floor_ms"], mixed_frac=mixed["frac"],
-                         mixed_bound=mixed["bound"], mixed_tok_s=mixed["tok_s"])
-            line["8b"] = block
+            for size, skip in (("8b", args.no_8b), ("32b", args.no_32b)):
+                if skip:
+                    continue
+                big = Bench(size, 0, args)
+                block = big.block(*few)
+                pre = big.prefill()
+                block.update(prefill_tok_s=pre["value"], prefill_ms=pre["ms"], prefill_frac=pre["frac"])
+                line[size] = block
+                big.close()
+                del big
     print(json.dumps(line))
     return 0
 

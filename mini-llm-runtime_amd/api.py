@@ -32,17 +32,20 @@ class LLM:
     def __init__(self, model, dtype="bfloat16", device="cuda:0", options: EngineOptions = None, **overrides):
         """`model`: a folder with config.json and model.safetensors.  `overrides` set single
         fields of EngineOptions (context_tokens, max_model_len, max_active, batch_tokens,
-        prefill_chunk, block_size, policy, ...)."""
+        prefill_chunk, block_size, policy, kv_dtype, device_budget_bytes, ...).  Left alone, the options
+        come from the model and the device: requests as long as the model's positions allow, a page pool
+        as large as the device's budget leaves room for, prompts in portions of 2048 tokens."""
+        from dataclasses import replace
         self.dtype = parse_dtype(dtype)
         self.folder = model
         self._tokenizer = None
-        self.model = DecoderModel.load(model, self.dtype, device)
-        opts = options or EngineOptions()
+        opts = replace(options) if options is not None else EngineOptions()
         for key, value in overrides.items():
             if not hasattr(opts, key):
                 raise ValueError(f"unknown engine option {key!r}")
             setattr(opts, key, value)
-        opts.max_model_len = min(opts.max_model_len, self.model.spec.max_positions)
+        # the same budget gates the weights and, in the engine, the cache and the scratch buffers
+        self.model = DecoderModel.load(model, self.dtype, device, device_budget_bytes=opts.device_budget_bytes)
         self.engine = Engine(self.model, opts)
 
     @property

@@ -290,6 +290,29 @@ class CacheManager:
             tables += (max_slots + 1) * ((max_length + size - 1) // size) * 4
         return kv, tables, state
 
+    @staticmethod
+    def tokens_that_fit(entry_specs, dtype, page_size, max_slots, max_length, budget_bytes):
+        """The largest pool (in tokens: a multiple of every group's page size) whose pages, tables and state fit
+        `budget_bytes`, at most what `max_slots` requests of `max_length` tokens can hold; 0 when not even one
+        unit fits.  What the reference calls kv_capacity_tokens (include/minillm/cuda/runtime.h:28), here derived
+        from the budget instead of asked of the user."""
+        import math
+        unit = 1
+        for spec in entry_specs:
+            paged = _as_paged(spec)
+            if paged is not None:
+                size = paged.page_size or page_size
+                unit = unit * size // math.gcd(unit, size)
+        most = max_slots * (-(-max_length // unit))          # units that the slots can hold at all
+        fits = lambda units: sum(CacheManager.plan(entry_specs, dtype, page_size, units * unit, max_slots, max_length)) <= budget_bytes
+        if fits(most):
+            return most * unit
+        lo, hi = 0, most                                     # fits(lo) (or lo == 0), not fits(hi)
+        while hi - lo > 1:
+            mid = (lo + hi) // 2
+            lo, hi = (mid, hi) if fits(mid) else (lo, mid)
+        return lo * unit if lo > 0 and fits(lo) else 0
+
     def __init__(self, entry_specs, dtype, device, page_size, max_tokens, max_slots, max_length):
         if page_size <= 0 or max_tokens <= 0:
             raise CacheError("page_size and max_tokens must be positive")

@@ -25,8 +25,8 @@ from .options import Option, OptionError, parse
 
 USAGE = """mini-llm (--model DIR | --random-weights CONFIG.json [--seed 0])
          (--prompt-ids 1,2,3 | --prompt TEXT | --prompts-file FILE) [--tokenizer tokenizer.json|DIR]
-         [--tokens 32] [--context 2048] [--batch 128] [--chunk 128] [--sequences 4]
-         [--dtype bfloat16|float32] [--temperature 0] [--sample-seed 0] [--page-size 16]
+         [--tokens 32] [--context MODEL'S] [--batch 2048] [--chunk BATCH] [--sequences 4]
+         [--dtype bfloat16|float32] [--kv-dtype auto] [--temperature 0] [--sample-seed 0] [--page-size 16]
          [--policy mixed|prefill_first] [--device 0] [--device-budget-bytes 0] [--ignore-eos]
          [--device-time] [--profile] [--check-finite] [--output NEW_REPORT.json]
          [--cuda-precision f32-pedantic] [--kv-layout paged]
@@ -38,12 +38,12 @@ TABLE = [
     Option("--device-time", "switch"), Option("--profile", "switch"), Option("--check-finite", "switch"),
     Option("--model"), Option("--random-weights"), Option("--output"), Option("--prompts-file"),
     Option("--prompt"), Option("--tokenizer"),
-    Option("--dtype", default="bfloat16"), Option("--policy", default="mixed"),
+    Option("--dtype", default="bfloat16"), Option("--policy", default="mixed"), Option("--kv-dtype", default="auto"),
     Option("--cuda-precision"), Option("--kv-layout", default="paged"),
     Option("--prompt-ids", "ints", default=[]),
     Option("--seed", "int", 0, 0, 2 ** 63 - 1), Option("--sample-seed", "int", 0, 0, 2 ** 63 - 1),
-    Option("--tokens", "int", 32, 1, 4096), Option("--context", "int", 2048, 1, 2 ** 31 - 1),
-    Option("--batch", "int", 128, 1, 2 ** 20), Option("--chunk", "int", None, 1, 2 ** 20),
+    Option("--tokens", "int", 32, 1, 4096), Option("--context", "int", None, 1, 2 ** 31 - 1),
+    Option("--batch", "int", 2048, 1, 2 ** 20), Option("--chunk", "int", None, 1, 2 ** 20),
     Option("--sequences", "int", 4, 1, 4096), Option("--page-size", "int", 16, 1, 1024),
     Option("--device", "int", 0, 0, 2 ** 31 - 1), Option("--device-budget-bytes", "int", 0, 0, 2 ** 63 - 1),
     Option("--temperature", "float", 0.0, 0.0, 1e6),
@@ -226,6 +226,8 @@ def main(argv=None):
                 raise OptionError("--cuda-precision f32-pedantic contradicts --dtype")
         if opts["--policy"] not in ("mixed", "prefill_first"):
             raise OptionError("--policy: mixed or prefill_first")
+        if opts["--kv-dtype"] not in ("auto", "bfloat16", "float32"):
+            raise OptionError("--kv-dtype: auto, bfloat16 or float32 (the engine's own element type)")
 
         import torch
         from .api import parse_dtype
@@ -256,8 +258,13 @@ def main(argv=None):
                                       model.spec.eos_token_ids)
             except TokenizerError as error:
                 raise OptionError(str(error)) from None
-        limit = min(context, model.spec.max_positions)
-        pool = sequences * ((limit + page - 1) // page) * page
+        # --context left out: requests as long as the model's positions allow, and a pool as large as the
+        # device's budget leaves room for (at most that of --sequences such requests); given: the reference's
+        # pool of --sequences x --context tokens (apps/cuda_main.cpp:60-69 sizes its cache so)
+        limit = min(context, model.spec.max_positions) if context is not None else model.spec.max_positions
+        pool = sequences * ((limit + page - 1) // page) * page if context is not None else None
+        batch = min(batch, limit)
+        chunk = min(chunk, batch)
         common = {"backend": "mini-llm-runtime_amd", "dtype": str(dtype).replace("torch.", "")}
         try:
             if opts.given("--prompts-file"):
@@ -267,7 +274,8 @@ def main(argv=None):
                         raise OptionError("a prompt and its output tokens exceed the context")
                 engine = Engine(model, EngineOptions(
                     context_tokens=pool, max_model_len=limit, max_active=sequences, batch_tokens=max(batch, sequences),
-                    prefill_chunk=min(chunk, max(batch, sequences)), block_size=page, policy=opts["--policy"]),
+                    prefill_chunk=min(chunk, max(batch, sequences)), block_size=page, policy=opts["--policy"],
+                    kv_dtype=opts["--kv-dtype"]),
                     device_budget_bytes=budget, check_finite=opts["--check-finite"], profile=opts["--profile"])
                 runner = engine.runner
                 report = many_requests(opts, engine, prompts, count, tokenizer)
@@ -284,7 +292,7 @@ def main(argv=None):
                     raise OptionError("prompt and the output tokens written to the cache exceed the context")
                 runner = Runner(model, max_tokens=pool, max_slots=sequences, max_length=limit, max_batch_tokens=batch,
                                 page_size=page, device_budget_bytes=budget, check_finite=opts["--check-finite"],
-                                profile=opts["--profile"])
+                                profile=opts["--profile"], kv_dtype=opts["--kv-dtype"])
                 sampler = Sampler(runner.kernels, runner.device, max_rows=1)
                 report = one_sequence(opts, model, runner, sampler, prompt, count, chunk, tokenizer)
         except MemoryBudgetError as error:

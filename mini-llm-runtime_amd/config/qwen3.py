@@ -180,8 +180,8 @@ class Qwen3Config:
     # ---- tensor names (src/minillm/qwen3_model.cpp:59-78, under their safetensors names) --
     @staticmethod
     def global_tensor_name(local):
-        return {"embed": "model.embed_tokens.weight", "final_norm.weight": "model.norm.weight",
-                "lm_head": "lm_head.weight"}[local]
+        return {"embed.weight": "model.embed_tokens.weight", "final_norm.weight": "model.norm.weight",
+                "head.weight": "lm_head.weight"}[local]
 
     @staticmethod
     def layer_tensor_name(layer, part, local):

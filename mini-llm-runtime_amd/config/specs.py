@@ -66,6 +66,21 @@ class LayerRun:
 
 
 @dataclass(frozen=True)
+class EmbedSpec:
+    kind: str                 # key in the embed registry, e.g. "token_embedding"
+    vocab_size: int
+    hidden: int
+
+
+@dataclass(frozen=True)
+class HeadSpec:
+    kind: str                 # key in the head registry, e.g. "linear_head"
+    vocab_size: int
+    hidden: int
+    tied: bool = False        # no tensor of its own: the embedding's table
+
+
+@dataclass(frozen=True)
 class ModelSpec:
     architecture: str
     vocab_size: int
@@ -76,3 +91,12 @@ class ModelSpec:
     tie_embeddings: bool
     max_positions: int
     eos_token_ids: Tuple[int, ...] = field(default_factory=tuple)
+    embed: Optional[object] = None      # any embed spec with a `kind`; None: a plain table [vocab_size, hidden]
+    head: Optional[object] = None       # any head spec with a `kind`; None: a plain projection, tied as `tie_embeddings` says
+
+    def embed_spec(self):
+        return self.embed if self.embed is not None else EmbedSpec("token_embedding", self.vocab_size, self.hidden)
+
+    def head_spec(self):
+        return self.head if self.head is not None else HeadSpec("linear_head", self.vocab_size, self.hidden,
+                                                                self.tie_embeddings)

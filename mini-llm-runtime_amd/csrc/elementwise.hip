@@ -18,6 +18,53 @@ __global__ void embed_gather_kernel(const int32_t* __restrict__ ids, const elem_
     for (int i = threadIdx.x; i < width; i += blockDim.x) out[i] = to_float(row[i]);
 }
 
+__device__ __forceinline__ float block_max(float v, float* scratch) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = (blockDim.x + 63) >> 6;
+    v = wave_max(v);
+    __syncthreads();
+    if (lane == 0) scratch[wave] = v;
+    __syncthreads();
+    float total = scratch[0];
+    for (int i = 1; i < waves; ++i) total = fmaxf(total, scratch[i]);
+    return total;
+}
+
+// A row whose sum of squares does not fit 32 bits (elements beyond about 1e19) or is no number: the
+// reference's way of norming (src/minillm/cuda/ops.cu:87-126), the row divided by its largest element before
+// it is squared, and eps scaled alike: largest = max(max |x|, sqrt(eps)), den = sqrt(mean((x / largest)^2) +
+// eps / largest^2), y = ((x / largest) / den) * w; a row with an infinity or a NaN comes out as NaN.  The usual
+// row never gets here, so it keeps its one pass and its bits.  x = hrow + drow (drow: what is still to be
+// added, or null).  WAVE: one wavefront serves the row, else the whole workgroup (every thread of it must
+// call, `scratch` holds 16 floats of LDS).
+template <bool WAVE>
+__device__ void norm_row_rescaled(const float* hrow, const elem_t* drow, const float* __restrict__ weight,
+                                  elem_t* __restrict__ orow, int width, float eps, float* scratch) {
+    __threadfence_block();                     // (the row may have been written back by other lanes just now)
+    const int t = WAVE ? (int)(threadIdx.x & 63) : (int)threadIdx.x, step = WAVE ? 64 : (int)blockDim.x;
+    float largest = 0.f;
+    for (int i = t; i < width; i += step) {
+        const float x = hrow[i] + (drow ? to_float(drow[i]) : 0.f);
+        largest = fmaxf(largest, isfinite(x) ? fabsf(x) : INFINITY);
+    }
+    largest = WAVE ? wave_max(largest) : block_max(largest, scratch);
+    largest = fmaxf(largest, sqrtf(eps));
+    if (!isfinite(largest)) {
+        for (int i = t; i < width; i += step) orow[i] = from_float<elem_t>(__int_as_float(0x7fc00000));
+        return;
+    }
+    float sum = 0.f;
+    for (int i = t; i < width; i += step) {
+        const float scaled = (hrow[i] + (drow ? to_float(drow[i]) : 0.f)) / largest;
+        sum += scaled * scaled;
+    }
+    sum = WAVE ? wave_sum(sum) : block_sum(sum, scratch);
+    const float den = sqrtf(sum / (float)width + (eps / largest) / largest);
+    for (int i = t; i < width; i += step) {
+        const float x = hrow[i] + (drow ? to_float(drow[i]) : 0.f);
+        orow[i] = from_float<elem_t>(((x / largest) / den) * weight[i]);
+    }
+}
+
 // For output row r: src = rows ? rows[r] : r;  x = h[src] + (delta ? delta[src] : 0);
 // if write_h: h[src] = x;  out[r] = (x * rsqrt(mean(x^2) + eps)) * weight.
 // One workgroup per row; the sum of squares is taken over the row in a fixed order.
@@ -40,8 +87,12 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ h, const elem_t* __restri
         sum += x * x;
     }
     sum = block_sum(sum, scratch);
-    const float scale = 1.0f / sqrtf(sum / (float)width + eps);
     elem_t* orow = out + (size_t)r * width;
+    if (!isfinite(sum)) {                      // (the same in every thread of the workgroup)
+        norm_row_rescaled<false>(hrow, (drow && !write_h) ? drow : nullptr, weight, orow, width, eps, scratch);
+        return;
+    }
+    const float scale = 1.0f / sqrtf(sum / (float)width + eps);
     for (int i = threadIdx.x; i < width; i += blockDim.x) {
         float x = hrow[i];
         if (drow && !write_h) x += to_float(drow[i]);
@@ -83,8 +134,12 @@ __global__ __launch_bounds__(256) void add_rmsnorm_row_vec_kernel(float* __restr
         for (int e = 0; e < MLR_VEC; ++e) sum += x[e] * x[e];
     }
     sum = block_sum(sum, scratch);
-    const float scale = 1.0f / sqrtf(sum / (float)width + eps);
     elem_t* orow = out + (size_t)r * width;
+    if (!isfinite(sum)) {
+        norm_row_rescaled<false>(hrow, (drow && !write_h) ? drow : nullptr, weight, orow, width, eps, scratch);
+        return;
+    }
+    const float scale = 1.0f / sqrtf(sum / (float)width + eps);
     for (int c = threadIdx.x * MLR_VEC; c < width; c += 256 * MLR_VEC) {
         float x[MLR_VEC], y[MLR_VEC];
 #pragma unroll
@@ -151,8 +206,12 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
         }
     }
     sum = wave_sum(sum);
-    const float scale = 1.0f / sqrtf(sum / (float)width + eps);
     elem_t* orow = out + (size_t)r * width;
+    if (!isfinite(sum)) {                      // (the same in every lane of the wavefront, which serves this row alone)
+        norm_row_rescaled<true>(hrow, (drow && !write_h) ? drow : nullptr, weight, orow, width, eps, nullptr);
+        return;
+    }
+    const float scale = 1.0f / sqrtf(sum / (float)width + eps);
 #pragma unroll
     for (int i = 0; i < ROW_REGS; ++i) {
         const int c = (lane + 64 * i) * MLR_VEC;

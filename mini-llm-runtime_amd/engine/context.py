@@ -121,6 +121,7 @@ class StepContext:
         self._group_upload = None
         self.fixed_groups = None      # a captured step's groups: {key: token_groups' result}, in tensors of their own
         self.status = None            # device int32 [2] when the hidden state is to be checked after every layer
+        self.partial_budget = None    # floats that split attention's partial results may take (the memory plan's)
 
     def begin_step(self):
         self._groups = {}
@@ -128,10 +129,11 @@ class StepContext:
 
     def token_groups(self, tokens_per_group, big_factor=0):
         """The step's rows cut into groups of consecutive tokens of one request, as device int32 vectors
-        (first row of each group, tokens in each group) with their number.  Returns (small, big, rows in
-        small groups): small groups hold at most `tokens_per_group` tokens; with big_factor > 0, a request
-        that brings more than `tokens_per_group` tokens is cut into big groups of at most big_factor *
-        tokens_per_group instead (prompt portions), else `big` is empty."""
+        (first row of each group, tokens in each group) with their number.  Returns (small, big, (rows in
+        small groups, one beyond the last batch row of a small group)): small groups hold at most
+        `tokens_per_group` tokens; with big_factor > 0, a request that brings more than `tokens_per_group`
+        tokens is cut into big groups of at most big_factor * tokens_per_group instead (prompt portions), else
+        `big` is empty."""
         key = (tokens_per_group, big_factor)
         hit = self._groups.get(key)
         if hit is not None:
@@ -139,7 +141,7 @@ class StepContext:
         if self.fixed_groups is not None and key in self.fixed_groups:
             return self.fixed_groups[key]
         first, count, big_first, big_count = [], [], [], []
-        small_rows = 0
+        small_rows = small_end = 0
         for _, row, n, _ in self.segments:
             if big_factor > 0 and n > tokens_per_group:
                 size = big_factor * tokens_per_group
@@ -148,6 +150,7 @@ class StepContext:
                     big_count.append(min(size, n - i))
             else:
                 small_rows += n
+                small_end = max(small_end, row + n)
                 for i in range(0, n, tokens_per_group):
                     first.append(row + i)
                     count.append(min(tokens_per_group, n - i))
@@ -161,7 +164,8 @@ class StepContext:
             if self._group_upload is None:
                 self._group_upload = Uploader(4096, dev.device)
             self._group_upload.send(first + count + big_first + big_count, dev)
-        hit = ((dev[:g], dev[g:2 * g], g), (dev[2 * g:2 * g + gb], dev[2 * g + gb:2 * g + 2 * gb], gb), small_rows)
+        hit = ((dev[:g], dev[g:2 * g], g), (dev[2 * g:2 * g + gb], dev[2 * g + gb:2 * g + 2 * gb], gb),
+               (small_rows, small_end))
         if self.fixed_groups is not None:
             self.fixed_groups[key] = hit
         self._groups[key] = hit
@@ -187,8 +191,39 @@ class StepContext:
         split; a longer context is split whatever the number of groups."""
         return self._split(max(1, groups * kv_heads), self.compute_units, batch_rows, q_heads, head_dim, longest)
 
+    def fixed_split(self, rows, q_heads, head_dim):
+        """(split_keys, max_splits, rows a launch, partial buffer) for the attention kernel whose results must
+        not depend on the batch by a single bit (the float engine's): a token's keys are always cut into ranges
+        of `split_keys` of the runner's setting, whatever else the step holds, so the sums that make up its
+        result and their order follow from its own position alone.  (A context of more than 1024 ranges
+        doubles their width: the merge kernel's limit.)  The partial results of all rows may exceed what was
+        planned for them; then the rows are served by several launches."""
+        base = self.split_keys
+        if base <= 0 or self.max_context <= base:
+            return 0, 1, rows, None
+        keys = base
+        while -(-self.max_context // keys) > 1024:
+            keys *= 2
+        max_splits = -(-self.max_context // keys)
+        per_row = self.kernels.attention_partial_numel(1, q_heads, head_dim, max_splits)
+        chunk = rows if self.partial_budget is None else max(1, min(rows, self.partial_budget // per_row))
+        return keys, max_splits, chunk, self.workspace.get("attn_partial", (chunk * per_row,), torch.float32)
+
+    @staticmethod
+    def forced_splits(max_length, base, longest):
+        """Key splits that a context of `max_length` needs at least when one workgroup walks at most `longest`
+        keys: ranges of the largest of base, 2 base, 4 base, ... that `longest` holds (1: no split needed)."""
+        if longest is None or max_length <= longest or base <= 0:
+            return 1
+        keys = base
+        while keys * 2 <= longest:
+            keys *= 2
+        return -(-max_length // keys)
+
     def _split(self, units, enough, batch_rows, q_heads, head_dim, longest=None):
-        """`units` workgroups without a split; no split when they are `enough`."""
+        """`units` workgroups without a split; no split when they are `enough`.  The partial results never take
+        more than `partial_budget` floats (when one is set: the runner's memory plan): key ranges are doubled
+        until they fit, which a forced split allows up to `longest`."""
         base = self.split_keys
         forced = longest is not None and self.max_context > longest
         if base <= 0 or (self.max_context <= base and not forced):
@@ -201,6 +236,12 @@ class StepContext:
                 keys //= 2
         elif units >= enough:
             return 0, 1, None
+        budget = self.partial_budget
+        numel = lambda k: self.kernels.attention_partial_numel(batch_rows, q_heads, head_dim, -(-self.max_context // k))
+        while budget is not None and numel(keys) > budget and (not forced or keys * 2 <= longest):
+            if keys >= self.max_context:                 # one range holds every key: no split, nothing to keep
+                return 0, 1, None
+            keys *= 2
         max_splits = -(-self.max_context // keys)
         if max_splits <= 1:
             return 0, 1, None

@@ -99,13 +99,17 @@ def schedule_batch(items, batch_tokens, prefill_chunk, policy="mixed", aging_ms=
 
 @dataclass
 class EngineOptions:
-    """Names and defaults after the reference's EngineConfig (include/llmserve/config.h:15-33)."""
-    context_tokens: int = 8192        # tokens the page pool holds
-    max_model_len: int = 2048         # longest prompt + output of one request
-    max_active: int = 8               # request slots
-    batch_tokens: int = 256           # token budget of one step
-    prefill_chunk: int = 128          # longest portion of one prompt in a step
-    block_size: int = 16              # tokens in a page
+    """Names after the reference's EngineConfig (include/llmserve/config.h:15-33).  Its defaults are the limits
+    of a laptop GPU (a pool of 8192 tokens, 8 slots, steps of 256 tokens, portions of 128); here what is left
+    None is taken from the model and the device when an engine is built (`resolved`): a 2048-token prompt is one
+    step, and the pool is what the device's budget leaves room for."""
+    context_tokens: Optional[int] = None   # tokens the page pool holds; None: what the device's budget leaves room
+                                           # for, at most max_active requests of max_model_len tokens
+    max_model_len: Optional[int] = None    # longest prompt + output of one request; None: the model's positions
+    max_active: int = 64                   # request slots
+    batch_tokens: Optional[int] = None     # token budget of one step; None: prefill_chunk + max_active
+    prefill_chunk: int = 2048              # longest portion of one prompt in a step
+    block_size: int = 16                   # tokens in a page
     aging_ms: int = 250
     admission_reserve_ms: int = 2000
     policy: str = "mixed"
@@ -113,14 +117,38 @@ class EngineOptions:
     portion_step: int = 32            # ours: portions that do not end their prompt are multiples of this, so
                                       # that step shapes come again and are replayed as graphs (0: the
                                       # reference's exact portions)
+    kv_dtype: str = "auto"            # the cache's element type: "auto" or the engine's own
+                                      # (include/minillm/cuda/runtime.h:18-30 has the cache's type and capacity
+                                      # beside the budget; another type than the engine's is refused)
+    device_budget_bytes: Optional[int] = 0   # the user's cap on what the runner may allocate; 0: none beside the rule
+                                             # min(80 % of free memory, free - 512 MiB); None: no gate at all
+
+    def resolved(self, max_positions):
+        """A copy with every None filled in, as far as that needs no device: max_model_len from the model,
+        batch_tokens from the portion and the slots.  context_tokens may stay None (the runner sizes the pool)."""
+        from dataclasses import replace
+        limit = min(self.max_model_len or max_positions, max_positions)
+        if self.max_model_len is None and self.context_tokens is not None:
+            limit = min(limit, self.context_tokens)       # (no request outgrows the pool)
+        chunk = self.prefill_chunk
+        batch = self.batch_tokens
+        if batch is None:
+            batch = chunk + self.max_active
+            if self.context_tokens is not None:
+                batch = max(min(batch, self.context_tokens), self.max_active)
+                chunk = min(chunk, batch)
+        return replace(self, max_model_len=limit, batch_tokens=batch, prefill_chunk=chunk)
 
     def validate(self):
-        """src/config.cpp:8-36."""
-        if self.block_size <= 0 or self.context_tokens <= 0 or self.context_tokens % self.block_size != 0:
+        """src/config.cpp:8-36, on resolved options (context_tokens may still be None)."""
+        if self.max_model_len is None or self.batch_tokens is None:
+            raise ValueError("validate() wants resolved options")
+        pool = self.context_tokens
+        if self.block_size <= 0 or (pool is not None and (pool <= 0 or pool % self.block_size != 0)):
             raise ValueError("context_tokens must be a positive multiple of block_size")
-        if self.max_model_len < 2 or self.max_model_len > self.context_tokens:
+        if self.max_model_len < 2 or (pool is not None and self.max_model_len > pool):
             raise ValueError("max_model_len must be in [2, context_tokens]")
-        if self.max_active <= 0 or self.batch_tokens < self.max_active or self.batch_tokens > self.context_tokens:
+        if self.max_active <= 0 or self.batch_tokens < self.max_active or (pool is not None and self.batch_tokens > pool):
             raise ValueError("require 1 <= max_active <= batch_tokens <= context_tokens")
         if self.prefill_chunk <= 0 or self.prefill_chunk > self.batch_tokens or self.queue_capacity <= 0:
             raise ValueError("invalid prefill or queue limit")
@@ -130,6 +158,10 @@ class EngineOptions:
             raise ValueError(f"policy must be one of {sorted(POLICIES)}")
         if self.portion_step < 0:
             raise ValueError("portion_step must not be negative")
+        if self.kv_dtype not in ("auto", "bfloat16", "float32"):
+            raise ValueError("kv_dtype must be auto, bfloat16 or float32")
+        if self.device_budget_bytes is not None and self.device_budget_bytes < 0:
+            raise ValueError("device_budget_bytes must not be negative")
 
 
 @dataclass
@@ -159,20 +191,25 @@ class Engine:
     """Continuous batching over one `Runner`.  Single-threaded: the caller drives `step()`."""
 
     def __init__(self, model, options: EngineOptions = None, clock=time.monotonic, runner=None, sampler=None,
-                 device_budget_bytes=None, check_finite=False, profile=False):
-        """`device_budget_bytes`, `check_finite`, `profile`: handed to the `Runner` that is built here (see
-        there): the budget gate before the cache is allocated, the check of the hidden state after every
-        layer, time per kernel class."""
-        self.options = options or EngineOptions()
+                 device_budget_bytes="options", check_finite=False, profile=False):
+        """`device_budget_bytes` (default: the options' own), `check_finite`, `profile`: handed to the `Runner`
+        that is built here (see there): the budget gate before the cache is allocated, the check of the hidden
+        state after every layer, time per kernel class."""
+        self.options = (options or EngineOptions()).resolved(model.spec.max_positions)
         self.options.validate()
         o = self.options
+        if device_budget_bytes == "options":
+            device_budget_bytes = o.device_budget_bytes
         self.model = model
         # (a step of the scheduler asks for at most one row of logits per request)
         self.runner = runner or Runner(model, max_tokens=o.context_tokens, max_slots=o.max_active,
-                                       max_length=min(o.max_model_len, model.spec.max_positions),
+                                       max_length=o.max_model_len,
                                        max_batch_tokens=o.batch_tokens, page_size=o.block_size,
                                        max_logits_rows=o.max_active, device_budget_bytes=device_budget_bytes,
-                                       check_finite=check_finite, profile=profile)
+                                       check_finite=check_finite, profile=profile, kv_dtype=o.kv_dtype)
+        if o.context_tokens is None:                      # the pool that the runner sized from the device's budget
+            o.context_tokens = getattr(self.runner, "max_tokens", None) or o.max_active * o.max_model_len
+            o.validate()
         self.sampler = sampler or Sampler(self.runner.kernels, self.runner.device, max_rows=o.max_active)
         self.clock = clock
         # pages are set aside in units that every group of the cache can serve (its page size, when all
@@ -213,7 +250,7 @@ class Engine:
             raise ValueError("prompt holds a token id outside the vocabulary")
         if max_tokens < 1:
             raise ValueError("max_tokens must be at least 1")
-        if len(prompt) + max_tokens > min(o.max_model_len, self.model.spec.max_positions):
+        if len(prompt) + max_tokens > o.max_model_len:
             raise ValueError("prompt + max_tokens exceed max_model_len")
         if self._pages_for(len(prompt) + max_tokens) > self.total_pages:
             raise ValueError("the request does not fit an otherwise idle page pool")

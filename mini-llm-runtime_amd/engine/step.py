@@ -18,7 +18,7 @@ from ..kernels import Kernels
 from ..kernels.ops import LIBRARY_GEMM_WORKSPACE
 from ..kernels.profile import Profiler
 from .context import StepContext, Uploader, Workspace
-from .memory import MemoryPlan
+from .memory import MemoryBudgetError, MemoryPlan, device_budget
 
 
 class StepError(ValueError):
@@ -36,13 +36,27 @@ class Entry:
     want: Sequence[int] = field(default_factory=list)     # places among `tokens` whose logits are asked for
 
 
+def _kv_dtype(name, engine_dtype):
+    if name in (None, "auto") or name == engine_dtype:
+        return engine_dtype
+    names = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32,
+             "f32": torch.float32}
+    if name in names:
+        return names[name]
+    raise ValueError(f"kv_dtype must be auto, bfloat16 or float32, got {name!r}")
+
+
 class Runner:
-    def __init__(self, model, max_tokens, max_slots=4, max_length=None, max_batch_tokens=None,
+    def __init__(self, model, max_tokens=None, max_slots=4, max_length=None, max_batch_tokens=None,
                  page_size=16, split_keys=256, split_max_tokens=256, use_graphs=True, graph_max_batch=256,
                  target_workgroups=512, graph_max_tokens=512, graph_after=4, max_graphs=128, library_gemm=True,
-                 max_logits_rows=None, device_budget_bytes=None, check_finite=False, profile=False):
-        """`max_tokens`: tokens the page pool holds; `max_length`: longest request; `max_batch_tokens`: most
-        tokens of one step; `max_logits_rows`: most wanted places of one step (default: every token).
+                 max_logits_rows=None, device_budget_bytes=None, check_finite=False, profile=False, kv_dtype="auto"):
+        """`max_tokens`: tokens the page pool holds, or None: as many as the device's budget leaves room for
+        beside everything else that is planned, at most what `max_slots` requests of `max_length` tokens hold
+        (the budget is then the rule below also with `device_budget_bytes` None); `max_length`: longest request;
+        `max_batch_tokens`: most tokens of one step; `max_logits_rows`: most wanted places of one step (default:
+        every token).  `kv_dtype`: the cache's element type, "auto" or the engine's own (the attention kernels
+        read the pages as the engine's element type; another one is refused).
         `device_budget_bytes`: None for no gate, else the device memory that the runner will hold is planned and
         compared with min(this cap (0: none), 80 % of the free memory, free - 512 MiB) before the cache is
         allocated (`MemoryBudgetError`).  `check_finite`: after every layer one small kernel looks at the
@@ -66,9 +80,25 @@ class Runner:
         limits = dict(max_length=self.max_length, page_size=page_size, split_keys=split_keys,
                       split_max_tokens=split_max_tokens, target_workgroups=target_workgroups)
         workspace_plan = model.workspace_plan(self.max_batch_tokens, self.max_logits_rows, limits)
+        uses_library = library_gemm and self.dtype == torch.bfloat16
+        if _kv_dtype(kv_dtype, self.dtype) != self.dtype:
+            raise ValueError(f"kv_dtype {kv_dtype}: the {self.dtype} engine's attention kernels read pages of their own "
+                             "element type only")
+        if max_tokens is None:
+            # the pool takes what the budget leaves beside the scratch buffers, the metadata and the library's
+            # scratch (the weights are resident already and no longer part of the free memory)
+            other = MemoryPlan(workspace=Workspace.plan_bytes(workspace_plan), metadata=5 * 4 * self.max_batch_tokens + 8,
+                               library_scratch=LIBRARY_GEMM_WORKSPACE if uses_library else 0).to_allocate()
+            room = device_budget(device_budget_bytes or 0, self.device) - other
+            max_tokens = CacheManager.tokens_that_fit(model.cache_entry_specs, self.dtype, page_size, max_slots,
+                                                      self.max_length, room)
+            if max_tokens <= 0:
+                raise MemoryBudgetError(f"the device's budget leaves {room} bytes for the cache: not one page a group")
+            if device_budget_bytes is None:
+                device_budget_bytes = 0
+        self.max_tokens = max_tokens
         kv, tables, state = CacheManager.plan(model.cache_entry_specs, self.dtype, page_size, max_tokens, max_slots,
                                               self.max_length)
-        uses_library = library_gemm and self.dtype == torch.bfloat16
         self.memory_plan = MemoryPlan(
             weights=model.arena.planned if model.arena is not None else model.weight_bytes(),
             kv_pages=kv, block_tables=tables, state=state, workspace=Workspace.plan_bytes(workspace_plan),
@@ -90,6 +120,8 @@ class Runner:
         self.ctx = StepContext(self.kernels, self.cache, self.workspace, self.dtype, self.max_length,
                                split_keys, split_max_tokens)
         self.ctx.target_workgroups = target_workgroups
+        # split attention keeps its partial results within what was planned for them
+        self.ctx.partial_budget = workspace_plan.get(("attn_partial", torch.float32))
         self.ctx.status = self._status if self.check_finite else None
         # one vector a step: token ids, positions, slots (a value a token), wanted rows, and -- for a model that
         # keeps state per request -- one slot per entry
@@ -148,7 +180,9 @@ class Runner:
         step = 1 if n <= 8 else 2 if n <= 16 else 4 if n <= 64 else 8
         fill = -(-n // step) * step - n
         total = sum(len(e.tokens) for e in entries) + fill
-        if n + fill > self.graph_max_batch or total > min(self.graph_max_tokens, self.max_batch_tokens):
+        wanted = sum(len(e.want) for e in entries) + fill       # (the scratch rows' logits are computed and dropped)
+        if (n + fill > self.graph_max_batch or total > min(self.graph_max_tokens, self.max_batch_tokens)
+                or wanted > self.max_logits_rows):
             return 0, False
         return fill, mixed
 
@@ -305,7 +339,12 @@ class Runner:
         try:
             for context in contexts:
                 bucket = self._context_bucket(context)
-                start = max(1, min(bucket // 2 + 1, bucket - 4)) if bucket > 512 else 1
+                # the first context of the bucket: one beyond the bucket below it (the largest of 512, 1024, ...
+                # under this one, which a capped top bucket is not twice of); three steps must stay inside
+                below = 512
+                while below * 2 < bucket:
+                    below *= 2
+                start = max(1, min(below + 1, bucket - 4)) if bucket > 512 else 1
                 for n in sorted(set(int(b) for b in batch_sizes if 1 <= b <= limit), reverse=True):
                     key = (((1, (0,)),) * n, bucket)
                     if key in self._graphs and self._graphs[key]["graph"] is not None:

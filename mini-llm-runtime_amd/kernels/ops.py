@@ -403,7 +403,8 @@ class Kernels:
                _c_int(page_size), _c_int(1 if write_cache else 0), _c_int(rot_dim), _c_int(1 if interleaved else 0),
                _stream()), "qk_norm_rope_kv")
 
-    def attention_partial_numel(self, rows, q_heads, head_dim, max_splits):
+    @staticmethod
+    def attention_partial_numel(rows, q_heads, head_dim, max_splits):
         """Floats of scratch memory for the partial results of split attention: per (row, head, split) the
         unnormalised output, its maximum and its sum (the prompt-portion kernel keeps them 16 bytes apart)."""
         return rows * q_heads * max_splits * (head_dim + 4)
@@ -451,10 +452,11 @@ class Kernels:
     @timed("attention")
     def attention_mfma(self, q, k_pages, v_pages, block_table, slots, positions, out, group_row0, group_ntok,
                        groups, q_heads, kv_heads, head_dim, page_size, scale, window=None, split_keys=0,
-                       max_splits=1, partial=None):
+                       max_splits=1, partial=None, partial_rows=None):
         """As `paged_attention`, on the matrix cores.  The batch rows are covered by `groups` groups of
         consecutive rows of one request each (group_row0[i], group_ntok[i]), at most 16 // (q_heads //
-        kv_heads) tokens a group."""
+        kv_heads) tokens a group.  `partial_rows`: the caller vouches that every group's rows lie below this
+        batch row (the partial results are indexed by batch row and need not reach further); default: all rows."""
         _need(self.mfma_attention_supported(q_heads, kv_heads, head_dim, page_size),
               "attention_mfma: sizes not supported (bfloat16, page_size % 16 == 0, head_dim % 16 == 0, "
               "at most 16 query heads per kv head)")
@@ -474,7 +476,8 @@ class Kernels:
                   lambda: f"split_keys must be a multiple of {ATTENTION_TILE_KEYS}")
             _need(partial is not None, "partial buffer needed for split attention")
             _tensor(partial, "partial", torch.float32, ndim=1)
-            _need(partial.numel() >= self.attention_partial_numel(m, q_heads, head_dim, max_splits),
+            reach = m if partial_rows is None else partial_rows
+            _need(0 < reach <= m and partial.numel() >= self.attention_partial_numel(reach, q_heads, head_dim, max_splits),
                   "partial buffer too small")
         _need((split_keys // page_size + 2 if max_splits > 1 else block_table.shape[1]) <= MFMA_MAX_PAGES,
               "attention_mfma: a workgroup's key range spans more than 4096 pages; split the keys")
@@ -587,6 +590,12 @@ class Kernels:
                 and page_size & (page_size - 1) == 0
                 and (split_keys > 0 or max_context <= PREFILL_MAX_PAGES * page_size)
                 and stride < 2 ** 24 and num_pages < 2 ** 24 and stride * num_pages < 2 ** 32)
+
+    @staticmethod
+    def tiles_sizes_supported(q_heads, kv_heads, head_dim, page_size):
+        """The part of `tiles_attention_supported` that the model's sizes and the page size decide (bfloat16 engine)."""
+        return (page_size % 16 == 0 and page_size & (page_size - 1) == 0 and head_dim % 16 == 0
+                and head_dim <= TILES_MAX_HEAD_DIM and q_heads % kv_heads == 0 and q_heads // kv_heads <= 16)
 
     @staticmethod
     def tiles_longest_context(page_size):

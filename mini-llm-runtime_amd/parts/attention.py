@@ -68,38 +68,48 @@ class GqaAttention:
         s = self.spec
         if not kernels.mfma_attention_supported(s.q_heads, s.kv_heads, s.head_dim, page_size):
             return                        # the scalar kernel walks the block table itself: no limit
-        longest = kernels.mfma_longest_context(page_size)
-        if max_length <= longest:
-            return
-        if split_keys <= 0:
-            raise PartError(f"max_length {max_length} with pages of {page_size} tokens needs key splits "
-                            f"(split_keys > 0): one workgroup walks at most {longest} keys")
-        if split_keys > longest:
-            raise PartError(f"split_keys {split_keys} exceeds the {longest} keys one workgroup can walk "
-                            f"with pages of {page_size} tokens")
-        keys = split_keys
-        while keys * 2 <= longest:
-            keys *= 2
-        if max_length > keys * kernels.max_key_splits():
-            raise PartError(f"max_length {max_length} needs more than {kernels.max_key_splits()} key splits "
-                            f"of {keys} keys")
+        # the kernel for single tokens and short portions, and the one for prompt portions where it takes the
+        # sizes: each keeps the page ids of a workgroup's key range in LDS
+        reaches = [("single tokens", kernels.mfma_longest_context(page_size))]
+        if kernels.dtype == torch.bfloat16 and kernels.tiles_sizes_supported(s.q_heads, s.kv_heads, s.head_dim, page_size):
+            reaches.append(("prompt portions", kernels.tiles_longest_context(page_size)))
+        for what, longest in reaches:
+            if split_keys > longest:
+                # (a portion's key ranges are never narrower than split_keys: refused also where max_length
+                # would fit, since a short portion of a long context may be split to fill the GPU)
+                raise PartError(f"split_keys {split_keys} exceeds the {longest} keys one workgroup can walk "
+                                f"for {what} with pages of {page_size} tokens")
+            if max_length <= longest:
+                continue
+            if split_keys <= 0:
+                if what == "prompt portions":
+                    continue              # (without splits such contexts go to the kernel for single tokens)
+                raise PartError(f"max_length {max_length} with pages of {page_size} tokens needs key splits "
+                                f"(split_keys > 0): one workgroup walks at most {longest} keys")
+            keys = split_keys
+            while keys * 2 <= longest:
+                keys *= 2
+            if max_length > keys * kernels.max_key_splits():
+                raise PartError(f"max_length {max_length} needs more than {kernels.max_key_splits()} key splits "
+                                f"of {keys} keys")
 
     def workspace_plan(self, rows, dtype, limits):
         """{(buffer name, dtype): elements} that `forward` asks the workspace for in a step of `rows` tokens
-        at most.  The partial results of split attention are bounded by how splits are chosen: a split is
-        made only while (workgroups without it) x (splits) stays below twice `target_workgroups`, each
-        workgroup serving at most 128 (token, head) columns; a context beyond one workgroup's reach is
-        split for every row."""
+        at most.  The partial results of split attention (indexed by batch row) are bounded twice: where a
+        split only serves to fill the GPU it is made while (workgroups without it) x (splits) stays below
+        twice `target_workgroups`, each workgroup serving at most 128 (token, head) columns; a context beyond
+        one workgroup's reach is split for every row, into as few ranges as that reach allows.  `StepContext`
+        keeps every choice of splits within this number (`partial_budget`)."""
+        from ..engine.context import StepContext
+        from ..kernels.ops import Kernels
         s = self.spec
         width = s.q_heads * s.head_dim
-        forced = 1
-        longest = (4096 - 2) * limits["page_size"]
-        if limits["max_length"] > longest and limits["split_keys"] > 0:
-            keys = limits["split_keys"]
-            while keys * 2 <= longest:
-                keys *= 2
-            forced = -(-limits["max_length"] // keys)
-        partial = max(2 * limits["target_workgroups"] * 128, rows * s.q_heads * forced) * (s.head_dim + 4)
+        page, base, longest_context = limits["page_size"], limits["split_keys"], limits["max_length"]
+        forced = StepContext.forced_splits(longest_context, base, Kernels.mfma_longest_context(page))
+        if dtype == torch.bfloat16 and Kernels.tiles_sizes_supported(s.q_heads, s.kv_heads, s.head_dim, page):
+            forced = max(forced, StepContext.forced_splits(longest_context, base, Kernels.tiles_longest_context(page)))
+        per_split = Kernels.attention_partial_numel(1, s.q_heads, s.head_dim, 1)
+        partial = max(2 * limits["target_workgroups"] * 128 * (s.head_dim + 4), rows * forced * per_split)
         tq = max(1, 16 // (s.q_heads // s.kv_heads))
         plan = {("qkv", dtype): rows * (width + 2 * s.kv_heads * s.head_dim), ("q", dtype): rows * width,
                 ("attn", dtype): rows * width, ("mixer_out", dtype): rows * s.hidden,
@@ -221,7 +231,7 @@ class GqaAttention:
             columns = 128 if m * s.q_heads >= 128 * ctx.compute_units else 64
             big_factor = (columns // 16 if tiles
                           else 4 if k.prefill_attention_supported(*sizes, ctx.max_context) else 0)
-            small, big, small_rows = ctx.token_groups(tq, big_factor)
+            small, big, (small_rows, small_end) = ctx.token_groups(tq, big_factor)
             if big[2] and tiles:
                 split_keys, max_splits, partial = ctx.group_split(
                     big[2], m, s.kv_heads, s.q_heads, s.head_dim, longest=k.tiles_longest_context(view.page_size))
@@ -236,17 +246,24 @@ class GqaAttention:
                                     big[0], big[1], big[2], s.q_heads, s.kv_heads, s.head_dim, view.page_size,
                                     float(s.scale), window=s.window, max_context=ctx.max_context)
             if small[2]:
+                # (partial results are indexed by batch row: they reach as far as the last row of a small group,
+                # which in the scheduler's batches -- single tokens first -- is the number of single tokens)
                 split_keys, max_splits, partial = ctx.attention_split(
-                    small_rows, m, s.kv_heads, s.q_heads, s.head_dim, longest=k.mfma_longest_context(view.page_size))
+                    small_rows, small_end, s.kv_heads, s.q_heads, s.head_dim, longest=k.mfma_longest_context(view.page_size))
                 self._hint(k)
                 k.attention_mfma(q, view.k_pages, view.v_pages, view.block_table, ctx.slots, ctx.positions, attn,
                                  small[0], small[1], small[2], s.q_heads, s.kv_heads, s.head_dim, view.page_size,
                                  float(s.scale), window=s.window, split_keys=split_keys, max_splits=max_splits,
-                                 partial=partial)
+                                 partial=partial, partial_rows=small_end)
         else:
-            split_keys, max_splits, partial = ctx.attention_split(m, m, s.kv_heads, s.q_heads, s.head_dim)
+            # the float engine (and sizes that the matrix-core kernels do not take): key ranges of a fixed width,
+            # so that a token's result is the same to the bit however the step was cut or batched
+            split_keys, max_splits, chunk, partial = ctx.fixed_split(m, s.q_heads, s.head_dim)
             self._hint(k)
-            k.paged_attention(q, view.k_pages, view.v_pages, view.block_table, ctx.slots, ctx.positions, attn,
-                              s.q_heads, s.kv_heads, s.head_dim, view.page_size, float(s.scale),
-                              window=s.window, split_keys=split_keys, max_splits=max_splits, partial=partial)
+            for r0 in range(0, m, chunk):
+                r1 = min(m, r0 + chunk)
+                k.paged_attention(q[r0:r1], view.k_pages, view.v_pages, view.block_table, ctx.slots[r0:r1],
+                                  ctx.positions[r0:r1], attn[r0:r1], s.q_heads, s.kv_heads, s.head_dim, view.page_size,
+                                  float(s.scale), window=s.window, split_keys=split_keys, max_splits=max_splits,
+                                  partial=partial)
         return attn

@@ -1,5 +1,5 @@
-"""A decoder model put together from a `ModelSpec`: embedding, the layers (blocks of parts) in
-the order the schedule gives, a final norm on the wanted rows and the output projection.
+"""A decoder model put together from a `ModelSpec`: an embedding part, the layers (blocks of parts) in
+the order the schedule gives, a final norm on the wanted rows and an output head part.
 
 Which class builds which part is decided by the specs' `kind`s through the parts registry;
 which tensor of the file feeds which part is decided by the architecture's configuration
@@ -21,14 +21,15 @@ def build_blocks(spec):
 
 
 def _tensor_plan(config, spec, blocks):
-    """[(global name, WeightSpec, owner, local name)] for every tensor of the model; owner is
-    "embed", "lm_head", ("final_norm",) or (layer index, part name)."""
-    plan = [(config.global_tensor_name("embed"), WeightSpec((spec.vocab_size, spec.hidden)), "embed", None)]
+    """([(global name, WeightSpec, owner, local name)] for every tensor of the model, the embedding part, the
+    final norm, the head part); owner is ("embed",), ("final_norm",), ("head",) or (layer index, part name)."""
+    embed = build_part("embed", spec.embed_spec())
     final = build_part("norm", spec.final_norm)
-    for local, ws in final.weight_specs().items():
-        plan.append((config.global_tensor_name(f"final_norm.{local}"), ws, ("final_norm",), local))
-    plan.append((config.global_tensor_name("lm_head"),
-                 WeightSpec((spec.vocab_size, spec.hidden), optional=spec.tie_embeddings), "lm_head", None))
+    head = build_part("head", spec.head_spec())
+    plan = []
+    for owner, part in (("embed", embed), ("final_norm", final), ("head", head)):
+        for local, ws in part.weight_specs().items():
+            plan.append((config.global_tensor_name(f"{owner}.{local}"), ws, (owner,), local))
     for i, block in enumerate(blocks):
         for part_name, part in block.parts().items():
             for local, ws in part.weight_specs().items():
@@ -38,13 +39,13 @@ def _tensor_plan(config, spec, blocks):
     names = [p[0] for p in plan]
     if len(set(names)) != len(names):
         raise PartError("two parts claim the same tensor name")
-    return plan, final
+    return plan, embed, final, head
 
 
 def expected_tensors(config):
     """{tensor name: WeightSpec} of the architecture described by `config`."""
     spec = config.model_spec()
-    plan, _ = _tensor_plan(config, spec, build_blocks(spec))
+    plan = _tensor_plan(config, spec, build_blocks(spec))[0]
     return {name: ws for name, ws, _, _ in plan}
 
 
@@ -61,20 +62,14 @@ class DecoderModel:
             if not 0 <= run.layer < len(spec.layers):
                 raise PartError(f"the schedule names layer {run.layer} of {len(spec.layers)}")
         self.blocks = build_blocks(spec)
-        plan, self.final_norm = _tensor_plan(config, spec, self.blocks)
+        plan, self.embed, self.final_norm, self.head = _tensor_plan(config, spec, self.blocks)
         by_owner = {}
         for name, ws, owner, local in plan:
-            if name not in weights:
-                continue
-            if owner == "embed":
-                self.embed = weights[name]
-            elif owner == "lm_head":
-                self.lm_head = weights[name]
-            else:
+            if name in weights:
                 by_owner.setdefault(owner, {})[local] = weights[name]
-        if not hasattr(self, "lm_head"):
-            self.lm_head = self.embed          # tied: the same memory, no copy
+        self.embed.bind(by_owner.get(("embed",), {}))
         self.final_norm.bind(by_owner[("final_norm",)])
+        self.head.bind(by_owner.get(("head",), {}), embed=self.embed)      # (tied: the embedding's memory, no copy)
         for i, block in enumerate(self.blocks):
             for part_name, part in block.parts().items():
                 part.bind(by_owner.get((i, part_name), {}))
@@ -105,41 +100,50 @@ class DecoderModel:
         model.arena = arena[0]
         return model
 
+    def _ends(self):
+        return [self.embed, self.final_norm, self.head]
+
     def libraries(self):
-        names = {"elementwise", "gemm"}
+        """The kernel libraries that the parts of this model launch (each part names its own)."""
+        names = set()
         if self.dtype == torch.bfloat16:
             names.add("library_gemm")            # projections of many rows go to the vendor library
-        for block in self.blocks:
-            for part in block.parts().values():
-                if hasattr(part, "libraries"):
-                    names.update(part.libraries())
+        for part in self._ends() + [p for block in self.blocks for p in block.parts().values()]:
+            if hasattr(part, "libraries"):
+                names.update(part.libraries())
         return sorted(names)
 
     def workspace_plan(self, rows, logits_rows, limits):
         """{(buffer name, dtype): elements} of every scratch buffer that a step of at most `rows` tokens with
-        at most `logits_rows` wanted places asks for: this model's own and those of the parts that state
-        theirs (`workspace_plan(rows, dtype, limits)`; a part without one gets its buffers on demand)."""
-        plan = {("hidden", torch.float32): rows * self.spec.hidden, ("final", self.dtype): logits_rows * self.spec.hidden,
-                ("logits", torch.float32): logits_rows * self.spec.vocab_size}
+        at most `logits_rows` wanted places asks for: the final norm's rows here, the rest from the parts that
+        state theirs (the ends: `workspace_plan(rows, logits_rows, dtype, limits)`; blocks and their parts:
+        `workspace_plan(rows, dtype, limits)`; a part without one gets its buffers on demand)."""
+        plan = {("final", self.dtype): logits_rows * self.spec.hidden}
+
+        def add(part_plan):
+            for key, count in part_plan.items():
+                plan[key] = max(plan.get(key, 0), count)
+        for part in (self.embed, self.head):
+            if hasattr(part, "workspace_plan"):
+                add(part.workspace_plan(rows, logits_rows, self.dtype, limits))
         for block in self.blocks:
             for part in [block, *block.parts().values()]:
                 if hasattr(part, "workspace_plan"):
-                    for key, count in part.workspace_plan(rows, self.dtype, limits).items():
-                        plan[key] = max(plan.get(key, 0), count)
+                    add(part.workspace_plan(rows, self.dtype, limits))
         return plan
 
     def graph_safe(self):
         """True when every part of every layer may be captured in a graph."""
         return all(getattr(part, "graph_safe", False) for block in self.blocks
-                   for part in [block, *block.parts().values()]) and getattr(self.final_norm, "graph_safe", False)
+                   for part in [block, *block.parts().values()]) and all(getattr(part, "graph_safe", False)
+                                                                         for part in self._ends())
 
     def weight_bytes(self):
         """Bytes of the tensors the model uses (each once; without the padding between them)."""
         seen, total = set(), 0
-        tensors = [self.embed, self.lm_head, self.final_norm.weight]
-        for block in self.blocks:
-            for part in block.parts().values():
-                tensors += [v for v in vars(part).values() if isinstance(v, torch.Tensor)]
+        tensors = []
+        for part in self._ends() + [p for block in self.blocks for p in block.parts().values()]:
+            tensors += [v for v in vars(part).values() if isinstance(v, torch.Tensor)]
         for t in tensors:
             if t.data_ptr() not in seen:
                 seen.add(t.data_ptr())
@@ -150,12 +154,10 @@ class DecoderModel:
         """Run the step's tokens through every scheduled layer; logits float [R, V] at the rows
         `want_rows` (device int32, indices into the step's tokens), or None when R = 0."""
         k = ctx.kernels
-        m = ctx.n_tokens
-        h = ctx.workspace.get("hidden", (m, self.spec.hidden), torch.float32)
         status = getattr(ctx, "status", None)            # the debug mode that looks at the hidden state
         if status is not None:
             k.status_reset(status)
-        k.embed_gather(ctx.token_ids, self.embed, h)
+        h = self.embed.forward(ctx)
         pending = None
         schedule = self.spec.schedule
         for i, run in enumerate(schedule):
@@ -173,6 +175,4 @@ class DecoderModel:
             return None
         final = ctx.workspace.get("final", (r, self.spec.hidden), self.dtype)
         self.final_norm.forward(ctx, h, pending, final, rows=want_rows, write_h=False)
-        logits = ctx.workspace.get("logits", (r, self.spec.vocab_size), torch.float32)
-        k.gemm(final, self.lm_head, logits)
-        return logits
+        return self.head.forward(ctx, final)

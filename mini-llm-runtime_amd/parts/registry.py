@@ -19,6 +19,12 @@ Interfaces (B = the tokens of a step, E = the model width, T = the engine's elem
                   (the previous block's last output) into h itself, fused with its first norm.
                   `pending` may also be a `Handoff` (h is complete and the first half of a norm is
                   done); a block may return one for `next_norm`, the norm the next block starts with.
+  embed           weight_specs(), bind(), libraries();  forward(ctx) -> the float residual stream [B, E] of
+                  the step's tokens (ctx.token_ids);  optional table() -> the [vocab, E] matrix that a tied head
+                  may share;  workspace_plan(rows, logits_rows, dtype, limits).
+  head            weight_specs(), bind(weights, embed=the embedding part), libraries();
+                  forward(ctx, final) -> float logits [R, V] of the normed rows final [R, E];
+                  workspace_plan(rows, logits_rows, dtype, limits).
   Optional, for steps of few rows (each falls back to forward when a part lacks it):
   norm            handoff-capable norms set `fusable_rmsnorm = True` and offer
                   prenorm(ctx, h, delta) -> Handoff.
@@ -54,7 +60,7 @@ from __future__ import annotations
 
 from dataclasses import dataclass
 
-_REGISTRIES = {"norm": {}, "position": {}, "mixer": {}, "ffn": {}, "block": {}}
+_REGISTRIES = {"norm": {}, "position": {}, "mixer": {}, "ffn": {}, "block": {}, "embed": {}, "head": {}}
 
 
 @dataclass

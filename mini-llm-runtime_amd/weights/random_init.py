@@ -21,18 +21,31 @@ def _generator(seed, name):
 
 
 def random_tensors(expected, seed, dtype=torch.bfloat16, matrix_std=0.02, norm_std=0.1):
-    """expected: {name: WeightSpec}.  Optional tensors are left out."""
-    out = {}
-    for name, spec in expected.items():
-        if spec.optional:
-            continue
+    """expected: {name: WeightSpec}.  Optional tensors are left out.  Every tensor has a generator of its own,
+    so they are drawn side by side in threads (the values do not depend on how many)."""
+    from concurrent.futures import ThreadPoolExecutor
+
+    def draw(item):
+        name, spec = item
         g = _generator(seed, name)
         if spec.keep_float32:
             t = 1.0 + norm_std * torch.randn(spec.shape, generator=g, dtype=torch.float32)
         else:
             t = matrix_std * torch.randn(spec.shape, generator=g, dtype=torch.float32)
-        out[name] = t.to(dtype)
-    return out
+        return name, t.to(dtype)
+    todo = [(name, spec) for name, spec in expected.items() if not spec.optional]
+    workers = max(1, min(16, os.cpu_count() or 1, len(todo)))
+    if workers == 1 or sum(_numel(spec.shape) for _, spec in todo) < (1 << 22):
+        return dict(draw(item) for item in todo)
+    with ThreadPoolExecutor(max_workers=workers) as pool:
+        return dict(pool.map(draw, todo))              # (in the order of `expected`)
+
+
+def _numel(shape):
+    count = 1
+    for extent in shape:
+        count *= int(extent)
+    return count
 
 
 def write_random_model(folder, config, seed, dtype=torch.bfloat16, matrix_std=0.02, norm_std=0.1):

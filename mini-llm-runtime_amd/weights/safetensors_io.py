@@ -105,17 +105,18 @@ def write_safetensors(path, tensors, metadata=None):
     for t in tensors.values():
         if t.dtype not in _NAMES:
             raise SafetensorsError(f"cannot write dtype {t.dtype}")
+    ordered = []
     for name in sorted(tensors, key=lambda n: (-tensors[n].element_size(), n)):
         t = tensors[name].detach().contiguous().cpu()
-        raw = t.view(torch.uint8).numpy().tobytes() if t.numel() else b""
-        header[name] = {"dtype": _NAMES[t.dtype], "shape": list(t.shape),
-                        "data_offsets": [offset, offset + len(raw)]}
-        blobs.append(raw)
-        offset += len(raw)
+        size = t.numel() * t.element_size()
+        header[name] = {"dtype": _NAMES[t.dtype], "shape": list(t.shape), "data_offsets": [offset, offset + size]}
+        ordered.append(t)
+        offset += size
     text = json.dumps(header, separators=(",", ":")).encode("utf-8")
     text += b" " * ((-len(text)) % 8)
     with open(path, "wb") as f:
         f.write(struct.pack("<Q", len(text)))
         f.write(text)
-        for blob in blobs:
-            f.write(blob)
+        for t in ordered:                                  # (straight from the tensor's memory: no second copy)
+            if t.numel():
+                f.write(memoryview(t.view(torch.uint8).reshape(-1).numpy()))

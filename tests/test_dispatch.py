@@ -73,3 +73,51 @@ def test_even_head_sizes_are_taken_and_odd_ones_refused():
     for d in (15, 258):
         with pytest.raises(PartError, match="head_dim"):
             attention_part(d)
+
+
+def test_the_planned_partial_results_hold_every_choice_of_splits():
+    """The 8B sizes with requests of up to 40960 tokens: whatever the step (single tokens, a 2048-token portion
+    behind 34816 tokens of context, one single token beside such a portion), the partial results of split
+    attention stay within what the part planned for them, and a forced split still covers the context."""
+    spec = AttentionSpec("gqa_attention", 4096, 32, 8, 128, 128 ** -0.5, NormSpec("rmsnorm", 128, 1e-6),
+                         PositionSpec("rope_split_half", 128, 1e6))
+    part = build_part("mixer", spec)
+    rows, page = 2048 + 64, 16
+    limits = dict(max_length=40960, page_size=page, split_keys=256, split_max_tokens=256, target_workgroups=512)
+    planned = part.workspace_plan(rows, torch.bfloat16, limits)[("attn_partial", torch.float32)]
+    tiles_longest, mfma_longest = Kernels.tiles_longest_context(page), Kernels.mfma_longest_context(page)
+    assert limits["max_length"] > tiles_longest          # prompt portions are split for every row at this length
+    seen = 0
+    for context in (300, 4096, 20000, tiles_longest, tiles_longest + 1, 34816 + 2048, 40960):
+        ctx = context_with_budget(context, planned)
+        for units_rows, batch_rows in ((1, 1), (8, 8), (64, 64), (1, rows), (8, rows), (200, rows)):
+            keys, splits, partial = ctx.attention_split(units_rows, batch_rows, 8, 32, 128, longest=mfma_longest)
+            assert partial is None or partial.numel() <= planned
+            assert splits == 1 or keys * splits >= context
+            seen = max(seen, 0 if partial is None else partial.numel())
+        for groups in (1, 16, 128):                        # groups of a prompt portion (16 tokens x 4 heads a kv head)
+            keys, splits, partial = ctx.group_split(groups, rows, 8, 32, 128, longest=tiles_longest)
+            assert partial is None or partial.numel() <= planned
+            if context > tiles_longest:
+                assert splits > 1 and keys <= tiles_longest and keys * splits >= context
+            seen = max(seen, 0 if partial is None else partial.numel())
+    assert seen == planned                                 # the plan is met by some step, not merely an upper bound
+    assert ctx.workspace.unplanned_bytes() <= 4 * planned  # (this workspace has no plan: one buffer, never beyond it)
+
+
+def context_with_budget(max_context, budget):
+    ctx = context(max_context)
+    ctx.partial_budget = budget
+    return ctx
+
+
+def test_a_smallest_key_range_beyond_the_portion_kernels_reach_is_refused_when_the_runner_is_built():
+    part, k = attention_part(), kernels_without_gpu()
+    longest = Kernels.tiles_longest_context(16)
+    part.check_limits(k, 40960, 16, longest - longest % 64)
+    with pytest.raises(PartError, match="prompt portions"):
+        part.check_limits(k, 40960, 16, 49152)             # fits the single-token kernel, not the portions'
+    with pytest.raises(PartError, match="prompt portions"):
+        part.check_limits(k, 4096, 16, 49152)              # refused whatever max_length: splits also fill the GPU
+    # pages that the portion kernel does not take (no power of two) leave only the other kernel's limit
+    part.check_limits(k, 40960, 48, 49152)

@@ -261,6 +261,26 @@ def test_warm_up_stops_at_the_number_of_graphs_the_runner_keeps(model_folders, d
     assert r.free_slots() == 4 and r.cache.free_pages() == r.cache.num_pages
 
 
+def test_warm_up_reaches_a_top_bucket_that_is_no_power_of_two(model_folders):
+    """A limit of 768 tokens: the buckets are 512 and 768 (the capped top one is not twice the one below), and
+    the warm-up captures the decoding step in both.  And a batch is never filled up beyond the rows of logits
+    that were planned: nine slots decode as nine rows, not as ten."""
+    import torch
+    from mini_llm_runtime_amd.engine import Entry, Runner
+    from mini_llm_runtime_amd.parts import DecoderModel
+    model = DecoderModel.load(model_folders["A"], torch.bfloat16, "cuda:0")
+    r = Runner(model, max_tokens=2048, max_slots=2, max_length=768, page_size=PAGE_SIZE["A"])
+    assert r.warm_up() == 4
+    one = (1, (0,))
+    assert all(r._graphs[((one,) * n, b)]["graph"] is not None for n in (1, 2) for b in (512, 768))
+    r = Runner(model, max_tokens=1024, max_slots=9, max_length=64, page_size=PAGE_SIZE["A"], max_logits_rows=9)
+    slots = [r.open_request() for _ in range(9)]
+    for _ in range(3):
+        assert r.step([Entry(s, [5], [0]) for s in slots]).shape[0] == 9
+    assert r.memory_report()["actual"]["workspace_beyond_plan"] == 0
+    assert r._graphs[((one,) * 9, 64)]["graph"] is not None and ((one,) * 10, 64) not in r._graphs
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_warm_up_captures_the_decoding_steps_ahead_of_the_requests(model_folders, plain_models, dtype):
     """`Engine.warm_up`: the decoding steps of every batch size (and of the context buckets that fit) are

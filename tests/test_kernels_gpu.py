@@ -76,11 +76,16 @@ def test_add_rmsnorm(dtype, width):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_rmsnorm_extremes(dtype):
-    """Amplitudes from 0 to 1e15 (tests/cuda_ops_tests.cu:274-301) stay finite."""
+@pytest.mark.parametrize("width,repeat", [(257, 1), (256, 1), (256, 10)])
+def test_rmsnorm_extremes(dtype, width, repeat):
+    """Amplitudes from 0 to the largest float and an eps from the smallest to the largest
+    (tests/cuda_ops_tests.cu:274-301): a row whose squares do not fit 32 bits is scaled by its largest element
+    first, as the reference's kernel does for every row (src/minillm/cuda/ops.cu:87-126).  The widths and row
+    counts reach each variant of the kernel (one workgroup a row, scalar or 16 bytes a thread; one wavefront a
+    row from 64 rows on), with and without a delta that is still to be added."""
     k = kernels(dtype)
-    width = 257
-    amps = [0.0, 1e-15, 1.0, 1e15]
+    top = float(np.finfo(np.float32).max)
+    amps = [0.0, 1e-30, 1e-15, 1.0, 1e15, 1e30, top] * repeat
     h = torch.zeros((len(amps), width))
     for r, a in enumerate(amps):
         h[r, 0::3] = -a
@@ -88,12 +93,22 @@ def test_rmsnorm_extremes(dtype):
         h[r, 2::3] = 0.5 * a
     h = h.cuda()
     w = torch.ones(width, device="cuda")
+    zero = torch.zeros((len(amps), width), dtype=dtype, device="cuda")
+    for eps in (float(np.finfo(np.float32).smallest_subnormal), 1e-6, top):
+        x = h.double()
+        want = x * torch.rsqrt((x * x).mean(-1, keepdim=True) + eps)
+        for delta, write_h in ((None, True), (zero, True), (zero, False)):
+            out = torch.full((len(amps), width), 7.0, dtype=dtype, device="cuda")
+            k.add_rmsnorm(h.clone(), delta, w, out, eps, write_h=write_h)
+            assert torch.isfinite(out.float()).all(), (eps, write_h)
+            torch.testing.assert_close(out.double(), want, **tol(dtype))
+    # an infinity or a NaN in a row gives a row of NaN, and only that row
+    bad = h.clone()
+    bad[3, 5], bad[4, 7] = float("inf"), float("nan")
     out = torch.empty((len(amps), width), dtype=dtype, device="cuda")
-    k.add_rmsnorm(h, None, w, out, 1e-6)
-    x = h.double()
-    want = x * torch.rsqrt((x * x).mean(-1, keepdim=True) + 1e-6)
-    assert torch.isfinite(out.float()).all()
-    torch.testing.assert_close(out.double(), want, **tol(dtype))
+    k.add_rmsnorm(bad, None, w, out, 1e-6)
+    assert torch.isnan(out[3].float()).all() and torch.isnan(out[4].float()).all()
+    assert torch.isfinite(out[[0, 1, 2, 5, 6]].float()).all()
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -990,6 +1005,89 @@ def test_decode_attention_that_norms_rotates_and_caches_itself(case):
         vv = torch.cat([values[s], v1[pg, :, :, at].cpu()[None]]).double()
         want = plain_attention(q1[s].double().cpu().view(hq, d), kk, vv, scale, window)
         torch.testing.assert_close(out2[s].double().cpu().view(hq, d), want, **tol(dtype))
+
+
+@pytest.mark.parametrize("d", [64, 128])
+def test_decoding_beyond_the_page_cache_of_a_workgroup(d):
+    """One new token behind 66 000 keys in pages of 16 (4125 pages: more than the 4096 ids that a workgroup of
+    the single-token kernels keeps), beside a short request: unsplit the calls are refused; with the key ranges
+    that the engine forces on such a context both kernels (queries prepared, and the one that norms, rotates and
+    caches inside itself) give the plain attention and the same cache.  Random keys would hide a range that is
+    skipped among thousands: a key near the start, the last key of the first range, the first of the last range
+    and the last cached key are made to stand out, each with a value of its own."""
+    from mini_llm_runtime_amd.kernels.ops import KernelError, Kernels
+    dtype = torch.bfloat16
+    k = kernels(dtype)
+    hq, hkv, page = 2, 1, 16
+    lengths = [66000, 40]
+    assert lengths[0] > Kernels.mfma_longest_context(page)
+    gen = torch.Generator().manual_seed(5)
+    n, max_len = len(lengths), max(lengths)
+    max_blocks = (max_len + page - 1) // page
+    n_pages = sum((L + page - 1) // page for L in lengths) + 3
+    perm = torch.randperm(n_pages, generator=gen).tolist()
+    table = torch.full((n, max_blocks), -1, dtype=torch.int32)
+    k_pages = torch.full((n_pages, hkv, page, d), float("nan"), dtype=dtype)
+    v_pages = torch.full((n_pages, hkv, d, page), float("nan"), dtype=dtype)
+    qkv = (torch.randn((n, (hq + 2 * hkv) * d), generator=gen) * 1.5).to(dtype)
+    split_keys = 32768
+    marked = [5, split_keys - 1, 2 * split_keys, lengths[0] - 2]
+    keys, values = [], []
+    for s, L in enumerate(lengths):
+        kk = torch.randn((L - 1, hkv, d), generator=gen).to(dtype)
+        vv = torch.randn((L - 1, hkv, d), generator=gen).to(dtype)
+        if s == 0:
+            for j, at in enumerate(marked):            # along the first head's query: a score far above the others'
+                kk[at, 0] = (qkv[0, :d].float() * (1.2 + 0.01 * j)).to(dtype)
+                vv[at, 0] = 0
+                vv[at, 0, j] = 8.0
+        keys.append(kk)
+        values.append(vv)
+        flat_k = torch.cat([kk, torch.full((1, hkv, d), float("nan"), dtype=dtype)])       # (the new token's place)
+        flat_v = torch.cat([vv, torch.full((1, hkv, d), float("nan"), dtype=dtype)])
+        for b in range((L + page - 1) // page):
+            pg = perm.pop()
+            table[s, b] = pg
+            cnt = min(page, L - b * page)
+            k_pages[pg, :, :cnt] = flat_k[b * page:b * page + cnt].transpose(0, 1)
+            v_pages[pg, :, :, :cnt] = flat_v[b * page:b * page + cnt].permute(1, 2, 0)
+    qkv = qkv.cuda()
+    scale = 1 / math.sqrt(d)
+    slots = torch.arange(n, dtype=torch.int32).cuda()
+    pos = torch.tensor([L - 1 for L in lengths], dtype=torch.int32).cuda()
+    first = torch.arange(n, dtype=torch.int32).cuda()
+    ones = torch.ones(n, dtype=torch.int32).cuda()
+    max_splits = (max_len + split_keys - 1) // split_keys
+    partial = torch.full((k.attention_partial_numel(n, hq, d, max_splits),), float("nan"), device="cuda")
+    # no norm and no rotation: what is cached is the raw key, so the plain result below needs no second path
+    k1, v1 = k_pages.clone().cuda(), v_pages.clone().cuda()
+    q1 = torch.empty((n, hq * d), dtype=dtype, device="cuda")
+    k.qk_norm_rope_kv(qkv, q1, k1, v1, table.cuda(), slots, pos, None, None, 0.0, None, hq, hkv, d, page)
+    out1 = torch.full((n, hq * d), float("nan"), dtype=dtype, device="cuda")
+    with pytest.raises(KernelError, match="4096 pages"):
+        k.attention_mfma(q1, k1, v1, table.cuda(), slots, pos, out1, first, ones, n, hq, hkv, d, page, scale)
+    k.attention_mfma(q1, k1, v1, table.cuda(), slots, pos, out1, first, ones, n, hq, hkv, d, page, scale,
+                     split_keys=split_keys, max_splits=max_splits, partial=partial)
+    k2, v2 = k_pages.clone().cuda(), v_pages.clone().cuda()
+    out2 = torch.full((n, hq * d), float("nan"), dtype=dtype, device="cuda")
+    with pytest.raises(KernelError, match="4096 pages"):
+        k.attention_decode_fused(qkv, k2, v2, table.cuda(), slots, pos, out2, first, ones, n, hq, hkv, d, page, scale,
+                                 None, None, 0.0, None, partial)
+    partial.fill_(float("nan"))
+    k.attention_decode_fused(qkv, k2, v2, table.cuda(), slots, pos, out2, first, ones, n, hq, hkv, d, page, scale,
+                             None, None, 0.0, None, partial, split_keys=split_keys, max_splits=max_splits)
+    same = lambda x, y: torch.equal(x.view(torch.int16), y.view(torch.int16))
+    assert same(k1, k2) and same(v1, v2)
+    own_k = qkv[:, hq * d:(hq + hkv) * d].cpu().view(n, 1, hkv, d)
+    own_v = qkv[:, (hq + hkv) * d:].cpu().view(n, 1, hkv, d)
+    for s, L in enumerate(lengths):
+        kk = torch.cat([keys[s], own_k[s]]).double()
+        vv = torch.cat([values[s], own_v[s]]).double()
+        want = plain_attention(qkv[s, :hq * d].double().cpu().view(hq, d), kk, vv, scale, None)
+        if s == 0:                                   # each marked key carries a visible share of the first head's result
+            assert all(float(want[0, j]) > 0.5 for j in range(len(marked))), want[0, :len(marked)]
+        for out in (out1, out2):
+            torch.testing.assert_close(out[s].double().cpu().view(hq, d), want, **tol(dtype))
 
 
 def test_bfloat16_widening_and_rounding():

@@ -214,3 +214,56 @@ def test_six_requests_decode_together(folders, name, dtype_name):
     steps[-1]["end"] = list(reqs)
     compare(run_steps(r, steps), want, dtype_name)
     r.cache.check()
+
+
+def test_a_request_of_70000_tokens_on_one_layer(tmp_path):
+    """`max_length` 70 000 with pages of 16: more pages than one workgroup of either attention kernel keeps ids
+    of, so the runner forces key ranges on prompt portions (from 32 736 keys on) and on single tokens (from
+    65 504 on).  One layer of two heads of 64 channels; the prompt in portions of 8192, the last tokens one by
+    one (captured and replayed in the bucket of 70 000), against the plain logits of the last positions, which
+    are computed from the plain parts for those rows alone."""
+    from helpers import run_steps
+    from plain import qwen3_plain as P
+    from mini_llm_runtime_amd.config import config_from_dict
+    from mini_llm_runtime_amd.engine import Runner
+    from mini_llm_runtime_amd.kernels import Kernels
+    from mini_llm_runtime_amd.parts import DecoderModel
+    from mini_llm_runtime_amd.weights import write_random_model
+    cfg = dict(architectures=["Qwen3ForCausalLM"], hidden_size=64, num_hidden_layers=1, num_attention_heads=2,
+               num_key_value_heads=1, head_dim=64, intermediate_size=96, vocab_size=301, max_position_embeddings=70000,
+               rms_norm_eps=1e-6, rope_theta=1000000.0, tie_word_embeddings=True)
+    total, tail = 69990, 6
+    assert total > Kernels.mfma_longest_context(16) > Kernels.tiles_longest_context(16)
+    folder = str(tmp_path)
+    write_random_model(folder, config_from_dict(cfg), seed=9, matrix_std=0.2, norm_std=0.1)
+    toks = make_requests(cfg["vocab_size"], [total], seed=12)["r0"]
+    plain = P.PlainQwen3(folder)
+    w, eps = plain.layers[0], cfg["rms_norm_eps"]
+    positions = np.arange(total)
+    h = P.embed(toks, plain.embed)
+    q, k, v = P.project_qkv(P.rms_norm(h, w["input_layernorm"], eps), w, cfg, positions)
+    wanted = [total - tail - 1] + list(range(total - tail, total))     # the prompt's last token, then every decoded one
+    rows = []
+    for t in wanted:
+        heads = []
+        for head in range(2):
+            s = (k[:t + 1, 0] @ q[t, head]) / np.sqrt(64)
+            a = np.exp(s - s.max())
+            heads.append((a / a.sum()) @ v[:t + 1, 0])
+        x = h[t] + np.concatenate(heads) @ w["o_proj"].T
+        x = x + P.swiglu_mlp(P.rms_norm(x, w["post_attention_layernorm"], eps)[None], w)[0]
+        rows.append(P.output_logits(x[None], plain.final_norm, plain.lm_head, eps)[0])
+    want = {("r0", t): row for t, row in zip(wanted, rows)}
+    cuts = list(range(0, total - tail, 8192)) + [total - tail]
+    steps = [dict(step=i, entries=[dict(id="r0", tokens=toks[lo:hi], want=[hi - lo - 1] if hi == total - tail else [])],
+                  end=[]) for i, (lo, hi) in enumerate(zip(cuts, cuts[1:]))]
+    steps += [dict(step=100 + p, entries=[dict(id="r0", tokens=[toks[p]], want=[0])], end=[]) for p in range(total - tail, total)]
+    steps[-1]["end"] = ["r0"]
+    model = DecoderModel.load(folder, torch.bfloat16)
+    r = Runner(model, max_tokens=70016, max_slots=1, max_length=70000, max_batch_tokens=8192, page_size=16)
+    compare(run_steps(r, steps), want, "bfloat16")
+    assert r.graph_failures == 0 and r._graphs[(((1, (0,)),), 70000)]["graph"] is not None
+    report = r.memory_report()
+    assert report["actual"]["workspace_beyond_plan"] == 0
+    r.cache.check()
+    assert r.cache.free_pages() == r.cache.num_pages

@@ -52,7 +52,7 @@ def test_stacked_projections_share_the_arena_without_a_copy(model_folders):
         for t in (block.mixer.qkv, block.mixer.o, block.ffn.gate_up, block.ffn.down, block.norm1.weight):
             assert lo <= t.data_ptr() < hi and t.is_contiguous()
         assert block.mixer.qkv.shape == (4 * 32 + 2 * 32, 80) and block.ffn.gate_up.shape == (2 * 208, 80)
-    assert lo <= model.embed.data_ptr() < hi and lo <= model.lm_head.data_ptr() < hi
+    assert lo <= model.embed.weight.data_ptr() < hi and lo <= model.head.weight.data_ptr() < hi
 
 
 def test_the_budget_gate_refuses_before_anything_is_allocated(model_folders):
@@ -77,6 +77,45 @@ def test_the_budget_gate_refuses_before_anything_is_allocated(model_folders):
         r.step([Entry(s, [1, 2, 3], [0, 1, 2])])
     assert r.length(s) == 0 and not r.poisoned
     assert r.step([Entry(s, [1, 2, 3], [0, 2])]).shape == (2, 256)
+
+
+def test_a_pool_sized_from_the_budget_is_the_largest_that_fits_the_plan(model_folders):
+    """`max_tokens=None`: the page pool takes what the budget leaves beside everything else that is planned
+    (the reference has the cache's capacity and the budget side by side in its configuration,
+    include/minillm/cuda/runtime.h:18-30, src/minillm/cuda/storage.cpp:168-181).  With a cap of the user's:
+    what is held is what was planned, the plan fits the cap and one page more in every layer would not; without
+    one and with few slots: the pool is what the slots can hold at all."""
+    from mini_llm_runtime_amd.cache import CacheManager
+    from mini_llm_runtime_amd.engine import Engine, EngineOptions, MemoryBudgetError, Runner
+    model = load(model_folders, "A", "float32")
+    cap = 24 << 20
+    r = Runner(model, max_tokens=None, max_slots=64, max_length=1024, max_batch_tokens=64, page_size=16,
+               device_budget_bytes=cap)
+    plan, actual = r.memory_plan, r.memory_report()["actual"]
+    assert r.max_tokens % 16 == 0 and 0 < r.max_tokens < 64 * 1024
+    assert plan.to_allocate() <= cap and actual["kv_pages"] == plan.kv_pages == r.cache.kv_bytes()
+    cache_bytes = plan.kv_pages + plan.block_tables + plan.state
+    more = sum(CacheManager.plan(model.cache_entry_specs, torch.float32, 16, r.max_tokens + 16, 64, 1024))
+    assert more > cache_bytes and plan.to_allocate() - cache_bytes + more > cap
+    small = Runner(model, max_tokens=None, max_slots=3, max_length=100, max_batch_tokens=64, page_size=16)
+    assert small.max_tokens == 3 * 112                       # three requests of 100 tokens, in whole pages
+    with pytest.raises(MemoryBudgetError, match="leaves"):
+        Runner(model, max_tokens=None, max_slots=4, max_length=1024, max_batch_tokens=64, page_size=16, device_budget_bytes=1 << 16)
+    # the cache's element type is the engine's own
+    with pytest.raises(ValueError, match="kv_dtype"):
+        Runner(model, max_tokens=256, max_slots=4, max_length=256, page_size=16, kv_dtype="bfloat16")
+    with pytest.raises(ValueError, match="kv_dtype"):
+        Runner(model, max_tokens=256, max_slots=4, max_length=256, page_size=16, kv_dtype="int8")
+    Runner(model, max_tokens=256, max_slots=4, max_length=256, page_size=16, kv_dtype="float32")
+    # through the engine's options: what is left alone comes from the model and the device
+    cap = 64 << 20
+    eng = Engine(model, EngineOptions(max_active=4, device_budget_bytes=cap))
+    o = eng.options
+    assert (o.max_model_len, o.prefill_chunk, o.batch_tokens) == (1024, 2048, 2052)
+    assert o.context_tokens == eng.runner.max_tokens == eng.total_pages * 16 == 4 * 1024
+    assert eng.runner.memory_plan.to_allocate() <= cap
+    out = eng.submit(list(range(1, 200)), max_tokens=4, ignore_eos=True)
+    assert len(eng.run_until_done()[out]) == 4 and eng.stats["batches"] == 4      # the whole prompt in one step
 
 
 # ------------------------------------------------------------------------------------- finite check

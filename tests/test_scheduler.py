@@ -35,12 +35,26 @@ def test_decodes_first_then_prompts_in_order():
 
 def test_options_validation():
     """src/config.cpp:8-36; tests/core_tests.cpp:148-158."""
-    EngineOptions().validate()
+    EngineOptions().resolved(4096).validate()
     for change in [dict(max_active=0), dict(batch_tokens=4), dict(context_tokens=65), dict(max_model_len=1),
-                   dict(prefill_chunk=0), dict(prefill_chunk=1000), dict(aging_ms=0), dict(policy="x"),
-                   dict(max_model_len=10000)]:
+                   dict(prefill_chunk=0), dict(prefill_chunk=1000, batch_tokens=256), dict(aging_ms=0), dict(policy="x"),
+                   dict(max_model_len=10000, context_tokens=8192), dict(kv_dtype="int8"), dict(device_budget_bytes=-1)]:
         with pytest.raises(ValueError):
-            EngineOptions(**change).validate()
+            EngineOptions(**change).resolved(40960).validate()
+    with pytest.raises(ValueError):
+        EngineOptions().validate()                               # not resolved: the model's positions are not known yet
+
+
+def test_options_left_alone_come_from_the_model_and_the_slots():
+    """What is None is filled in: requests as long as the model allows, a step that holds one portion of 2048
+    tokens beside a token of every slot; the pool stays None for the runner to size from the device's budget."""
+    o = EngineOptions().resolved(40960)
+    assert (o.max_model_len, o.prefill_chunk, o.batch_tokens, o.context_tokens) == (40960, 2048, 2048 + o.max_active, None)
+    assert EngineOptions(max_model_len=1 << 20).resolved(40960).max_model_len == 40960
+    o = EngineOptions(context_tokens=256, max_active=4).resolved(1024)            # a small pool bounds the step
+    assert (o.batch_tokens, o.prefill_chunk) == (256, 256)
+    o.validate()
+    assert EngineOptions(batch_tokens=16, prefill_chunk=8).resolved(64).batch_tokens == 16
 
 
 # ------------------------------------------------------------------------------- fake step function

@@ -116,6 +116,71 @@ def register_toys():
                 out[first:first + n] = ((sums / (seen[pos0:] + 1).float()[:, None]) @ self.up.t()).to(x.dtype)
             return out
 
+    @dataclass(frozen=True)
+    class ScaledEmbedSpec:
+        kind: str
+        vocab_size: int
+        hidden: int
+        multiplier: float
+
+    @register_part("embed", "toy_scaled_embedding")
+    class ScaledEmbedding:
+        """The residual stream starts as multiplier * table[token]: the framework's gather, then a factor."""
+        graph_safe = True
+
+        def __init__(self, spec):
+            self.spec = spec
+
+        def weight_specs(self):
+            return {"weight": WeightSpec((self.spec.vocab_size, self.spec.hidden))}
+
+        def bind(self, weights):
+            self.weight = weights["weight"]
+
+        def libraries(self):
+            return ["elementwise"]
+
+        def workspace_plan(self, rows, logits_rows, dtype, limits):
+            return {("hidden", torch.float32): rows * self.spec.hidden}
+
+        def forward(self, ctx):
+            h = ctx.workspace.get("hidden", (ctx.n_tokens, self.spec.hidden), torch.float32)
+            ctx.kernels.embed_gather(ctx.token_ids, self.weight, h)
+            return h.mul_(self.spec.multiplier)
+
+    @dataclass(frozen=True)
+    class CappedHeadSpec:
+        kind: str
+        vocab_size: int
+        hidden: int
+        cap: float
+
+    @register_part("head", "toy_capped_head")
+    class CappedHead:
+        """logits = cap * tanh((final . W^T + bias) / cap): a bias and a cap on a head of its own (never tied)."""
+        graph_safe = True
+
+        def __init__(self, spec):
+            self.spec = spec
+
+        def weight_specs(self):
+            return {"weight": WeightSpec((self.spec.vocab_size, self.spec.hidden)),
+                    "bias": WeightSpec((self.spec.vocab_size,), keep_float32=True)}
+
+        def bind(self, weights, embed=None):
+            self.weight, self.bias = weights["weight"], weights["bias"]
+
+        def libraries(self):
+            return ["gemm"]
+
+        def workspace_plan(self, rows, logits_rows, dtype, limits):
+            return {("logits", torch.float32): logits_rows * self.spec.vocab_size}
+
+        def forward(self, ctx, final):
+            logits = ctx.workspace.get("logits", (final.shape[0], self.spec.vocab_size), torch.float32)
+            ctx.kernels.gemm(final, self.weight, logits)
+            return logits.add_(self.bias).div_(self.spec.cap).tanh_().mul_(self.spec.cap)
+
     def attention(hidden, heads, kv_heads, head_dim, eps, position=None):
         return AttentionSpec("gqa_attention", hidden, heads, kv_heads, head_dim, 1 / math.sqrt(head_dim),
                              NormSpec("rmsnorm", head_dim, eps),
@@ -237,7 +302,8 @@ def register_toys():
 
         @staticmethod
         def global_tensor_name(local):
-            return {"embed": "tok.weight", "final_norm.weight": "out_norm.weight", "lm_head": "out.weight"}[local]
+            return {"embed.weight": "tok.weight", "final_norm.weight": "out_norm.weight", "head.weight": "out.weight",
+                    "head.bias": "out.bias"}[local]
 
         @staticmethod
         def layer_tensor_name(layer, part, local):
@@ -326,6 +392,19 @@ def register_toys():
                               LayerSpec("prenorm", norm, LatentMeanSpec("toy_latent_mean", self.hidden, 6, 4), norm, ffn),
                               LayerSpec("prenorm", norm, near, norm, ffn)),
                              (LayerRun(0, 0), LayerRun(1, 1), LayerRun(2, 2)), norm, False, 512)
+
+    @register_architecture("ToyEndsForTests")
+    class ToyEnds(ToyBase):
+        """Two attention layers between an embedding with a multiplier and a head with a bias and a cap."""
+
+        def model_spec(self):
+            norm = NormSpec("rmsnorm", self.hidden, 1e-5)
+            ffn = MlpSpec("swiglu", self.hidden, self.inter)
+            layer = LayerSpec("prenorm", norm, attention(self.hidden, 2, 1, 16, 1e-5), norm, ffn)
+            return ModelSpec("ToyEndsForTests", self.vocab, self.hidden, (layer, layer), (LayerRun(0, 0), LayerRun(1, 1)),
+                             norm, False, 512,
+                             embed=ScaledEmbedSpec("toy_scaled_embedding", self.vocab, self.hidden, 3.5),
+                             head=CappedHeadSpec("toy_capped_head", self.vocab, self.hidden, 2.0))
 
     return ToyState, ToyOrder, ToyRouted, ToyWindow
 
@@ -730,3 +809,45 @@ def test_a_mixer_that_keeps_something_of_its_own_per_token_in_pages_of_its_own_s
     r.close_request(slot)
     assert all(r.cache.free_pages(g) == r.cache.group_pages[g] for g in range(3))
 
+
+
+def plain_toy_ends(w, tokens):
+    pos = np.arange(len(tokens))
+    h = 3.5 * P.embed(tokens, w["tok.weight"])
+    for i in range(2):
+        lw = plain_layer_weights(w, i)
+        x = P.rms_norm(h, w[f"layer{i}.norm1.weight"], 1e-5)
+        h = h + P.attention_block(x, lw, dict(ATTN_CFG, num_key_value_heads=1), pos)
+        h = h + P.swiglu_mlp(P.rms_norm(h, w[f"layer{i}.norm2.weight"], 1e-5), lw)
+    plain = P.output_logits(h, w["out_norm.weight"], w["out.weight"], 1e-5)
+    return 2.0 * np.tanh((plain + w["out.bias"]) / 2.0)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_an_embedding_with_a_multiplier_and_a_head_with_a_bias_and_a_cap(tmp_path, dtype):
+    """The model's two ends are parts like the others: an embedding and a head defined here are registered,
+    named by the architecture's `ModelSpec`, given their tensors by name (the head's bias among them), asked
+    for their libraries and scratch buffers, and stepped: whole, in portions, single tokens as captured steps."""
+    from helpers import compare, last_one_by_one, make_requests, portions, run_steps, whole
+    from mini_llm_runtime_amd.engine import Runner
+    from mini_llm_runtime_amd.parts import DecoderModel, expected_tensors
+    from mini_llm_runtime_amd.config import load_config
+    folder = write_folder(tmp_path, "ToyEndsForTests", seed=6)
+    assert {"tok.weight", "out.weight", "out.bias"} <= set(expected_tensors(load_config(folder)))
+    model = DecoderModel.load(folder, dtype)
+    assert type(model.embed).__name__ == "ScaledEmbedding" and type(model.head).__name__ == "CappedHead"
+    assert model.head.weight.data_ptr() != model.embed.weight.data_ptr()
+    w = plain_weights(folder)
+    w["out.bias"] = w["out.bias"] - 1.0          # (random norm-like vectors are drawn around 1: spread the bias around 0)
+    model.head.bias.sub_(1.0)
+    reqs = make_requests(97, [40, 17, 33], seed=3)
+    want = {(rid, p): row for rid, toks in reqs.items() for p, row in enumerate(plain_toy_ends(w, toks))}
+    assert max(np.abs(row).max() for row in want.values()) > 1.2, "the cap must matter"
+    name = "float32" if dtype == torch.float32 else "bfloat16"
+    r = Runner(model, max_tokens=128, max_slots=4, page_size=8)
+    compare(run_steps(r, whole(reqs)), want, name)
+    compare(run_steps(r, portions(reqs)), want, name)
+    compare(run_steps(r, last_one_by_one(reqs)), want, name)
+    assert r.use_graphs and r.graph_failures == 0 and r._graphs[(((1, (0,)),), 512)]["graph"] is not None
+    report = r.memory_report()
+    assert report["actual"]["workspace_beyond_plan"] == 0
