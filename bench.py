@@ -12,7 +12,8 @@ many gigabytes).  Every runner is built with the product's own defaults.  One JS
     the HBM roofline (bytes it has to read: every weight once and the live requests' cache; 8 TB/s);
   * points: the same at batch 1 and 64, and at batch 8 behind contexts of 1024, 8192 and 32768 tokens;
     prefill: 2048 tokens in one step (the median of several; the fastest beside it), with its share of the
-    MFMA peak;
+    MFMA peak, and `generate_ms`: the same prompt through the scheduler with its options left alone, from
+    submission to the first generated token;
   * with the default size, a block "8b" and a block "32b": decode at batch 64, 8 and 1, the prefill and a mixed
     step (64 decoding requests beside a 2048-token prompt portion in ONE step) at those sizes, each with its
     share of its roofline; the 64 requests of a block are filled once and serve all of its measurements.
@@ -196,6 +197,27 @@ class Bench:
         del runner
         torch.cuda.empty_cache()
         return out
+
+    def generate_prompt(self, reps=6):
+        """A 2048-token prompt through the scheduler with its options left alone but for the slots (`Engine`, as
+        `LLM.generate` drives it): milliseconds from submission to the first generated token (the median), to be
+        held against the one-step prefill."""
+        from mini_llm_runtime_amd.engine import Engine, EngineOptions
+        torch, c = self.torch, self.cfg
+        engine = Engine(self.model, EngineOptions(max_active=4))
+        times = []
+        for _ in range(reps + 1):
+            ids = torch.randint(0, c.vocab_size, (PREFILL_TOKENS,), generator=self.g).tolist()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            engine.submit(ids, max_tokens=1, ignore_eos=True)
+            engine.run_until_done()
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t0)
+        steps = engine.stats["batches"] / (reps + 1)
+        del engine
+        torch.cuda.empty_cache()
+        return dict(ms=round(statistics.median(times[1:]) * 1e3, 3), steps=steps)
 
     def prompt(self, portion=PREFILL_TOKENS):
         """One prompt of --context tokens, run in portions of `portion` tokens (the last one wants its logits):
@@ -473,6 +495,8 @@ def main():
         line["profile"] = report
     if not args.no_points and args.only == "all":
         line["prefill"] = bench.prefill()
+        through = bench.generate_prompt()
+        line["prefill"].update(generate_ms=through["ms"], generate_steps=through["steps"])
         points = {}
         few = (max(8, args.steps // 2), max(2, args.warmup // 2))
         for batch in (1, 64):
