@@ -51,6 +51,26 @@ def test_greedy_generation_through_the_python_entry_point(model_folders, plain_m
         assert one == outs[0] == plain_models[name].greedy(prompts[0], 8)
 
 
+def test_options_left_alone_through_the_python_entry_point(model_folders, plain_models):
+    """`LLM(folder)` and nothing else: requests as long as the model's positions, 64 slots, a step that holds a
+    2048-token portion beside a token of every slot, and a page pool sized by the runner (here: what the slots
+    can hold at all, far below the device's budget).  Every prompt, a 300-token one among them, runs whole in the
+    first step; then the requests decode together."""
+    from mini_llm_runtime_amd.api import LLM
+    llm = LLM(model_folders["A"])
+    o = llm.engine.options
+    assert (o.max_model_len, o.max_active, o.prefill_chunk, o.batch_tokens) == (1024, 64, 2048, 2112)
+    assert o.context_tokens == 64 * 1024 == llm.runner.max_tokens and o.device_budget_bytes == 0
+    prompts = prompts_for("A") + [make_requests(TINY["A"]["vocab_size"], [300], seed=77)["r0"]]
+    outs = llm.generate(prompts, max_tokens=6, ignore_eos=True)
+    for prompt, out in zip(prompts, outs):
+        assert len(out) == 6
+        check_greedy(plain_models["A"], prompt, out, "bfloat16")
+    assert llm.engine.stats["batches"] == 6 and llm.engine.stats["mixed_batches"] == 0
+    assert llm.runner.cache.free_pages() == llm.runner.cache.num_pages
+    assert llm.runner.memory_report()["actual"]["workspace_beyond_plan"] == 0
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_prefill_first_through_the_engine(model_folders, plain_models, dtype):
     """Policy prefill_first on the GPU, requests arriving while others decode: decoding requests are left out
