@@ -248,3 +248,36 @@ def test_a_spec_names_what_a_page_holds_and_groups_have_page_sizes_of_their_own(
     m.check()
     odd = CacheManager([KvSpec(1, 16), PagedSpec((("x", (PAGE,)),), page_size=24)], torch.float32, "cpu", 16, 96, 2, 96)
     assert odd.reserve_unit() == 48
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_the_largest_pool_that_fits_a_budget(seed):
+    """`CacheManager.tokens_that_fit`: a multiple of every group's page size, within the budget by the manager's
+    own plan, one unit more would not be (unless the slots cannot hold more), and nothing when not one unit fits."""
+    import math
+    import torch
+    from mini_llm_runtime_amd.cache import CacheManager, KvSpec, PagedSpec, StateSpec, PAGE
+    rng = random.Random(seed)
+    specs = [KvSpec(rng.randint(1, 4), rng.choice([16, 32, 64]), None) for _ in range(rng.randint(1, 3))]
+    if rng.random() < 0.5:
+        specs.append(KvSpec(2, 16, rng.choice([8, 24])))                         # a windowed group of its own
+    if rng.random() < 0.5:
+        specs.append(PagedSpec((("latent", (PAGE, 6)),), page_size=rng.choice([4, 12]), dtype=torch.float32))
+    if rng.random() < 0.5:
+        specs.append(StateSpec((rng.randint(1, 40),), torch.float32))
+    rng.shuffle(specs)
+    page, slots, length = rng.choice([8, 16, 32]), rng.randint(1, 9), rng.randint(10, 500)
+    unit = 1
+    for s in specs:
+        size = getattr(s, "page_size", None) or (page if not isinstance(s, StateSpec) else 1)
+        unit = unit * size // math.gcd(unit, size)
+    total = lambda tokens: sum(CacheManager.plan(specs, torch.bfloat16, page, tokens, slots, length))
+    most = slots * -(-length // unit) * unit
+    for budget in (total(most) + 5, total(most) - 1, total(3 * unit), total(unit) + 1, total(unit) - 1, 0):
+        got = CacheManager.tokens_that_fit(specs, torch.bfloat16, page, slots, length, budget)
+        assert got % unit == 0 and 0 <= got <= most
+        if got:
+            assert total(got) <= budget
+            assert got == most or total(got + unit) > budget
+        else:
+            assert total(unit) > budget

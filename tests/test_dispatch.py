@@ -121,3 +121,24 @@ def test_a_smallest_key_range_beyond_the_portion_kernels_reach_is_refused_when_t
         part.check_limits(k, 4096, 16, 49152)              # refused whatever max_length: splits also fill the GPU
     # pages that the portion kernel does not take (no power of two) leave only the other kernel's limit
     part.check_limits(k, 40960, 48, 49152)
+
+
+def test_key_ranges_of_one_width_whatever_the_batch():
+    """The float engine's attention (`StepContext.fixed_split`): the width of a key range is the runner's setting
+    for every number of rows and every context (so a token's sums do not depend on the batch), the ranges cover
+    the context, and rows whose partial results would not fit what was planned are served by several launches."""
+    per = lambda splits: Kernels.attention_partial_numel(1, 16, 128, splits)
+    for max_context in (100, 256, 257, 4096, 40960):
+        for rows in (1, 7, 300, 2048):
+            ctx = context_with_budget(max_context, 2 * 512 * 128 * 132)
+            keys, splits, chunk, partial = ctx.fixed_split(rows, 16, 128)
+            if max_context <= 256:
+                assert (keys, splits, chunk, partial) == (0, 1, rows, None)
+                continue
+            assert keys == 256 and splits == -(-max_context // 256)
+            assert 1 <= chunk <= rows and partial.numel() == chunk * per(splits) <= ctx.partial_budget
+            assert chunk == rows or (chunk + 1) * per(splits) > ctx.partial_budget
+    # beyond 1024 ranges the width doubles (the merge kernel keeps one weight a range in LDS)
+    ctx = context_with_budget(300000, None)
+    keys, splits, chunk, _ = ctx.fixed_split(3, 16, 128)
+    assert keys == 512 and splits == -(-300000 // 512) <= MAX_KEY_SPLITS and chunk == 3

@@ -229,9 +229,13 @@ def test_command_line(model_folders, plain_models, tmp_path):
                        (["--model", model_folders["A"], "--prompt-ids", ids, "--cuda-precision", "f16-matrix-f32acc"],
                         "f32-pedantic"),
                        (["--model", model_folders["A"], "--prompt-ids", ids, "--device-budget-bytes", "1000"], "exceed"),
+                       (["--model", model_folders["A"], "--prompt-ids", ids, "--kv-dtype", "int8"], "--kv-dtype"),
+                       (["--model", model_folders["A"], "--prompt-ids", ids, "--kv-dtype", "float32"], "element type"),
                        (["--model", str(tmp_path), "--prompt-ids", "1"], "config.json")]:
         bad = run_cli(args)
         assert bad.returncode == 1 and text in bad.stderr, (args, bad.stderr)
+    ok = run_cli(["--model", model_folders["A"], "--prompt-ids", ids, "--tokens", "6", "--kv-dtype", "bfloat16", "--context", "64"])
+    assert ok.returncode == 0, ok.stderr                             # (the bfloat16 engine's own element type)
     assert run_cli(["--help"]).returncode == 0 and run_cli([]).returncode == 1
 
 
