@@ -71,10 +71,16 @@ class Profiler:
                 calls, ms, nbytes, flops = self._sums[kind]
                 seconds = ms / 1e3
                 out[kind] = {"calls": calls, "ms": round(ms, 4),
-                             "gb_s": round(nbytes / seconds / 1e9, 1) if seconds > 0 else None,
-                             "tflop_s": round(flops / seconds / 1e12, 2) if seconds > 0 else None}
+                             "gb_s": _significant(nbytes / seconds / 1e9) if seconds > 0 else None,
+                             "tflop_s": _significant(flops / seconds / 1e12) if seconds > 0 else None}
         out["total_ms"] = round(sum(v[1] for v in self._sums.values()), 4)
         return out
+
+
+def _significant(value, digits=4):
+    """`value` to `digits` significant digits: a small model's rates (a first product's time holds the
+    library's set-up) stay above zero where a fixed number of decimals would round them away."""
+    return float(f"{value:.{digits}g}")
 
 
 def timed(kind, work=None):
