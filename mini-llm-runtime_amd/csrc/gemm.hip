@@ -201,6 +201,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_bf16_kernel(
 struct SkinnyEpilogue {
     const float* ss;          // EPI_SCALE: [M][ss_parts] partial sums of squares of the rows
     int ss_parts;
+    int ss_vec;               // ss_parts is a multiple of 4 and ss 16-byte aligned: four sums a load
     float eps, inv_size;
     float* h;                 // EPI_RESIDUAL: [M][N] the residual stream
     const float* next_w;      // [N] weights of the norm that follows, or null
@@ -245,15 +246,41 @@ __global__ __launch_bounds__(SKINNY_WAVES * 64) void gemm_skinny_kernel(const __
     float4 h4b = h4, nw4b = h4;                            // ... and, PAIR, at the second strip's columns n0 + 16 + 4 b ..
     if constexpr (EPI == EPI_SCALE) {
         // the row's partial sums are dealt out to the 32 (wavefront, lane block) pairs in runs of q; a run is
-        // added in ascending order, the four runs of a wavefront as (0 + 1) + (2 + 3), the wavefronts in the
-        // order 0..7: an order that depends on nothing but the number of partial sums
-        const int q = (epi.ss_parts + 4 * SKINNY_WAVES - 1) / (4 * SKINNY_WAVES);
+        // added in ascending order (four sums that lie side by side as (0 + 1) + (2 + 3) first, when their number
+        // allows 16-byte loads), the four runs of a wavefront as (0 + 1) + (2 + 3), the wavefronts in the order
+        // 0..7: an order that depends on nothing but the number of partial sums.  Four loads are asked for before
+        // the first is used: a load a turn of the loop would cost a trip to the cache each, one after the other,
+        // before the workgroup has asked for any of its weight.
         const float* row = epi.ss + (size_t)min(r16, M - 1) * epi.ss_parts;
-        const int first = (wave * 4 + b) * q;
-        for (int j = 0; j < q; ++j) {
-            const int at = first + j;
-            const float v = row[min(at, epi.ss_parts - 1)];
-            ss_mine += at < epi.ss_parts ? v : 0.f;
+        const int pair = wave * 4 + b;
+        if (epi.ss_vec) {
+            const int quads = epi.ss_parts >> 2;
+            const int q = (quads + 4 * SKINNY_WAVES - 1) / (4 * SKINNY_WAVES);
+            const float4* row4 = reinterpret_cast<const float4*>(row);
+            for (int j0 = 0; j0 < q; j0 += 4) {
+                float4 v[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) v[j] = row4[min(pair * q + j0 + j, quads - 1)];
+                asm volatile("" : "+v"(v[0].x), "+v"(v[1].x), "+v"(v[2].x), "+v"(v[3].x));   // (all four are loaded, none behind a branch)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const bool mine = j0 + j < q && pair * q + j0 + j < quads;
+                    ss_mine += mine ? (v[j].x + v[j].y) + (v[j].z + v[j].w) : 0.f;
+                }
+            }
+        } else {
+            const int q = (epi.ss_parts + 4 * SKINNY_WAVES - 1) / (4 * SKINNY_WAVES);
+            for (int j0 = 0; j0 < q; j0 += 4) {
+                float v[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) v[j] = row[min(pair * q + j0 + j, epi.ss_parts - 1)];
+                asm volatile("" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]));
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const bool mine = j0 + j < q && pair * q + j0 + j < epi.ss_parts;
+                    ss_mine += mine ? v[j] : 0.f;
+                }
+            }
         }
     }
     if constexpr (EPI == EPI_RESIDUAL) {
@@ -945,6 +972,7 @@ extern "C" int mlr_gemm_prenormed(const void* x, const float* ss, int ss_parts, 
     SkinnyEpilogue epi{};
     epi.ss = ss;
     epi.ss_parts = ss_parts;
+    epi.ss_vec = (ss_parts % 4 == 0 && reinterpret_cast<uintptr_t>(ss) % 16 == 0) ? 1 : 0;
     epi.eps = eps;
     epi.inv_size = 1.0f / (float)norm_size;
     if (gated) return launch_skinny<1, true, EPI_SCALE>(x, w, out, M, N, K, 0, stream, epi);
