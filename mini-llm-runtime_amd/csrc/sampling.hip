@@ -52,10 +52,21 @@ __global__ __launch_bounds__(THREADS) void chunk_max_kernel(const float* __restr
     float best = -INFINITY;
     int best_i = 0x7fffffff;
     bool nonfinite = false;
-    for (int i = cb + t; i < ce; i += THREADS) {
-        const float x = row[i];
-        if (!(fabsf(x) <= 3.402823466e38f)) nonfinite = true;
-        if (x > best) { best = x; best_i = i; }
+    // (four loads are asked for before the first is used, each at an index inside the chunk: one load a turn
+    // would cost a trip to memory each, one after the other)
+    for (int i0 = cb + t; i0 < ce; i0 += 4 * THREADS) {
+        float x[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) x[j] = row[min(i0 + j * THREADS, ce - 1)];
+        asm volatile("" : "+v"(x[0]), "+v"(x[1]), "+v"(x[2]), "+v"(x[3]));      // (all four loaded here, none moved behind a branch)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int i = i0 + j * THREADS;
+            if (i < ce) {
+                if (!(fabsf(x[j]) <= 3.402823466e38f)) nonfinite = true;
+                if (x[j] > best) { best = x[j]; best_i = i; }
+            }
+        }
     }
     if (nonfinite) bad = 1;
     vals[t] = best;
@@ -118,7 +129,15 @@ __global__ __launch_bounds__(THREADS) void chunk_sum_kernel(const float* __restr
     const int begin = min(ce, cb + t * per), end = min(ce, begin + per);
     const float inv_t = 1.0f / temp, row_max = rmax[r];
     float sum = 0.f;
-    for (int i = begin; i < end; ++i) sum += expf((row[i] - row_max) * inv_t);
+    for (int i0 = begin; i0 < end; i0 += 4) {          // (four loads asked for at once; added in ascending order)
+        float x[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) x[j] = row[min(i0 + j, end - 1)];
+        asm volatile("" : "+v"(x[0]), "+v"(x[1]), "+v"(x[2]), "+v"(x[3]));
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            if (i0 + j < end) sum += expf((x[j] - row_max) * inv_t);
+    }
     vals[t] = sum;
     __syncthreads();
     if (t == 0) {                                   // ascending order
@@ -167,7 +186,15 @@ __global__ __launch_bounds__(THREADS) void pick_kernel(const float* __restrict__
     const int begin = min(ce, cb + t * per), end = min(ce, begin + per);
     const float inv_t = 1.0f / temp, row_max = rmax[r];
     float sum = 0.f;
-    for (int i = begin; i < end; ++i) sum += expf((row[i] - row_max) * inv_t);
+    for (int i0 = begin; i0 < end; i0 += 4) {          // (four loads asked for at once; added in ascending order)
+        float x[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) x[j] = row[min(i0 + j, end - 1)];
+        asm volatile("" : "+v"(x[0]), "+v"(x[1]), "+v"(x[2]), "+v"(x[3]));
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            if (i0 + j < end) sum += expf((x[j] - row_max) * inv_t);
+    }
     vals[t] = sum;
     __syncthreads();
     if (t == 0) {
