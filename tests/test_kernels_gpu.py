@@ -815,10 +815,13 @@ def test_rows_prenorm(rows, width):
 
 @pytest.mark.parametrize("gated", [False, True])
 @pytest.mark.parametrize("mnk,parts", [((1, 48, 64), 1), ((8, 4096, 1024), 64), ((16, 100, 1024), 3), ((5, 208, 96), 6),
-                                       ((3, 40, 4096), 256), ((7, 24, 32), 2), ((2, 50, 100), 7), ((16, 333, 2048), 128)])
+                                       ((3, 40, 4096), 256), ((7, 24, 32), 2), ((2, 50, 100), 7), ((16, 333, 2048), 128),
+                                       ((4, 48, 8320), 520), ((6, 32, 2096), 131), ((9, 64, 5120), 320)])
 def test_projection_after_a_handed_over_norm(mnk, parts, gated):
     """`gemm_prenormed`: the rows' scale rsqrt(sum of the partial sums / K + eps), applied to the finished sums
-    of x . w^T (or inside the gated activation), equals the projection of the normed rows."""
+    of x . w^T (or inside the gated activation), equals the projection of the normed rows.  The partial sums are
+    read four a load where their number is a multiple of four and they start at a multiple of 16 bytes, else
+    one a load, in rounds of four loads (520 and 131 parts: more than one round)."""
     m, n, kk = mnk
     k = kernels(torch.bfloat16)
     assert k.handoff_supported(m) and not k.handoff_supported(17) and not kernels(torch.float32).handoff_supported(m)
@@ -844,6 +847,13 @@ def test_projection_after_a_handed_over_norm(mnk, parts, gated):
         one = torch.full((1, n), float("nan"), dtype=torch.bfloat16, device="cuda")
         k.gemm_prenormed(x[m - 1:].contiguous(), ss[m - 1:].contiguous(), eps, w, one, gated=gated)
         assert torch.equal(one[0], out[m - 1])
+    # the same sums at an address that is no multiple of 16 bytes (read one a load)
+    shifted = torch.empty(m * parts + 1, dtype=torch.float32, device="cuda")[1:].view(m, parts)
+    shifted.copy_(ss)
+    assert shifted.data_ptr() % 16 == 4
+    again = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    k.gemm_prenormed(x, shifted, eps, w, again, gated=gated)
+    torch.testing.assert_close(again.double(), want, atol=1e-2 * float(want.abs().max()), rtol=1e-2)
 
 
 @pytest.mark.parametrize("mnk", [(1, 64, 48), (8, 1024, 2048), (16, 1024, 3072), (5, 96, 208), (3, 4096, 4096), (7, 50, 96),
