@@ -122,3 +122,20 @@ def test_the_benchmark_refuses_more_than_one_gpu():
     done = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
                           timeout=120)
     assert done.returncode == 2 and len(done.stdout.strip().splitlines()) == 1 and "--gpus 2" in done.stdout
+
+
+def test_the_package_exports_its_entry_points():
+    """What a user imports first is at the top level, and importing it touches no GPU."""
+    import mini_llm_runtime_amd as package
+    from mini_llm_runtime_amd.api import LLM, generate
+    assert package.LLM is LLM and package.generate is generate
+    for name in package.__all__:
+        assert hasattr(package, name), name
+
+
+def test_profiler_rates_keep_their_leading_digits():
+    """A small model's rates (a first product's time holds the library's set-up) must not round to zero."""
+    from mini_llm_runtime_amd.kernels.profile import _significant
+    assert _significant(0.00012345678) == 0.0001235
+    assert _significant(1234.5678) == 1235.0
+    assert _significant(0.0) == 0.0
