@@ -539,7 +539,8 @@ __global__ __launch_bounds__(SKINNY_WAVES * 64) void gemm_skinny_kernel(const __
 
 // Columns of a workgroup when two strips side by side deal the work out more evenly than strips of 16 do, else 0.
 // Only where the weight is long enough for the memory's rate to count (k from 2048).
-static int skinny_pair_columns(int N, int K) {
+// Compute units of the current device, asked for once; -1 when the device does not say.
+static int compute_units() {
     static int units = 0;
     if (units == 0) {
         int device = 0;
@@ -547,6 +548,11 @@ static int skinny_pair_columns(int N, int K) {
             hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || units <= 0)
             units = -1;
     }
+    return units;
+}
+
+static int skinny_pair_columns(int N, int K) {
+    const int units = compute_units();
     if (units < 0 || K < 2048 || N % 4 != 0) return 0;
     const int strips = (N + 15) / 16;
     const int turns = (strips + units - 1) / units;       // strips of 16: the busiest unit's share, in strips
@@ -602,10 +608,15 @@ static int launch_skinny(const void* a, const void* w, void* out, int M, int N, 
     if constexpr (MT == 1 && !GATED) {
         // Two rows or more and a long k: the activation goes through LDS.  (Measured: with a short k the
         // extra step costs what it saves, and the gated variant, whose turns would have to shrink to stay
-        // within the registers of two workgroups a compute unit, gains nothing.)
+        // within the registers of two workgroups a compute unit, gains nothing.  At k = 2048 it pays where the
+        // strips leave half of the compute units idle -- a workgroup's requests go through its unit's cache
+        // one after the other, and there the activation's are half of them: 4.9 us for 5.4 on 1024 columns and
+        // 8 rows, 5.2 for 6.1 with 16 -- and costs 3-6 % with a strip for every unit.)
         const size_t lds = (size_t)SKINNY_WAVES * M * SKINNY_STAGE_PITCH(4);
         const bool pair = skinny_pair_columns(N, K) > 0;     // (two strips: without the stage)
-        if (!pair && M >= 2 && K % 64 == 0 && K > 2048 && lds <= SKINNY_STAGE_LDS)
+        const int units = compute_units();
+        const bool long_k = K > 2048 || (K == 2048 && units > 0 && 2 * ((N + 15) / 16) <= units);
+        if (!pair && M >= 2 && K % 64 == 0 && long_k && lds <= SKINNY_STAGE_LDS)
             return launch_skinny_as<MT, GATED, 4, true, EPI>(a, w, out, M, N, K, out_float, lds, epi, stream);
     }
     if (short_k) return launch_skinny_as<MT, GATED, 2, false, EPI>(a, w, out, M, N, K, out_float, 0, epi, stream);
