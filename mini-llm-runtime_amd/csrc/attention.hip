@@ -39,7 +39,7 @@ struct AttnArgs {
 };
 
 __global__ __launch_bounds__(256) void paged_attention_kernel(AttnArgs a) {
-    extern __shared__ float lds[];
+    extern __shared__ __attribute__((aligned(16))) float lds[];
     const int D = a.head_dim;
     const int group = a.q_heads / a.kv_heads;
     const int head_chunks = (group + HEADS_PER_BLOCK - 1) / HEADS_PER_BLOCK;
@@ -322,7 +322,7 @@ struct DecodeFusion {
 template <int NCH, bool FUSED>   // NCH: ceil(head_dim / 32)
 __global__ __launch_bounds__(256, (NCH <= 4 ? 2 : 1)) void attention_mfma_kernel(AttnArgs a, const int32_t* __restrict__ group_row0,
                                                              const int32_t* __restrict__ group_ntok, DecodeFusion f) {
-    extern __shared__ float lds[];
+    extern __shared__ __attribute__((aligned(16))) float lds[];
     __shared__ int32_t page_lds[DECODE_PAGE_CACHE];    // the request's page ids for this workgroup's key range
     const int D = a.head_dim, P = a.page_size;
     const int g = a.q_heads / a.kv_heads;
@@ -575,14 +575,14 @@ __global__ __launch_bounds__(256, (NCH <= 4 ? 2 : 1)) void attention_mfma_kernel
     l_run += __shfl_xor(l_run, 32, MLR_WAVE);
 
     // merge the wavefronts: 1..3 park their state in LDS, 0 merges in ascending order
-    const int stride = 16 * D + 32;                        // floats per wavefront: out^T [D][16], max[16], sum[16]
+    const int stride = 16 * D + 32;                        // floats per wavefront: the sums [D / 4][16 columns][4], max[16], sum[16]
     if (wave > 0) {
         float* dst = lds + (size_t)(wave - 1) * stride;
 #pragma unroll
         for (int db = 0; db < 2 * NCH; ++db) {
             if (16 * db >= D) break;
-#pragma unroll
-            for (int r = 0; r < 4; ++r) dst[(16 * db + 4 * b + r) * 16 + col] = o[db][r];
+            // (a lane's four sums side by side: one 16-byte access, consecutive lanes consecutive addresses)
+            *reinterpret_cast<floatx4*>(dst + ((4 * db + b) * 16 + col) * 4) = o[db];
         }
         if (b == 0) {
             dst[16 * D + col] = m_run;
@@ -609,8 +609,9 @@ __global__ __launch_bounds__(256, (NCH <= 4 ? 2 : 1)) void attention_mfma_kernel
 #pragma unroll
             for (int db = 0; db < 2 * NCH; ++db) {
                 if (16 * db >= D) break;
+                const floatx4 other = *reinterpret_cast<const floatx4*>(src + ((4 * db + b) * 16 + col) * 4);
 #pragma unroll
-                for (int r = 0; r < 4; ++r) o[db][r] += src[(16 * db + 4 * b + r) * 16 + col] * f;
+                for (int r = 0; r < 4; ++r) o[db][r] += other[r] * f;
             }
         }
         if (col_valid) {
